@@ -1,0 +1,133 @@
+/*
+ * librzlinear — C ABI of the MI355X (gfx950) RzLinear hot path.
+ *
+ * RzLinear is a linear layer whose logical weight W[K,N] is never stored: tile
+ * (tk,tn) of W, BK x BN elements, is the contiguous slice
+ *     hashed_weight[off(tk,tn) : off(tk,tn) + BK*BN]     viewed row-major [BK,BN]
+ * of a 1-D parameter hashed_weight[H].  The three device entry points compute
+ *     forward      Y   = (X  . W  ) * init_factor
+ *     input-grad   dX  = (dY . W^T) * init_factor
+ *     weight-grad  dHW = scatter_add over tiles of (X^T . dY) * init_factor
+ * without materialising W.
+ *
+ * Conventions shared by every entry point
+ *   - plain pointers and sizes only; device pointers are HIP device memory that
+ *     the caller owns; no entry point allocates or frees device memory or
+ *     synchronises with the host; work is enqueued on `stream` (a hipStream_t
+ *     passed as void*, NULL = the default stream).
+ *   - matrices are row-major with unit column stride; `ld*` is the row pitch in
+ *     ELEMENTS.  Any M, K, N >= 1 is accepted (edge tiles read as zero).
+ *   - R[8] are the hash constants: R[0] = P (prime), R[1..7] in [0,P).  R[6] is
+ *     carried but takes part in no formula, exactly as in the reference.
+ *   - BK, BN: powers of two in [16, 256]; H > BK*BN.
+ *   - return value: RZ_OK (0) or a negative rz_status; never throws.
+ *
+ * Reference interface that each entry point replaces is cited as
+ * file:line of the reference checkout (python/rz_linear/...).
+ */
+#ifndef RZLINEAR_H
+#define RZLINEAR_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum rz_status {
+  RZ_OK = 0,
+  RZ_ERR_NULL_POINTER = -1,
+  RZ_ERR_BAD_SHAPE = -2,       /* M, K, N < 1, ld too small, sizes beyond int32 tiling */
+  RZ_ERR_BAD_TILE = -3,        /* BK/BN not a power of two in [16,256] */
+  RZ_ERR_HASH_RANGE = -4,      /* H <= BK*BN  (reference: assert H > BLOCK_SIZE_K*BLOCK_SIZE_N) */
+  RZ_ERR_BAD_DTYPE = -5,
+  RZ_ERR_HASH_OVERFLOW = -6,   /* hash intermediates would leave int32 (reference computes in int32) */
+  RZ_ERR_WORKSPACE = -7,       /* workspace missing or too small */
+  RZ_ERR_LAUNCH = -8,          /* HIP reported a launch error */
+  RZ_ERR_BAD_ARGUMENT = -9
+} rz_status;
+
+typedef enum rz_dtype {
+  RZ_F32 = 0,
+  RZ_BF16 = 1,
+  RZ_F16 = 2
+} rz_dtype;
+
+/* Library / ABI version (major*10000 + minor*100 + patch). */
+int rz_version(void);
+
+/* Human-readable text for a status code (static storage). */
+const char* rz_status_string(int status);
+
+/*
+ * Tile offsets on the HOST, bit-exact integer hash.
+ *   hash_levels = 2:  off = (((tk*R3 + tn*R2 + R1) % R0) * R0 + ((tk*R7 + tn*R5 + R4) % R0)) % (H - BK*BN)
+ *       replaces the inline hash of rz_linear_forward_core           impl/RzLinearForward.py:316,:349
+ *       rz_linear_backward_weight_grad_core                           impl/RzLinearBackward.py:369
+ *       rz_linear_backward_input_grad_core                            impl/RzLinearBackward.py:686,:716
+ *   hash_levels = 1:  off = ((tk*R3 + tn*R2 + R1) % R0) % (H - BK*BN)
+ *       replaces the hash of rz_linear_idx_kernel                     impl/RzLinearIdx.py:70-71
+ * out has ceil(K/BK)*ceil(N/BN) entries, index tk*ceil(N/BN) + tn.
+ */
+int rz_tile_offsets(int32_t* out, int K, int N, int H, int BK, int BN, const int32_t R[8],
+                    int hash_levels);
+
+/*
+ * Forward: Y[M,N] = (X[M,K] . W) * init_factor.
+ * Replaces rz_linear_forward_tl                                       impl/RzLinearForward.py:6-85
+ * (kernel rz_linear_forward_core                                      impl/RzLinearForward.py:271-357).
+ * X, HW, Y are device pointers of element type `dtype`; Y is fully overwritten.
+ */
+int rz_forward(const void* X, const void* HW, void* Y, int M, int K, int N, int H, int BK, int BN,
+               const int32_t R[8], float init_factor, int64_t ldx, int64_t ldy, int dtype,
+               void* stream);
+
+/*
+ * Input gradient: dX[M,K] = (dY[M,N] . W^T) * init_factor.
+ * Replaces rz_linear_backward_input_grad_tl                           impl/RzLinearBackward.py:374-449
+ * (kernel rz_linear_backward_input_grad_core                          impl/RzLinearBackward.py:642-727).
+ */
+int rz_input_grad(const void* dY, const void* HW, void* dX, int M, int K, int N, int H, int BK,
+                  int BN, const int32_t R[8], float init_factor, int64_t lddy, int64_t lddx,
+                  int dtype, void* stream);
+
+/*
+ * Bytes of device workspace rz_weight_grad needs for this problem (0 when none).
+ * The 16-bit types reduce into an fp32 image of dHW kept in the workspace.
+ */
+size_t rz_weight_grad_workspace_bytes(int M, int K, int N, int H, int BK, int BN, int dtype);
+
+/*
+ * Weight gradient: dHW[H] = sum over tiles (tk,tn) of (X^T . dY)[tile] * init_factor added at
+ * off(tk,tn); dHW is zeroed and fully overwritten by the call (element type `dtype`).
+ * Replaces rz_linear_backward_weight_grad_tl                          impl/RzLinearBackward.py:23-97
+ * (kernel rz_linear_backward_weight_grad_core                         impl/RzLinearBackward.py:291-371).
+ * Accumulation and the scatter are done in fp32 for every dtype; floating-point
+ * summation order across tiles is not fixed (atomic adds), as in the reference.
+ */
+int rz_weight_grad(const void* X, const void* dY, void* dHW, void* workspace,
+                   size_t workspace_bytes, int M, int K, int N, int H, int BK, int BN,
+                   const int32_t R[8], float init_factor, int64_t ldx, int64_t lddy, int dtype,
+                   void* stream);
+
+/*
+ * Materialise W[K,N] (row pitch ldw) from hashed_weight; edge tiles are clipped.
+ * Replaces rz_linear_idx_tl                                           impl/RzLinearIdx.py:6-45
+ * (kernel rz_linear_idx_kernel                                        impl/RzLinearIdx.py:48-77),
+ * which uses hash_levels = 1; hash_levels = 2 gives the W that the three kernels above see.
+ */
+int rz_materialize(const void* HW, void* W, int K, int N, int H, int BK, int BN,
+                   const int32_t R[8], int hash_levels, int64_t ldw, int dtype, void* stream);
+
+/*
+ * Tile offsets computed on the DEVICE into d_out[ceil(K/BK)*ceil(N/BN)] (int32), same
+ * formulas as rz_tile_offsets; lets a test compare the device hash bit for bit.
+ */
+int rz_tile_offsets_device(int32_t* d_out, int K, int N, int H, int BK, int BN,
+                           const int32_t R[8], int hash_levels, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* RZLINEAR_H */

@@ -1,0 +1,116 @@
+"""ctypes binding of librzlinear.so (the gfx950 HIP kernels behind a C ABI).
+
+The library is built in-tree by ``python -m rzlinear_amd.build``.  There is no CPU or
+PyTorch fallback: if the shared object is missing, or a tensor is not on a ROCm device,
+the operators raise.
+"""
+import ctypes
+import os
+
+import torch
+
+_PKG_DIR = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_PKG_DIR, "librzlinear.so")
+
+RZ_F32, RZ_BF16, RZ_F16 = 0, 1, 2
+_DTYPES = {torch.float32: RZ_F32, torch.bfloat16: RZ_BF16, torch.float16: RZ_F16}
+
+# every symbol that include/rzlinear.h declares
+EXPORTS = (
+    "rz_version", "rz_status_string", "rz_tile_offsets", "rz_tile_offsets_device", "rz_forward",
+    "rz_input_grad", "rz_weight_grad_workspace_bytes", "rz_weight_grad", "rz_materialize",
+)
+
+_lib = None
+
+
+class RzLinearError(RuntimeError):
+    """A librzlinear entry point returned a non-zero status."""
+
+    def __init__(self, status, message):
+        super().__init__("librzlinear: %s (status %d)" % (message, status))
+        self.status = status
+
+
+def load():
+    """Load librzlinear.so once and declare the argument types of its entry points."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            "librzlinear.so is not built (%s missing); run `python -m rzlinear_amd.build`. "
+            "rzlinear_amd has no fallback path." % LIB_PATH)
+    lib = ctypes.CDLL(LIB_PATH)
+    c_int, c_i64, c_f, c_vp, c_sz = ctypes.c_int, ctypes.c_int64, ctypes.c_float, ctypes.c_void_p, ctypes.c_size_t
+    i32p = ctypes.POINTER(ctypes.c_int32)
+    lib.rz_version.restype = c_int
+    lib.rz_version.argtypes = []
+    lib.rz_status_string.restype = ctypes.c_char_p
+    lib.rz_status_string.argtypes = [c_int]
+    lib.rz_tile_offsets.restype = c_int
+    lib.rz_tile_offsets.argtypes = [i32p, c_int, c_int, c_int, c_int, c_int, i32p, c_int]
+    lib.rz_tile_offsets_device.restype = c_int
+    lib.rz_tile_offsets_device.argtypes = [c_vp, c_int, c_int, c_int, c_int, c_int, i32p, c_int, c_vp]
+    lib.rz_forward.restype = c_int
+    lib.rz_forward.argtypes = [c_vp, c_vp, c_vp, c_int, c_int, c_int, c_int, c_int, c_int, i32p, c_f,
+                               c_i64, c_i64, c_int, c_vp]
+    lib.rz_input_grad.restype = c_int
+    lib.rz_input_grad.argtypes = lib.rz_forward.argtypes
+    lib.rz_weight_grad_workspace_bytes.restype = c_sz
+    lib.rz_weight_grad_workspace_bytes.argtypes = [c_int] * 7
+    lib.rz_weight_grad.restype = c_int
+    lib.rz_weight_grad.argtypes = [c_vp, c_vp, c_vp, c_vp, c_sz, c_int, c_int, c_int, c_int, c_int, c_int,
+                                   i32p, c_f, c_i64, c_i64, c_int, c_vp]
+    lib.rz_materialize.restype = c_int
+    lib.rz_materialize.argtypes = [c_vp, c_vp, c_int, c_int, c_int, c_int, c_int, i32p, c_int, c_i64,
+                                   c_int, c_vp]
+    _lib = lib
+    return lib
+
+
+def check(status):
+    if status != 0:
+        raise RzLinearError(status, load().rz_status_string(status).decode())
+
+
+def hash_constants(R7, R6, R5, R4, R3, R2, R1, R0):
+    """The eight hash constants as the int32[8] array the C ABI takes (index = subscript)."""
+    return (ctypes.c_int32 * 8)(int(R0), int(R1), int(R2), int(R3), int(R4), int(R5), int(R6), int(R7))
+
+
+def dtype_code(t):
+    try:
+        return _DTYPES[t.dtype]
+    except KeyError:
+        raise TypeError("rzlinear_amd supports float32, bfloat16 and float16, got %s" % t.dtype)
+
+
+def require_gpu(*tensors):
+    """All tensors must live on one ROCm device; returns the raw HIP stream handle to use."""
+    dev = tensors[0].device
+    for t in tensors:
+        if t.device.type != "cuda":
+            raise RuntimeError("rzlinear_amd runs on a ROCm GPU only; got a tensor on %s" % t.device)
+        if t.device != dev:
+            raise RuntimeError("rzlinear_amd: tensors on different devices (%s, %s)" % (dev, t.device))
+    return torch.cuda.current_stream(dev).cuda_stream
+
+
+def rows(t):
+    """A 2-D tensor with unit column stride (copied only if it has to be) and its row pitch."""
+    if t.stride(1) != 1 or (t.shape[0] > 1 and t.stride(0) < t.shape[1]):
+        t = t.contiguous()
+    ld = t.stride(0) if t.shape[0] > 1 else max(t.shape[1], 1)
+    return t, ld
+
+
+def tile_offsets(K, N, H, BLOCK_SIZE_K, BLOCK_SIZE_N, random_numbers, hash_levels=2):
+    """Host-side tile offsets as an int32 tensor [ceil(K/BK), ceil(N/BN)] (bit-exact hash)."""
+    lib = load()
+    TK, TN = -(-K // BLOCK_SIZE_K), -(-N // BLOCK_SIZE_N)
+    out = torch.empty((TK, TN), dtype=torch.int32)
+    R = (ctypes.c_int32 * 8)(*[int(v) for v in random_numbers])
+    check(lib.rz_tile_offsets(ctypes.cast(out.data_ptr(), ctypes.POINTER(ctypes.c_int32)), K, N, H,
+                              BLOCK_SIZE_K, BLOCK_SIZE_N, R, hash_levels))
+    return out

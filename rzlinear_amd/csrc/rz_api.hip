@@ -1,0 +1,274 @@
+// C ABI of librzlinear: argument checks, the host-side tile hash, small utility kernels
+// (materialise, device-side offsets, zero fill, fp32 -> element conversion) and dispatch to
+// the contraction kernels.
+#include "../../include/rzlinear.h"
+
+#include "rz_common.h"
+#include "rz_launch.h"
+
+namespace rz {
+
+static int ilog2_exact(int v) {
+  int s = 0;
+  while ((1 << s) < v) s++;
+  return ((1 << s) == v) ? s : -1;
+}
+
+static int check_tile(int BK, int BN) {
+  if (BK < 16 || BK > 256 || BN < 16 || BN > 256) return RZ_ERR_BAD_TILE;
+  if (ilog2_exact(BK) < 0 || ilog2_exact(BN) < 0) return RZ_ERR_BAD_TILE;
+  return RZ_OK;
+}
+
+// Validates the hash inputs and fills HashParams.  The reference evaluates the hash in
+// signed 32-bit arithmetic; reject inputs whose intermediates would not fit, rather than
+// silently computing something else.
+static int make_hash(HashParams* h, int K, int N, int H, int BK, int BN, const int32_t* R,
+                     int levels) {
+  if (R == nullptr) return RZ_ERR_NULL_POINTER;
+  if (K < 1 || N < 1 || H < 1) return RZ_ERR_BAD_SHAPE;
+  int st = check_tile(BK, BN);
+  if (st != RZ_OK) return st;
+  if ((long long)H <= (long long)BK * BN) return RZ_ERR_HASH_RANGE;
+  if (levels != 1 && levels != 2) return RZ_ERR_BAD_ARGUMENT;
+  for (int i = 0; i < 8; i++)
+    if (R[i] < 0) return RZ_ERR_BAD_ARGUMENT;
+  if (R[0] < 1) return RZ_ERR_BAD_ARGUMENT;
+  const long long lim = 2147483647LL;
+  const long long TK = ((long long)K + BK - 1) / BK, TN = ((long long)N + BN - 1) / BN;
+  if (TK * R[3] + TN * R[2] + R[1] > lim) return RZ_ERR_HASH_OVERFLOW;
+  if (TK * R[7] + TN * R[5] + R[4] > lim) return RZ_ERR_HASH_OVERFLOW;
+  if (levels == 2 && ((long long)R[0] - 1) * R[0] + (R[0] - 1) > lim) return RZ_ERR_HASH_OVERFLOW;
+  h->R0 = (uint32_t)R[0];
+  h->R1 = (uint32_t)R[1];
+  h->R2 = (uint32_t)R[2];
+  h->R3 = (uint32_t)R[3];
+  h->R4 = (uint32_t)R[4];
+  h->R5 = (uint32_t)R[5];
+  h->R7 = (uint32_t)R[7];
+  h->range = (uint32_t)(H - BK * BN);
+  h->BK = BK;
+  h->BN = BN;
+  h->bk_shift = ilog2_exact(BK);
+  h->bn_shift = ilog2_exact(BN);
+  h->levels = levels;
+  return RZ_OK;
+}
+
+static int dtype_bytes(int dtype) {
+  switch (dtype) {
+    case RZ_F32: return 4;
+    case RZ_BF16:
+    case RZ_F16: return 2;
+    default: return 0;
+  }
+}
+
+static hipError_t launch_gemm(int dtype, int op, const GemmParams& p, hipStream_t s) {
+  switch (dtype) {
+    case RZ_F32: return launch_gemm_f32(op, p, s);
+    case RZ_BF16: return launch_gemm_bf16(op, p, s);
+    case RZ_F16: return launch_gemm_f16(op, p, s);
+    default: return hipErrorInvalidValue;
+  }
+}
+
+// ---- utility kernels ------------------------------------------------------------------------
+__global__ void tile_offsets_kernel(int32_t* out, int TK, int TN, HashParams h) {
+  const int t = blockIdx.x * blockDim.x + threadIdx.x;
+  if (t < TK * TN) out[t] = (int32_t)tile_offset(h, (uint32_t)(t / TN), (uint32_t)(t % TN));
+}
+
+// One workgroup per W tile: the slice is copied row by row, clipped at K and N.
+template <typename E>
+__global__ void materialize_kernel(const E* __restrict__ hw, E* __restrict__ W, int K, int N, int TN,
+                                   int64_t ldw, HashParams h) {
+  const int tk = blockIdx.x / TN, tn = blockIdx.x % TN;
+  const uint32_t off = tile_offset(h, (uint32_t)tk, (uint32_t)tn);
+  const int elems = h.BK * h.BN;
+  for (int e = threadIdx.x; e < elems; e += blockDim.x) {
+    const int kk = e >> h.bn_shift, nn = e & (h.BN - 1);
+    const int k = tk * h.BK + kk, n = tn * h.BN + nn;
+    if (k < K && n < N) W[(int64_t)k * ldw + n] = hw[off + e];
+  }
+}
+
+__global__ void fill_zero_kernel(uint32_t* p, size_t words) {
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (; i < words; i += stride) p[i] = 0u;
+}
+
+template <typename T>
+__global__ void convert_from_f32_kernel(const float* __restrict__ src, T* __restrict__ dst, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) dst[i] = ElemTraits<T>::from_float(src[i]);
+}
+
+static hipError_t zero_words(void* p, size_t bytes, hipStream_t s) {
+  // bytes is a multiple of 4 for every caller (fp32 images)
+  const size_t words = bytes / 4;
+  if (words == 0) return hipSuccess;
+  size_t blocks = (words + 255) / 256;
+  if (blocks > 4096) blocks = 4096;
+  hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)blocks), dim3(256), 0, s, (uint32_t*)p, words);
+  return hipGetLastError();
+}
+
+}  // namespace rz
+
+using namespace rz;
+
+extern "C" {
+
+#define RZ_API __attribute__((visibility("default")))
+
+RZ_API int rz_version(void) { return 100; }
+
+RZ_API const char* rz_status_string(int status) {
+  switch (status) {
+    case RZ_OK: return "ok";
+    case RZ_ERR_NULL_POINTER: return "null pointer argument";
+    case RZ_ERR_BAD_SHAPE: return "bad shape: M, K, N must be >= 1 and every row pitch >= the row length";
+    case RZ_ERR_BAD_TILE: return "BLOCK_SIZE_K and BLOCK_SIZE_N must be powers of two in [16, 256]";
+    case RZ_ERR_HASH_RANGE: return "hashed_weight too small: need H > BLOCK_SIZE_K * BLOCK_SIZE_N";
+    case RZ_ERR_BAD_DTYPE: return "unsupported dtype (expected float32, bfloat16 or float16)";
+    case RZ_ERR_HASH_OVERFLOW: return "hash intermediates exceed int32 for these constants and dimensions";
+    case RZ_ERR_WORKSPACE: return "workspace missing or smaller than rz_weight_grad_workspace_bytes";
+    case RZ_ERR_LAUNCH: return "HIP kernel launch failed";
+    case RZ_ERR_BAD_ARGUMENT: return "bad argument";
+    default: return "unknown status";
+  }
+}
+
+RZ_API int rz_tile_offsets(int32_t* out, int K, int N, int H, int BK, int BN, const int32_t R[8],
+                           int hash_levels) {
+  if (out == nullptr) return RZ_ERR_NULL_POINTER;
+  HashParams h;
+  int st = make_hash(&h, K, N, H, BK, BN, R, hash_levels);
+  if (st != RZ_OK) return st;
+  const int TK = (K + BK - 1) / BK, TN = (N + BN - 1) / BN;
+  for (int tk = 0; tk < TK; tk++)
+    for (int tn = 0; tn < TN; tn++)
+      out[(size_t)tk * TN + tn] = (int32_t)tile_offset(h, (uint32_t)tk, (uint32_t)tn);
+  return RZ_OK;
+}
+
+RZ_API int rz_tile_offsets_device(int32_t* d_out, int K, int N, int H, int BK, int BN,
+                                  const int32_t R[8], int hash_levels, void* stream) {
+  if (d_out == nullptr) return RZ_ERR_NULL_POINTER;
+  HashParams h;
+  int st = make_hash(&h, K, N, H, BK, BN, R, hash_levels);
+  if (st != RZ_OK) return st;
+  const int TK = (K + BK - 1) / BK, TN = (N + BN - 1) / BN;
+  const int total = TK * TN;
+  hipLaunchKernelGGL(tile_offsets_kernel, dim3((total + 255) / 256), dim3(256), 0,
+                     (hipStream_t)stream, d_out, TK, TN, h);
+  return hipGetLastError() == hipSuccess ? RZ_OK : RZ_ERR_LAUNCH;
+}
+
+RZ_API int rz_forward(const void* X, const void* HW, void* Y, int M, int K, int N, int H, int BK,
+                      int BN, const int32_t R[8], float init_factor, int64_t ldx, int64_t ldy,
+                      int dtype, void* stream) {
+  if (X == nullptr || HW == nullptr || Y == nullptr) return RZ_ERR_NULL_POINTER;
+  if (dtype_bytes(dtype) == 0) return RZ_ERR_BAD_DTYPE;
+  if (M < 1 || ldx < K || ldy < N) return RZ_ERR_BAD_SHAPE;
+  GemmParams p = {};
+  int st = make_hash(&p.h, K, N, H, BK, BN, R, 2);
+  if (st != RZ_OK) return st;
+  p.A = X;
+  p.HW = HW;
+  p.C = Y;
+  p.I = M;
+  p.J = N;
+  p.R = K;
+  p.lda = ldx;
+  p.ldc = ldy;
+  p.scale = init_factor;
+  return launch_gemm(dtype, kForward, p, (hipStream_t)stream) == hipSuccess ? RZ_OK : RZ_ERR_LAUNCH;
+}
+
+RZ_API int rz_input_grad(const void* dY, const void* HW, void* dX, int M, int K, int N, int H,
+                         int BK, int BN, const int32_t R[8], float init_factor, int64_t lddy,
+                         int64_t lddx, int dtype, void* stream) {
+  if (dY == nullptr || HW == nullptr || dX == nullptr) return RZ_ERR_NULL_POINTER;
+  if (dtype_bytes(dtype) == 0) return RZ_ERR_BAD_DTYPE;
+  if (M < 1 || lddy < N || lddx < K) return RZ_ERR_BAD_SHAPE;
+  GemmParams p = {};
+  int st = make_hash(&p.h, K, N, H, BK, BN, R, 2);
+  if (st != RZ_OK) return st;
+  p.A = dY;
+  p.HW = HW;
+  p.C = dX;
+  p.I = M;
+  p.J = K;
+  p.R = N;
+  p.lda = lddy;
+  p.ldc = lddx;
+  p.scale = init_factor;
+  return launch_gemm(dtype, kInputGrad, p, (hipStream_t)stream) == hipSuccess ? RZ_OK : RZ_ERR_LAUNCH;
+}
+
+RZ_API size_t rz_weight_grad_workspace_bytes(int M, int K, int N, int H, int BK, int BN, int dtype) {
+  (void)M; (void)K; (void)N; (void)BK; (void)BN;
+  if (H < 1) return 0;
+  // the 16-bit types reduce into an fp32 image of dHW
+  return (dtype == RZ_BF16 || dtype == RZ_F16) ? (size_t)H * sizeof(float) : 0;
+}
+
+RZ_API int rz_weight_grad(const void* X, const void* dY, void* dHW, void* workspace,
+                          size_t workspace_bytes, int M, int K, int N, int H, int BK, int BN,
+                          const int32_t R[8], float init_factor, int64_t ldx, int64_t lddy,
+                          int dtype, void* stream) {
+  if (X == nullptr || dY == nullptr || dHW == nullptr) return RZ_ERR_NULL_POINTER;
+  if (dtype_bytes(dtype) == 0) return RZ_ERR_BAD_DTYPE;
+  if (M < 1 || ldx < K || lddy < N) return RZ_ERR_BAD_SHAPE;
+  GemmParams p = {};
+  int st = make_hash(&p.h, K, N, H, BK, BN, R, 2);
+  if (st != RZ_OK) return st;
+  const size_t need = rz_weight_grad_workspace_bytes(M, K, N, H, BK, BN, dtype);
+  if (need > 0 && (workspace == nullptr || workspace_bytes < need)) return RZ_ERR_WORKSPACE;
+  hipStream_t s = (hipStream_t)stream;
+  float* image = (dtype == RZ_F32) ? (float*)dHW : (float*)workspace;
+  if (zero_words(image, (size_t)H * sizeof(float), s) != hipSuccess) return RZ_ERR_LAUNCH;
+  p.A = X;
+  p.B = dY;
+  p.scatter = image;
+  p.I = K;
+  p.J = N;
+  p.R = M;
+  p.lda = ldx;
+  p.ldb = lddy;
+  p.scale = init_factor;
+  if (launch_gemm(dtype, kWeightGrad, p, s) != hipSuccess) return RZ_ERR_LAUNCH;
+  if (dtype == RZ_BF16) {
+    hipLaunchKernelGGL(convert_from_f32_kernel<bf16_t>, dim3((H + 255) / 256), dim3(256), 0, s, image,
+                       (bf16_t*)dHW, H);
+  } else if (dtype == RZ_F16) {
+    hipLaunchKernelGGL(convert_from_f32_kernel<f16_t>, dim3((H + 255) / 256), dim3(256), 0, s, image,
+                       (f16_t*)dHW, H);
+  }
+  return hipGetLastError() == hipSuccess ? RZ_OK : RZ_ERR_LAUNCH;
+}
+
+RZ_API int rz_materialize(const void* HW, void* W, int K, int N, int H, int BK, int BN,
+                          const int32_t R[8], int hash_levels, int64_t ldw, int dtype, void* stream) {
+  if (HW == nullptr || W == nullptr) return RZ_ERR_NULL_POINTER;
+  if (dtype_bytes(dtype) == 0) return RZ_ERR_BAD_DTYPE;
+  if (ldw < N) return RZ_ERR_BAD_SHAPE;
+  HashParams h;
+  int st = make_hash(&h, K, N, H, BK, BN, R, hash_levels);
+  if (st != RZ_OK) return st;
+  const int TK = (K + BK - 1) / BK, TN = (N + BN - 1) / BN;
+  if ((long long)TK * TN > 0x7fffffffLL) return RZ_ERR_BAD_SHAPE;
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == RZ_F32)
+    hipLaunchKernelGGL(materialize_kernel<uint32_t>, dim3(TK * TN), dim3(256), 0, s,
+                       (const uint32_t*)HW, (uint32_t*)W, K, N, TN, ldw, h);
+  else
+    hipLaunchKernelGGL(materialize_kernel<uint16_t>, dim3(TK * TN), dim3(256), 0, s,
+                       (const uint16_t*)HW, (uint16_t*)W, K, N, TN, ldw, h);
+  return hipGetLastError() == hipSuccess ? RZ_OK : RZ_ERR_LAUNCH;
+}
+
+}  // extern "C"

@@ -1,0 +1,106 @@
+// Shared device/host definitions of the gfx950 RzLinear kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace rz {
+
+// ---- element types -------------------------------------------------------------------------
+// 16-bit floats travel as raw uint16_t; only the MFMA builtins and the final conversion care
+// which format they are.
+struct bf16_t { uint16_t bits; };
+struct f16_t { uint16_t bits; };
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8_t;
+typedef __attribute__((ext_vector_type(4))) short s16x4_t;
+typedef __attribute__((ext_vector_type(16))) float f32x16_t;
+typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;
+typedef __attribute__((ext_vector_type(2))) uint32_t u32x2_t;
+
+template <typename T> struct ElemTraits;
+template <> struct ElemTraits<float> {
+  static constexpr int kBytes = 4;
+  static constexpr int kVec = 4;        // elements per 16-byte chunk
+  static constexpr int kMfmaK = 2;      // contraction depth of one v_mfma_f32_32x32x2_f32
+  static __device__ __forceinline__ float from_float(float v) { return v; }
+  static __device__ __forceinline__ float to_float(float v) { return v; }
+};
+template <> struct ElemTraits<bf16_t> {
+  static constexpr int kBytes = 2;
+  static constexpr int kVec = 8;
+  static constexpr int kMfmaK = 16;     // v_mfma_f32_32x32x16_bf16
+  static __device__ __forceinline__ bf16_t from_float(float v) {
+    __bf16 b = (__bf16)v;               // round to nearest even
+    bf16_t r;
+    __builtin_memcpy(&r.bits, &b, 2);
+    return r;
+  }
+  static __device__ __forceinline__ float to_float(bf16_t v) {
+    uint32_t u = (uint32_t)v.bits << 16;
+    float f;
+    __builtin_memcpy(&f, &u, 4);
+    return f;
+  }
+};
+template <> struct ElemTraits<f16_t> {
+  static constexpr int kBytes = 2;
+  static constexpr int kVec = 8;
+  static constexpr int kMfmaK = 16;     // v_mfma_f32_32x32x16_f16
+  static __device__ __forceinline__ f16_t from_float(float v) {
+    _Float16 h = (_Float16)v;
+    f16_t r;
+    __builtin_memcpy(&r.bits, &h, 2);
+    return r;
+  }
+  static __device__ __forceinline__ float to_float(f16_t v) {
+    _Float16 h;
+    __builtin_memcpy(&h, &v.bits, 2);
+    return (float)h;
+  }
+};
+
+// ---- tile hash -----------------------------------------------------------------------------
+// off(tk,tn) = (((tk*R3 + tn*R2 + R1) % R0) * R0 + ((tk*R7 + tn*R5 + R4) % R0)) % (H - BK*BN)
+// (levels == 1 keeps only the first term).  The host checks that every intermediate stays
+// below 2^31, so unsigned 32-bit arithmetic equals the reference's signed 32-bit arithmetic.
+struct HashParams {
+  uint32_t R0, R1, R2, R3, R4, R5, R7;
+  uint32_t range;      // H - BK*BN
+  int bk_shift, bn_shift;
+  int BK, BN;
+  int levels;
+};
+
+__host__ __device__ __forceinline__ uint32_t tile_offset(const HashParams& h, uint32_t tk,
+                                                         uint32_t tn) {
+  const uint32_t hi = (tk * h.R3 + tn * h.R2 + h.R1) % h.R0;
+  if (h.levels == 1) return hi % h.range;
+  const uint32_t lo = (tk * h.R7 + tn * h.R5 + h.R4) % h.R0;
+  return (hi * h.R0 + lo) % h.range;
+}
+
+// ---- the three contractions as one GEMM shape ----------------------------------------------
+// C[I,J] = sum_r A(i,r) * B(r,j)
+//   forward      I=M J=N R=K   A = X  (rows i, contiguous r)   B = W tiles (rows r=k, contiguous j=n)
+//   input-grad   I=M J=K R=N   A = dY (rows i, contiguous r)   B = W tiles (rows j=k, contiguous r=n)
+//   weight-grad  I=K J=N R=M   A = X  (rows r=m, contiguous i) B = dY      (rows r=m, contiguous j)
+enum Op { kForward = 0, kInputGrad = 1, kWeightGrad = 2 };
+
+struct GemmParams {
+  const void* A;
+  const void* B;      // plain B operand (weight-grad) — else unused
+  const void* HW;     // hashed weight (forward, input-grad)
+  void* C;            // plain output (forward, input-grad)
+  float* scatter;     // fp32 image of dHW (weight-grad)
+  int I, J, R;
+  int64_t lda, ldb, ldc;
+  int tiles_i, tiles_j;
+  int r_chunk;        // rows of R handled by one blockIdx.y slice (multiple of the R step)
+  float scale;
+  HashParams h;
+};
+
+}  // namespace rz

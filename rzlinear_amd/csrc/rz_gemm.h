@@ -1,0 +1,376 @@
+// One MFMA-tiled kernel template for the three RzLinear contractions on gfx950.
+//
+// A workgroup of WI*WJ wavefronts owns a TI x TJ tile of C and walks the contracted
+// dimension R in steps of TR (128 bytes of R per step).  Per step the A and B tiles go
+// global -> registers (issued one step ahead) -> LDS -> MFMA fragments.  The hashed operand
+// (W) is fetched as 16-byte pieces of hashed_weight at off(tk,tn) + kk*BN + nn; the pieces may
+// start at any element, so the loads are unaligned and rely on the hardware's unaligned
+// global access.  Tile offsets are hashed by a few threads into a small LDS table, two steps
+// ahead of their use, so the integer modulos stay off the critical path.
+//
+// LDS layouts (X = I or J extent of the operand)
+//   16-bit, R contiguous in the source : [X][TR + 8]   fragment = one ds_read_b128 per lane
+//   16-bit, X contiguous in the source : [TR][X + 16]  fragment = two ds_read_b64_tr_b16
+//       (the LDS transpose read returns, to lane c of a 16-lane group, column c of a 4 x 16
+//        block whose rows the group's lanes address four-per-row)
+//   fp32                                : [TR][X + pad], one ds_read_b32 per lane; a source
+//       with R contiguous is transposed while it is written (pad 1), else copied (pad 4)
+#pragma once
+
+#include "rz_common.h"
+
+namespace rz {
+
+enum Layout { kRContig = 0, kRStrided = 1 };
+
+template <typename T> struct Mfma;
+template <> struct Mfma<float> {
+  typedef float Frag;
+  static __device__ __forceinline__ f32x16_t run(Frag a, Frag b, f32x16_t c) {
+    return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
+  }
+};
+template <> struct Mfma<bf16_t> {
+  typedef u32x4_t Frag;
+  static __device__ __forceinline__ f32x16_t run(Frag a, Frag b, f32x16_t c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a),
+                                                   __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+  }
+};
+template <> struct Mfma<f16_t> {
+  typedef u32x4_t Frag;
+  static __device__ __forceinline__ f32x16_t run(Frag a, Frag b, f32x16_t c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, a),
+                                                  __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
+  }
+};
+
+// 16 bytes of a plain row-major matrix at (row, col..col+VEC), zero where out of range.
+template <typename T>
+__device__ __forceinline__ u32x4_t load_plain(const T* __restrict__ base, int64_t ld, int row,
+                                              int row_lim, int col, int col_lim) {
+  constexpr int VEC = ElemTraits<T>::kVec;
+  u32x4_t v = {0u, 0u, 0u, 0u};
+  if (row < row_lim && col < col_lim) {
+    const T* p = base + (int64_t)row * ld + col;
+    if (col + VEC <= col_lim) {
+      __builtin_memcpy(&v, p, 16);
+    } else {
+#pragma unroll
+      for (int e = 0; e < VEC; e++) {
+        if (col + e < col_lim) {
+          if constexpr (sizeof(T) == 2) {
+            uint16_t b;
+            __builtin_memcpy(&b, p + e, 2);
+            v[e >> 1] |= (uint32_t)b << (16 * (e & 1));
+          } else {
+            uint32_t b;
+            __builtin_memcpy(&b, p + e, 4);
+            v[e] = b;
+          }
+        }
+      }
+    }
+  }
+  return v;
+}
+
+// Zero the elements e of a 16-byte piece with col + e >= col_lim.
+template <typename T>
+__device__ __forceinline__ u32x4_t mask_tail(u32x4_t v, int col, int col_lim) {
+  constexpr int VEC = ElemTraits<T>::kVec;
+  if (col + VEC > col_lim) {
+#pragma unroll
+    for (int e = 0; e < VEC; e++) {
+      if (col + e >= col_lim) {
+        if constexpr (sizeof(T) == 2) v[e >> 1] &= (e & 1) ? 0x0000ffffu : 0xffff0000u;
+        else v[e] = 0u;
+      }
+    }
+  }
+  return v;
+}
+
+template <typename T, int OP, int TI, int TJ, int WI, int WJ>
+struct GemmKernel {
+  typedef ElemTraits<T> Tr;
+  typedef typename Mfma<T>::Frag Frag;
+  static constexpr int kThreads = 64 * WI * WJ;
+  static constexpr int VEC = Tr::kVec;
+  static constexpr bool k16 = (Tr::kBytes == 2);
+  static constexpr int TR = 128 / Tr::kBytes;
+  static constexpr int KS = Tr::kMfmaK;
+  static constexpr int A_LAYOUT = (OP == kWeightGrad) ? kRStrided : kRContig;
+  static constexpr int B_LAYOUT = (OP == kInputGrad) ? kRContig : kRStrided;
+  static constexpr int WTI = TI / WI, WTJ = TJ / WJ;   // wavefront tile
+  static constexpr int MI = WTI / 32, MJ = WTJ / 32;   // 32x32 MFMA blocks per wavefront
+  static_assert(WTI % 32 == 0 && WTJ % 32 == 0, "wavefront tile must be a multiple of 32");
+
+  template <int LAYOUT, int TX> struct Lds {
+    static constexpr int kPitch = k16 ? (LAYOUT == kRContig ? TR + 8 : TX + 16)
+                                      : (LAYOUT == kRContig ? TX + 1 : TX + 4);
+    static constexpr int kRows = (k16 && LAYOUT == kRContig) ? TX : TR;
+    static constexpr int kElems = ((kPitch * kRows + 7) / 8) * 8;
+    // source tile as seen by the global loads
+    static constexpr int kSrcRows = (LAYOUT == kRContig) ? TX : TR;
+    static constexpr int kSrcCols = (LAYOUT == kRContig) ? TR : TX;
+    static constexpr int kCpr = kSrcCols / VEC;                 // 16-byte pieces per source row
+    static constexpr int kPieces = kSrcRows * kCpr / kThreads;  // pieces per thread
+    static_assert(kSrcRows * kCpr % kThreads == 0, "tile must split evenly over the threads");
+  };
+  typedef Lds<A_LAYOUT, TI> LA;
+  typedef Lds<B_LAYOUT, TJ> LB;
+
+  static constexpr int kOffEntries =
+      (OP == kWeightGrad) ? (TI / 16) * (TJ / 16) : 2 * (TR / 16 > 0 ? TR / 16 : 1) * (TJ / 16);
+
+  struct Smem {
+    alignas(16) T a[LA::kElems];
+    alignas(16) T b[LB::kElems];
+    int off[kOffEntries];
+  };
+
+  // ---- LDS write of one staged piece -------------------------------------------------------
+  template <int LAYOUT, typename L>
+  static __device__ __forceinline__ void lds_put(T* lds, int srow, int scc, u32x4_t v) {
+    if constexpr (k16 || LAYOUT == kRStrided) {
+      *reinterpret_cast<u32x4_t*>(lds + srow * L::kPitch + scc * VEC) = v;
+    } else {
+      // fp32, R contiguous in the source: transpose to [r][x]
+#pragma unroll
+      for (int e = 0; e < 4; e++)
+        reinterpret_cast<uint32_t*>(lds)[(scc * 4 + e) * L::kPitch + srow] = v[e];
+    }
+  }
+
+  // ---- MFMA fragment of the 32-wide block starting at x_base, R sub-step ks ------------------
+  template <int LAYOUT, typename L>
+  static __device__ __forceinline__ Frag lds_frag(const T* lds, int x_base, int ks, int lane) {
+    if constexpr (!k16) {
+      return reinterpret_cast<const float*>(lds)[(ks * 2 + (lane >> 5)) * L::kPitch + x_base +
+                                                 (lane & 31)];
+    } else if constexpr (LAYOUT == kRContig) {
+      return *reinterpret_cast<const u32x4_t*>(lds + (x_base + (lane & 31)) * L::kPitch + ks * 16 +
+                                               8 * (lane >> 5));
+    } else {
+      const int g = lane >> 4, jl = lane & 15;
+      const T* p = lds + (ks * 16 + 8 * (g >> 1) + (jl >> 2)) * L::kPitch + x_base + 16 * (g & 1) +
+                   4 * (jl & 3);
+      typedef s16x4_t __attribute__((address_space(3))) * lds_s16x4_ptr;
+      const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(p));
+      const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(p + 4 * L::kPitch));
+      const u32x2_t l2 = __builtin_bit_cast(u32x2_t, lo), h2 = __builtin_bit_cast(u32x2_t, hi);
+      u32x4_t r = {l2[0], l2[1], h2[0], h2[1]};
+      return r;
+    }
+  }
+
+  // ---- hashed tiles touched by one R step ---------------------------------------------------
+  struct OffWindow { int tk0, tn0, ntn, count; };
+  static __device__ __forceinline__ OffWindow off_window(const HashParams& h, int x0_k, int span_k,
+                                                         int x0_n, int span_n) {
+    OffWindow w;
+    w.tk0 = x0_k >> h.bk_shift;
+    w.tn0 = x0_n >> h.bn_shift;
+    const int ntk = (span_k >> h.bk_shift) > 0 ? (span_k >> h.bk_shift) : 1;
+    w.ntn = (span_n >> h.bn_shift) > 0 ? (span_n >> h.bn_shift) : 1;
+    w.count = ntk * w.ntn;
+    return w;
+  }
+  static __device__ __forceinline__ void off_fill(int* tab, const HashParams& h, const OffWindow& w,
+                                                  int tid) {
+    if (tid < w.count)
+      tab[tid] = (int)tile_offset(h, (uint32_t)(w.tk0 + tid / w.ntn), (uint32_t)(w.tn0 + tid % w.ntn));
+  }
+
+  // 16 bytes of W at (k, n..n+VEC) through the offset table; zero outside K x N.
+  static __device__ __forceinline__ u32x4_t load_hashed(const T* __restrict__ hw, const HashParams& h,
+                                                        const int* tab, const OffWindow& w, int k,
+                                                        int K, int n, int N) {
+    u32x4_t v = {0u, 0u, 0u, 0u};
+    if (k < K && n < N) {
+      const int off = tab[((k >> h.bk_shift) - w.tk0) * w.ntn + ((n >> h.bn_shift) - w.tn0)];
+      const T* p = hw + off + (k & (h.BK - 1)) * h.BN + (n & (h.BN - 1));
+      __builtin_memcpy(&v, p, 16);
+      v = mask_tail<T>(v, n, N);
+    }
+    return v;
+  }
+
+  static __device__ void run(const GemmParams& p, Smem& sm) {
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int wave_i = wave / WJ, wave_j = wave % WJ;
+
+    // Workgroup ids are dealt round-robin to the 8 XCDs; renumber so that each XCD (one L2)
+    // gets a contiguous run of tiles, then walk tiles with J fastest (forward/input-grad
+    // share the streamed A panel) or in square-ish groups (weight-grad streams both).
+    int id = blockIdx.x;
+    {
+      const int nwg = gridDim.x, per = nwg >> 3, rem = nwg & 7, x = id & 7, q = id >> 3;
+      id = x * per + (x < rem ? x : rem) + q;
+    }
+    int ti, tj;
+    if constexpr (OP == kWeightGrad) {
+      constexpr int G = 8;
+      const int in_group = G * p.tiles_j;
+      const int first = (id / in_group) * G;
+      const int gsz = (p.tiles_i - first) < G ? (p.tiles_i - first) : G;
+      ti = first + (id % in_group) % gsz;
+      tj = (id % in_group) / gsz;
+    } else {
+      ti = id / p.tiles_j;
+      tj = id % p.tiles_j;
+    }
+    const int i0 = ti * TI, j0 = tj * TJ;
+    const int r_begin = blockIdx.y * p.r_chunk;
+    const int r_end = (r_begin + p.r_chunk) < p.R ? (r_begin + p.r_chunk) : p.R;
+    const int steps = (r_end - r_begin + TR - 1) / TR;
+
+    const T* __restrict__ gA = static_cast<const T*>(p.A);
+    const T* __restrict__ gB = static_cast<const T*>(p.B);
+    const T* __restrict__ gHW = static_cast<const T*>(p.HW);
+    constexpr int kOffHalf = kOffEntries / 2;
+
+    f32x16_t acc[MI][MJ];
+#pragma unroll
+    for (int a = 0; a < MI; a++)
+#pragma unroll
+      for (int b = 0; b < MJ; b++)
+#pragma unroll
+        for (int e = 0; e < 16; e++) acc[a][b][e] = 0.f;
+
+    u32x4_t ra[LA::kPieces], rb[LB::kPieces];
+
+    auto window = [&](int r0) -> OffWindow {
+      if constexpr (OP == kForward) return off_window(p.h, r0, TR, j0, TJ);
+      else return off_window(p.h, j0, TJ, r0, TR);
+    };
+    auto fetch = [&](int r0, const int* tab) {
+#pragma unroll
+      for (int q = 0; q < LA::kPieces; q++) {
+        const int c = tid + q * kThreads, srow = c / LA::kCpr, scol = (c % LA::kCpr) * VEC;
+        if constexpr (A_LAYOUT == kRContig)
+          ra[q] = load_plain<T>(gA, p.lda, i0 + srow, p.I, r0 + scol, r_end);
+        else
+          ra[q] = load_plain<T>(gA, p.lda, r0 + srow, r_end, i0 + scol, p.I);
+      }
+      OffWindow w;
+      if constexpr (OP != kWeightGrad) w = window(r0);
+#pragma unroll
+      for (int q = 0; q < LB::kPieces; q++) {
+        const int c = tid + q * kThreads, srow = c / LB::kCpr, scol = (c % LB::kCpr) * VEC;
+        if constexpr (OP == kForward)
+          rb[q] = load_hashed(gHW, p.h, tab, w, r0 + srow, r_end, j0 + scol, p.J);
+        else if constexpr (OP == kInputGrad)
+          rb[q] = load_hashed(gHW, p.h, tab, w, j0 + srow, p.J, r0 + scol, r_end);
+        else
+          rb[q] = load_plain<T>(gB, p.ldb, r0 + srow, r_end, j0 + scol, p.J);
+      }
+    };
+    auto commit = [&]() {
+#pragma unroll
+      for (int q = 0; q < LA::kPieces; q++) {
+        const int c = tid + q * kThreads;
+        lds_put<A_LAYOUT, LA>(sm.a, c / LA::kCpr, c % LA::kCpr, ra[q]);
+      }
+#pragma unroll
+      for (int q = 0; q < LB::kPieces; q++) {
+        const int c = tid + q * kThreads;
+        lds_put<B_LAYOUT, LB>(sm.b, c / LB::kCpr, c % LB::kCpr, rb[q]);
+      }
+    };
+
+    if (steps > 0) {
+      if constexpr (OP != kWeightGrad) {
+        OffWindow w0 = window(r_begin);
+        off_fill(sm.off, p.h, w0, tid);
+        if (steps > 1) {
+          OffWindow w1 = window(r_begin + TR);
+          off_fill(sm.off + kOffHalf, p.h, w1, tid);
+        }
+        __syncthreads();
+      }
+      fetch(r_begin, sm.off);
+    }
+
+    for (int s = 0; s < steps; s++) {
+      commit();
+      __syncthreads();
+      if (s + 1 < steps) fetch(r_begin + (s + 1) * TR, sm.off + ((s + 1) & 1) * kOffHalf);
+      if constexpr (OP != kWeightGrad) {
+        // slot s&1 was last read by the fetch of step s, issued before the barrier above
+        if (s + 2 < steps) {
+          OffWindow w2 = window(r_begin + (s + 2) * TR);
+          off_fill(sm.off + (s & 1) * kOffHalf, p.h, w2, tid);
+        }
+      }
+#pragma unroll
+      for (int ks = 0; ks < TR / KS; ks++) {
+        Frag fa[MI], fb[MJ];
+#pragma unroll
+        for (int a = 0; a < MI; a++)
+          fa[a] = lds_frag<A_LAYOUT, LA>(sm.a, wave_i * WTI + a * 32, ks, lane);
+#pragma unroll
+        for (int b = 0; b < MJ; b++)
+          fb[b] = lds_frag<B_LAYOUT, LB>(sm.b, wave_j * WTJ + b * 32, ks, lane);
+#pragma unroll
+        for (int a = 0; a < MI; a++)
+#pragma unroll
+          for (int b = 0; b < MJ; b++) acc[a][b] = Mfma<T>::run(fa[a], fb[b], acc[a][b]);
+      }
+      __syncthreads();
+    }
+
+    // ---- epilogue ---------------------------------------------------------------------------
+    // accumulator element e of a 32x32 block: row (e/4)*8 + (lane/32)*4 + e%4, column lane%32
+    if constexpr (OP == kWeightGrad) {
+      if (steps <= 0) return;
+      OffWindow w = off_window(p.h, i0, TI, j0, TJ);
+      off_fill(sm.off, p.h, w, tid);
+      if (kThreads < w.count) {  // never true for the instantiated tiles; kept for safety
+        for (int t = tid + kThreads; t < w.count; t += kThreads)
+          sm.off[t] = (int)tile_offset(p.h, (uint32_t)(w.tk0 + t / w.ntn), (uint32_t)(w.tn0 + t % w.ntn));
+      }
+      __syncthreads();
+#pragma unroll
+      for (int a = 0; a < MI; a++)
+#pragma unroll
+        for (int b = 0; b < MJ; b++) {
+          const int n = j0 + wave_j * WTJ + b * 32 + (lane & 31);
+#pragma unroll
+          for (int e = 0; e < 16; e++) {
+            const int k = i0 + wave_i * WTI + a * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
+            if (k < p.I && n < p.J) {
+              const int off = sm.off[((k >> p.h.bk_shift) - w.tk0) * w.ntn + ((n >> p.h.bn_shift) - w.tn0)];
+              float* dst = p.scatter + off + (k & (p.h.BK - 1)) * p.h.BN + (n & (p.h.BN - 1));
+              unsafeAtomicAdd(dst, acc[a][b][e] * p.scale);
+            }
+          }
+        }
+    } else {
+      T* __restrict__ gC = static_cast<T*>(p.C);
+#pragma unroll
+      for (int a = 0; a < MI; a++)
+#pragma unroll
+        for (int b = 0; b < MJ; b++) {
+          const int col = j0 + wave_j * WTJ + b * 32 + (lane & 31);
+#pragma unroll
+          for (int e = 0; e < 16; e++) {
+            const int row = i0 + wave_i * WTI + a * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
+            if (row < p.I && col < p.J) gC[(int64_t)row * p.ldc + col] = Tr::from_float(acc[a][b][e] * p.scale);
+          }
+        }
+    }
+  }
+};
+
+template <typename T, int OP, int TI, int TJ, int WI, int WJ>
+__global__ __launch_bounds__(64 * WI * WJ) void rz_gemm_kernel(GemmParams p) {
+  typedef GemmKernel<T, OP, TI, TJ, WI, WJ> K;
+  __shared__ typename K::Smem sm;
+  K::run(p, sm);
+}
+
+}  // namespace rz

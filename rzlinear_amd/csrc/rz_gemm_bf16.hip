@@ -1,0 +1,8 @@
+// Instantiation of the contraction kernels for element type bf16_t.
+#include "rz_gemm_inst.h"
+
+namespace rz {
+hipError_t launch_gemm_bf16(int op, GemmParams p, hipStream_t stream) {
+  return launch_gemm_t<bf16_t>(op, p, stream);
+}
+}  // namespace rz

@@ -1,0 +1,8 @@
+// Instantiation of the contraction kernels for element type f16_t.
+#include "rz_gemm_inst.h"
+
+namespace rz {
+hipError_t launch_gemm_f16(int op, GemmParams p, hipStream_t stream) {
+  return launch_gemm_t<f16_t>(op, p, stream);
+}
+}  // namespace rz

@@ -1,0 +1,8 @@
+// Instantiation of the contraction kernels for element type float.
+#include "rz_gemm_inst.h"
+
+namespace rz {
+hipError_t launch_gemm_f32(int op, GemmParams p, hipStream_t stream) {
+  return launch_gemm_t<float>(op, p, stream);
+}
+}  // namespace rz

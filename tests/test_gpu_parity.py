@@ -1,0 +1,118 @@
+"""GPU parity: the HIP kernels, called through the launchers (ctypes -> C ABI), against the
+CPU oracle on the same seeded inputs."""
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import SEED_CONSTANTS, TOL, make_inputs, rargs, rel_err
+
+pytestmark = pytest.mark.gpu
+
+R1024 = SEED_CONSTANTS[1024]
+
+# (M, K, N, H, BK, BN)
+SHAPES = [
+    (128, 128, 128, 65536, 64, 64),       # one workgroup tile, no edges
+    (256, 512, 384, 20000, 32, 64),       # reference default tile
+    (50, 100, 150, 5000, 32, 64),         # ragged everywhere, not multiples of the vector width
+    (1, 16, 16, 300, 16, 16),             # smallest tile, single row
+    (333, 257, 129, 40000, 64, 32),       # odd sizes, tile of the reference's weight-grad test
+    (200, 1024, 256, 70000, 32, 128),     # tile of the reference's idx test
+    (192, 300, 520, 70000, 128, 128),
+    (64, 600, 200, 9000, 256, 16),
+    (96, 96, 700, 9000, 16, 256),
+    (1024, 1024, 1024, 65536, 64, 64),    # the reference's CPU-path configuration
+]
+DTYPES = [torch.float32, torch.bfloat16, torch.float16]
+
+
+def _say(*a):
+    print(*a, flush=True)
+    sys.stdout.flush()
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=lambda d: str(d).split(".")[-1])
+@pytest.mark.parametrize("shape", SHAPES, ids=lambda s: "x".join(map(str, s)))
+def test_forward(oracle, shape, dtype):
+    from rzlinear_amd.impl.RzLinearForward import rz_linear_forward_tl
+    M, K, N, H, BK, BN = shape
+    _say("forward", shape, dtype)
+    (x, hw, _), (x64, hw64, _) = make_inputs(M, K, N, H, dtype, seed=1)
+    y = rz_linear_forward_tl(x, hw, 0.75, M, K, N, H, *rargs(R1024), BLOCK_SIZE_K=BK, BLOCK_SIZE_N=BN)
+    torch.cuda.synchronize()
+    assert y.shape == (M, N) and y.dtype == dtype
+    ref = oracle.forward(x64, hw64, N, BK, BN, R1024, 0.75)
+    assert rel_err(y.float().cpu().numpy(), ref) <= TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=lambda d: str(d).split(".")[-1])
+@pytest.mark.parametrize("shape", SHAPES, ids=lambda s: "x".join(map(str, s)))
+def test_input_grad(oracle, shape, dtype):
+    from rzlinear_amd.impl.RzLinearBackward import rz_linear_backward_input_grad_tl
+    M, K, N, H, BK, BN = shape
+    _say("input_grad", shape, dtype)
+    (_, hw, dy), (_, hw64, dy64) = make_inputs(M, K, N, H, dtype, seed=2)
+    dx = rz_linear_backward_input_grad_tl(dy, hw, 1.25, M, K, N, H, *rargs(R1024), BLOCK_SIZE_K=BK,
+                                          BLOCK_SIZE_N=BN)
+    torch.cuda.synchronize()
+    assert dx.shape == (M, K) and dx.dtype == dtype
+    ref = oracle.input_grad(dy64, hw64, K, BK, BN, R1024, 1.25)
+    assert rel_err(dx.float().cpu().numpy(), ref) <= TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=lambda d: str(d).split(".")[-1])
+@pytest.mark.parametrize("shape", SHAPES, ids=lambda s: "x".join(map(str, s)))
+def test_weight_grad(oracle, shape, dtype):
+    from rzlinear_amd.impl.RzLinearBackward import rz_linear_backward_weight_grad_tl
+    M, K, N, H, BK, BN = shape
+    _say("weight_grad", shape, dtype)
+    (x, _, dy), (x64, _, dy64) = make_inputs(M, K, N, H, dtype, seed=3)
+    dhw = rz_linear_backward_weight_grad_tl(x, dy, 0.5, M, K, N, H, *rargs(R1024), BLOCK_SIZE_K=BK,
+                                            BLOCK_SIZE_N=BN)
+    torch.cuda.synchronize()
+    assert dhw.shape == (H,) and dhw.dtype == dtype
+    ref = oracle.weight_grad(x64, dy64, H, BK, BN, R1024, 0.5)
+    assert rel_err(dhw.float().cpu().numpy(), ref) <= TOL[dtype]
+    # slots that no tile covers stay exactly zero
+    untouched = np.ones(H, dtype=bool)
+    untouched[np.unique(oracle.index_map(K, N, H, BK, BN, R1024))] = False
+    assert (dhw.float().cpu().numpy()[untouched] == 0).all()
+
+
+@pytest.mark.parametrize("cfg", [
+    (1024, 1024, 65536, 64, 64), (4096, 4096, 16778, 64, 64), (512, 1024, 5243, 64, 64),
+    (4096, 16384, 67109, 64, 64), (2048, 2048, 32768, 64, 64), (1000, 77, 20000, 32, 64),
+    (99999, 16, 300, 16, 16)], ids=lambda c: "x".join(map(str, c)))
+@pytest.mark.parametrize("levels", [1, 2])
+def test_device_tile_offsets_bit_exact(oracle, cfg, levels):
+    import ctypes
+    from rzlinear_amd import _lib
+    K, N, H, BK, BN = cfg
+    _say("tile_offsets", cfg, levels)
+    lib = _lib.load()
+    TK, TN = -(-K // BK), -(-N // BN)
+    for seed, R in SEED_CONSTANTS.items():
+        out = torch.empty((TK, TN), dtype=torch.int32, device="cuda")
+        _lib.check(lib.rz_tile_offsets_device(out.data_ptr(), K, N, H, BK, BN, (ctypes.c_int32 * 8)(*R),
+                                              levels, torch.cuda.current_stream().cuda_stream))
+        torch.cuda.synchronize()
+        ref = oracle.c_tile_offsets(K, N, H, BK, BN, R, levels)
+        assert np.array_equal(out.cpu().numpy().astype(np.int64), ref)
+        host = _lib.tile_offsets(K, N, H, BK, BN, R, levels).numpy().astype(np.int64)
+        assert np.array_equal(host, ref)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=lambda d: str(d).split(".")[-1])
+def test_materialize_both_hashes(oracle, dtype):
+    from rzlinear_amd.impl.RzLinearIdx import rz_linear_idx_tl, rz_linear_weight_tl
+    K, N, H, BK, BN = 1024, 1024, 65536, 32, 128
+    _say("materialize", dtype)
+    hw = torch.arange(H).to(dtype).cuda() if dtype == torch.float32 else torch.randn(H).to(dtype).cuda()
+    hw64 = hw.double().cpu().numpy()
+    R = R1024
+    w1 = rz_linear_idx_tl(hw, K, N, H, R[3], R[2], R[1], R[0], BK, BN)
+    assert np.array_equal(w1.double().cpu().numpy(), oracle.materialize(hw64, K, N, BK, BN, R, 1))
+    w2 = rz_linear_weight_tl(hw, 1000, 900, H, *rargs(R), BLOCK_SIZE_K=BK, BLOCK_SIZE_N=BN)
+    assert np.array_equal(w2.double().cpu().numpy(), oracle.materialize(hw64, 1000, 900, BK, BN, R, 2))
