@@ -1,0 +1,87 @@
+"""CPU checks of the C ABI: the library loads, exports what include/rzlinear.h declares, the
+host-side hash is bit-exact against the oracle, and bad arguments come back as status codes.
+No device compute is called here."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+R1024 = [45007, 20011, 38363, 15263, 24507, 36489, 12234, 43027]
+R0 = [45007, 29440, 22221, 32190, 14791, 1316, 35275, 26448]
+
+
+@pytest.fixture(scope="module")
+def lib():
+    from rzlinear_amd import _lib
+    if not os.path.exists(_lib.LIB_PATH):
+        from rzlinear_amd import build
+        build.build(verbose=False)
+    return _lib.load()
+
+
+def _declared():
+    text = open(os.path.join(ROOT, "include", "rzlinear.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(rz_[a-z_0-9]+)\s*\(", text)))
+
+
+def test_every_declared_symbol_is_exported(lib):
+    from rzlinear_amd import _lib
+    names = _declared()
+    assert sorted(_lib.EXPORTS) == names
+    for n in names:
+        assert hasattr(lib, n), n
+    assert lib.rz_version() >= 100
+
+
+def _R(r):
+    return (ctypes.c_int32 * 8)(*r)
+
+
+@pytest.mark.parametrize("cfg", [(1024, 1024, 65536, 64, 64), (1024, 1024, 16384, 64, 64),
+                                 (2048, 2048, 16384, 64, 64), (4096, 4096, 16778, 64, 64),
+                                 (512, 1024, 5243, 64, 64), (4096, 16384, 67109, 64, 64),
+                                 (2048, 2048, 32768, 64, 64), (4096, 4096, 16778, 32, 64),
+                                 (1000, 77, 20000, 32, 64), (99999, 99999, 66000, 256, 256),
+                                 (99999, 16, 300, 16, 16)])
+@pytest.mark.parametrize("levels", [1, 2])
+def test_host_tile_offsets_bit_exact(lib, oracle, cfg, levels):
+    from rzlinear_amd import _lib
+    K, N, H, BK, BN = cfg
+    for R in (R1024, R0):
+        got = _lib.tile_offsets(K, N, H, BK, BN, R, levels).numpy().astype(np.int64)
+        assert np.array_equal(got, oracle.c_tile_offsets(K, N, H, BK, BN, R, levels))
+
+
+def test_status_codes(lib):
+    out = (ctypes.c_int32 * 64)()
+    i32p = ctypes.POINTER(ctypes.c_int32)
+    call = lambda K, N, H, BK, BN, R, lv=2: lib.rz_tile_offsets(ctypes.cast(out, i32p), K, N, H, BK, BN, _R(R), lv)
+    assert call(128, 128, 65536, 64, 64, R1024) == 0
+    assert call(128, 128, 4096, 64, 64, R1024) == -4            # H == BK*BN
+    assert call(128, 128, 100, 64, 64, R1024) == -4
+    assert call(128, 128, 65536, 48, 64, R1024) == -3           # not a power of two
+    assert call(128, 128, 65536, 8, 64, R1024) == -3
+    assert call(128, 128, 65536, 64, 512, R1024) == -3
+    assert call(0, 128, 65536, 64, 64, R1024) == -2
+    assert call(128, 128, 65536, 64, 64, [2**31 - 1] + R1024[1:]) == -6
+    assert call(128, 128, 65536, 64, 64, [45007, -1] + R1024[2:]) == -9
+    assert call(128, 128, 65536, 64, 64, R1024, 3) == -9
+    assert lib.rz_tile_offsets(None, 128, 128, 65536, 64, 64, _R(R1024), 2) == -1
+    # device entry points validate before they touch the GPU
+    assert lib.rz_forward(None, None, None, 1, 1, 1, 65536, 64, 64, _R(R1024), 1.0, 1, 1, 0, None) == -1
+    one = ctypes.c_void_p(1)
+    assert lib.rz_forward(one, one, one, 8, 128, 128, 65536, 64, 64, _R(R1024), 1.0, 128, 128, 7, None) == -5
+    assert lib.rz_forward(one, one, one, 8, 128, 128, 65536, 64, 64, _R(R1024), 1.0, 64, 128, 0, None) == -2
+    assert lib.rz_input_grad(one, one, one, 8, 128, 128, 4096, 64, 64, _R(R1024), 1.0, 128, 128, 0, None) == -4
+    assert lib.rz_weight_grad(one, one, one, None, 0, 8, 128, 128, 65536, 64, 64, _R(R1024), 1.0, 128, 128, 1,
+                              None) == -7                         # bf16 needs the fp32 workspace
+    assert lib.rz_materialize(one, one, 128, 128, 65536, 64, 64, _R(R1024), 2, 64, 0, None) == -2
+    assert lib.rz_weight_grad_workspace_bytes(8, 128, 128, 65536, 64, 64, 0) == 0
+    assert lib.rz_weight_grad_workspace_bytes(8, 128, 128, 65536, 64, 64, 1) == 65536 * 4
+    for code in range(0, -10, -1):
+        assert lib.rz_status_string(code) not in (None, b"", b"unknown status")
+    assert lib.rz_status_string(-99) == b"unknown status"
