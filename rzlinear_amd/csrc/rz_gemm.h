@@ -2,11 +2,12 @@
 //
 // A workgroup of WI*WJ wavefronts owns a TI x TJ tile of C and walks the contracted
 // dimension R in steps of TR (128 bytes of R per step).  Per step the A and B tiles go
-// global -> registers (issued one step ahead) -> LDS -> MFMA fragments.  The hashed operand
+// global -> registers (issued one or two steps ahead) -> LDS (one or two stages) -> MFMA
+// fragments.  The hashed operand
 // (W) is fetched as 16-byte pieces of hashed_weight at off(tk,tn) + kk*BN + nn; the pieces may
 // start at any element, so the loads are unaligned and rely on the hardware's unaligned
-// global access.  Tile offsets are hashed by a few threads into a small LDS table, two steps
-// ahead of their use, so the integer modulos stay off the critical path.
+// global access.  Tile offsets are hashed by a few threads into a small LDS table, several
+// steps ahead of their use, so the integer modulos stay off the critical path.
 //
 // LDS layouts (X = I or J extent of the operand)
 //   16-bit, R contiguous in the source : [X][TR + 8]   fragment = one ds_read_b128 per lane
@@ -45,12 +46,17 @@ template <> struct Mfma<f16_t> {
   }
 };
 
-// 16 bytes of a plain row-major matrix at (row, col..col+VEC), zero where out of range.
-template <typename T>
+// 16 bytes of a plain row-major matrix at (row, col..col+VEC), zero where out of range
+// (FULL: the caller guarantees the piece is in range, no checks).
+template <typename T, bool FULL>
 __device__ __forceinline__ u32x4_t load_plain(const T* __restrict__ base, int64_t ld, int row,
                                               int row_lim, int col, int col_lim) {
   constexpr int VEC = ElemTraits<T>::kVec;
   u32x4_t v = {0u, 0u, 0u, 0u};
+  if constexpr (FULL) {
+    __builtin_memcpy(&v, base + (int64_t)row * ld + col, 16);
+    return v;
+  }
   if (row < row_lim && col < col_lim) {
     const T* p = base + (int64_t)row * ld + col;
     if (col + VEC <= col_lim) {
@@ -91,7 +97,7 @@ __device__ __forceinline__ u32x4_t mask_tail(u32x4_t v, int col, int col_lim) {
   return v;
 }
 
-template <typename T, int OP, int TI, int TJ, int WI, int WJ>
+template <typename T, int OP, int TI, int TJ, int WI, int WJ, int NSTAGE, bool FULL>
 struct GemmKernel {
   typedef ElemTraits<T> Tr;
   typedef typename Mfma<T>::Frag Frag;
@@ -121,12 +127,16 @@ struct GemmKernel {
   typedef Lds<A_LAYOUT, TI> LA;
   typedef Lds<B_LAYOUT, TJ> LB;
 
+  // offset table: kOffSlots windows (one per R step in flight) of kOffWindow entries; the
+  // weight-grad epilogue reuses it for the (TI/16) x (TJ/16) tiles of its C tile
+  static constexpr int kOffSlots = 4;
+  static constexpr int kOffWindow = (TR / 16) * (TJ / 16);
   static constexpr int kOffEntries =
-      (OP == kWeightGrad) ? (TI / 16) * (TJ / 16) : 2 * (TR / 16 > 0 ? TR / 16 : 1) * (TJ / 16);
+      (OP == kWeightGrad) ? (TI / 16) * (TJ / 16) : kOffSlots * kOffWindow;
 
   struct Smem {
-    alignas(16) T a[LA::kElems];
-    alignas(16) T b[LB::kElems];
+    alignas(16) T a[NSTAGE][LA::kElems];
+    alignas(16) T b[NSTAGE][LB::kElems];
     int off[kOffEntries];
   };
 
@@ -183,16 +193,20 @@ struct GemmKernel {
       tab[tid] = (int)tile_offset(h, (uint32_t)(w.tk0 + tid / w.ntn), (uint32_t)(w.tn0 + tid % w.ntn));
   }
 
-  // 16 bytes of W at (k, n..n+VEC) through the offset table; zero outside K x N.
-  static __device__ __forceinline__ u32x4_t load_hashed(const T* __restrict__ hw, const HashParams& h,
-                                                        const int* tab, const OffWindow& w, int k,
+  // Element index in hashed_weight of W[k, n] through the offset table (k, n inside the window).
+  static __device__ __forceinline__ int hashed_index(const HashParams& h, const int* tab,
+                                                     const OffWindow& w, int k, int n) {
+    const int off = tab[((k >> h.bk_shift) - w.tk0) * w.ntn + ((n >> h.bn_shift) - w.tn0)];
+    return off + (k & (h.BK - 1)) * h.BN + (n & (h.BN - 1));
+  }
+
+  // 16 bytes of W starting at element `idx` of hashed_weight; zero outside K x N.
+  static __device__ __forceinline__ u32x4_t load_hashed(const T* __restrict__ hw, int idx, int k,
                                                         int K, int n, int N) {
     u32x4_t v = {0u, 0u, 0u, 0u};
-    if (k < K && n < N) {
-      const int off = tab[((k >> h.bk_shift) - w.tk0) * w.ntn + ((n >> h.bn_shift) - w.tn0)];
-      const T* p = hw + off + (k & (h.BK - 1)) * h.BN + (n & (h.BN - 1));
-      __builtin_memcpy(&v, p, 16);
-      v = mask_tail<T>(v, n, N);
+    if (FULL || (k < K && n < N)) {
+      __builtin_memcpy(&v, hw + idx, 16);
+      if constexpr (!FULL) v = mask_tail<T>(v, n, N);
     }
     return v;
   }
@@ -231,7 +245,6 @@ struct GemmKernel {
     const T* __restrict__ gA = static_cast<const T*>(p.A);
     const T* __restrict__ gB = static_cast<const T*>(p.B);
     const T* __restrict__ gHW = static_cast<const T*>(p.HW);
-    constexpr int kOffHalf = kOffEntries / 2;
 
     f32x16_t acc[MI][MJ];
 #pragma unroll
@@ -243,84 +256,155 @@ struct GemmKernel {
 
     u32x4_t ra[LA::kPieces], rb[LB::kPieces];
 
-    auto window = [&](int r0) -> OffWindow {
+    auto window = [&](int step) -> OffWindow {
+      const int r0 = r_begin + step * TR;
       if constexpr (OP == kForward) return off_window(p.h, r0, TR, j0, TJ);
       else return off_window(p.h, j0, TJ, r0, TR);
     };
-    auto fetch = [&](int r0, const int* tab) {
+    // hash the tiles of R step `step` into its slot of the offset table
+    auto hash_step = [&](int step) {
+      if constexpr (OP != kWeightGrad) {
+        if (step < steps) {
+          const OffWindow w = window(step);
+          off_fill(sm.off + (step & (kOffSlots - 1)) * kOffWindow, p.h, w, tid);
+        }
+      }
+    };
+    // global -> registers for R step `step`
+    auto fetch = [&](int step) {
+      const int r0 = r_begin + step * TR;
 #pragma unroll
       for (int q = 0; q < LA::kPieces; q++) {
         const int c = tid + q * kThreads, srow = c / LA::kCpr, scol = (c % LA::kCpr) * VEC;
         if constexpr (A_LAYOUT == kRContig)
-          ra[q] = load_plain<T>(gA, p.lda, i0 + srow, p.I, r0 + scol, r_end);
+          ra[q] = load_plain<T, FULL>(gA, p.lda, i0 + srow, p.I, r0 + scol, r_end);
         else
-          ra[q] = load_plain<T>(gA, p.lda, r0 + srow, r_end, i0 + scol, p.I);
+          ra[q] = load_plain<T, FULL>(gA, p.lda, r0 + srow, r_end, i0 + scol, p.I);
       }
-      OffWindow w;
-      if constexpr (OP != kWeightGrad) w = window(r0);
+      if constexpr (OP == kWeightGrad) {
 #pragma unroll
-      for (int q = 0; q < LB::kPieces; q++) {
-        const int c = tid + q * kThreads, srow = c / LB::kCpr, scol = (c % LB::kCpr) * VEC;
-        if constexpr (OP == kForward)
-          rb[q] = load_hashed(gHW, p.h, tab, w, r0 + srow, r_end, j0 + scol, p.J);
-        else if constexpr (OP == kInputGrad)
-          rb[q] = load_hashed(gHW, p.h, tab, w, j0 + srow, p.J, r0 + scol, r_end);
-        else
-          rb[q] = load_plain<T>(gB, p.ldb, r0 + srow, r_end, j0 + scol, p.J);
+        for (int q = 0; q < LB::kPieces; q++) {
+          const int c = tid + q * kThreads, srow = c / LB::kCpr, scol = (c % LB::kCpr) * VEC;
+          rb[q] = load_plain<T, FULL>(gB, p.ldb, r0 + srow, r_end, j0 + scol, p.J);
+        }
+      } else {
+        // all table lookups first (one LDS round trip), then the loads
+        const OffWindow w = window(step);
+        const int* tab = sm.off + (step & (kOffSlots - 1)) * kOffWindow;
+        int idx[LB::kPieces];
+#pragma unroll
+        for (int q = 0; q < LB::kPieces; q++) {
+          const int c = tid + q * kThreads, srow = c / LB::kCpr, scol = (c % LB::kCpr) * VEC;
+          const int k = (OP == kForward) ? r0 + srow : j0 + srow;
+          const int n = (OP == kForward) ? j0 + scol : r0 + scol;
+          idx[q] = hashed_index(p.h, tab, w, k, n);
+        }
+#pragma unroll
+        for (int q = 0; q < LB::kPieces; q++) {
+          const int c = tid + q * kThreads, srow = c / LB::kCpr, scol = (c % LB::kCpr) * VEC;
+          if constexpr (OP == kForward)
+            rb[q] = load_hashed(gHW, idx[q], r0 + srow, r_end, j0 + scol, p.J);
+          else
+            rb[q] = load_hashed(gHW, idx[q], j0 + srow, p.J, r0 + scol, r_end);
+        }
       }
     };
-    auto commit = [&]() {
+    // registers -> LDS stage `st`
+    auto commit = [&](int st) {
 #pragma unroll
       for (int q = 0; q < LA::kPieces; q++) {
         const int c = tid + q * kThreads;
-        lds_put<A_LAYOUT, LA>(sm.a, c / LA::kCpr, c % LA::kCpr, ra[q]);
+        lds_put<A_LAYOUT, LA>(sm.a[st], c / LA::kCpr, c % LA::kCpr, ra[q]);
       }
 #pragma unroll
       for (int q = 0; q < LB::kPieces; q++) {
         const int c = tid + q * kThreads;
-        lds_put<B_LAYOUT, LB>(sm.b, c / LB::kCpr, c % LB::kCpr, rb[q]);
+        lds_put<B_LAYOUT, LB>(sm.b[st], c / LB::kCpr, c % LB::kCpr, rb[q]);
+      }
+    };
+    // MFMAs of one R step out of LDS stage `st`; fragments are read one sub-step ahead
+    auto compute = [&](int st) {
+      constexpr int NKS = TR / KS;
+      Frag fa[2][MI], fb[2][MJ];
+      auto frags = [&](int ks, int buf) {
+#pragma unroll
+        for (int a = 0; a < MI; a++)
+          fa[buf][a] = lds_frag<A_LAYOUT, LA>(sm.a[st], wave_i * WTI + a * 32, ks, lane);
+#pragma unroll
+        for (int b = 0; b < MJ; b++)
+          fb[buf][b] = lds_frag<B_LAYOUT, LB>(sm.b[st], wave_j * WTJ + b * 32, ks, lane);
+      };
+      frags(0, 0);
+#pragma unroll
+      for (int ks = 0; ks < NKS; ks++) {
+        if (ks + 1 < NKS) frags(ks + 1, (ks + 1) & 1);
+#pragma unroll
+        for (int a = 0; a < MI; a++)
+#pragma unroll
+          for (int b = 0; b < MJ; b++)
+            acc[a][b] = Mfma<T>::run(fa[ks & 1][a], fb[ks & 1][b], acc[a][b]);
+        // scheduling hint: spread the LDS reads of the next sub-step between this sub-step's
+        // MFMAs (one read after each MFMA), so that their latency hides behind matrix work
+        constexpr int kReads = (k16 && A_LAYOUT == kRStrided ? 2 : 1) * MI +
+                               (k16 && B_LAYOUT == kRStrided ? 2 : 1) * MJ;
+        if constexpr (MI * MJ >= kReads) {
+          if (ks + 1 < NKS) {
+#pragma unroll
+            for (int i = 0; i < kReads; i++) {
+              __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // 1 MFMA
+              __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // 1 LDS read
+            }
+            __builtin_amdgcn_sched_group_barrier(0x008, MI * MJ - kReads, 0);
+          } else {
+            __builtin_amdgcn_sched_group_barrier(0x008, MI * MJ, 0);
+          }
+        }
       }
     };
 
     if (steps > 0) {
-      if constexpr (OP != kWeightGrad) {
-        OffWindow w0 = window(r_begin);
-        off_fill(sm.off, p.h, w0, tid);
-        if (steps > 1) {
-          OffWindow w1 = window(r_begin + TR);
-          off_fill(sm.off + kOffHalf, p.h, w1, tid);
-        }
+      hash_step(0);
+      hash_step(1);
+      hash_step(2);
+      if constexpr (OP != kWeightGrad) __syncthreads();
+      fetch(0);
+    }
+    if constexpr (NSTAGE == 1) {
+      // one LDS stage: write it, read it, two barriers per step; relies on several
+      // workgroups per compute unit to overlap the phases
+      for (int s = 0; s < steps; s++) {
+        commit(0);
+        __syncthreads();
+        if (s + 1 < steps) fetch(s + 1);
+        hash_step(s + 3);
+        compute(0);
         __syncthreads();
       }
-      fetch(r_begin, sm.off);
-    }
-
-    for (int s = 0; s < steps; s++) {
-      commit();
-      __syncthreads();
-      if (s + 1 < steps) fetch(r_begin + (s + 1) * TR, sm.off + ((s + 1) & 1) * kOffHalf);
-      if constexpr (OP != kWeightGrad) {
-        // slot s&1 was last read by the fetch of step s, issued before the barrier above
-        if (s + 2 < steps) {
-          OffWindow w2 = window(r_begin + (s + 2) * TR);
-          off_fill(sm.off + (s & 1) * kOffHalf, p.h, w2, tid);
+    } else {
+      // two LDS stages, one barrier per step: while stage s&1 feeds the MFMAs, the registers
+      // loaded during the previous step go into the other stage and the loads of step s+2
+      // are issued.  The steady-state loop carries no conditions; the last two steps are peeled.
+      if (steps > 0) {
+        commit(0);
+        if (steps > 1) fetch(1);
+        hash_step(3);
+        __syncthreads();
+        int s = 0;
+        for (; s + 2 < steps; s++) {
+          commit((s + 1) & 1);
+          fetch(s + 2);
+          hash_step(s + 4);
+          compute(s & 1);
+          __syncthreads();
         }
+        if (s + 1 < steps) {
+          commit((s + 1) & 1);
+          compute(s & 1);
+          __syncthreads();
+          s++;
+        }
+        compute(s & 1);
       }
-#pragma unroll
-      for (int ks = 0; ks < TR / KS; ks++) {
-        Frag fa[MI], fb[MJ];
-#pragma unroll
-        for (int a = 0; a < MI; a++)
-          fa[a] = lds_frag<A_LAYOUT, LA>(sm.a, wave_i * WTI + a * 32, ks, lane);
-#pragma unroll
-        for (int b = 0; b < MJ; b++)
-          fb[b] = lds_frag<B_LAYOUT, LB>(sm.b, wave_j * WTJ + b * 32, ks, lane);
-#pragma unroll
-        for (int a = 0; a < MI; a++)
-#pragma unroll
-          for (int b = 0; b < MJ; b++) acc[a][b] = Mfma<T>::run(fa[a], fb[b], acc[a][b]);
-      }
-      __syncthreads();
     }
 
     // ---- epilogue ---------------------------------------------------------------------------
@@ -342,7 +426,7 @@ struct GemmKernel {
 #pragma unroll
           for (int e = 0; e < 16; e++) {
             const int k = i0 + wave_i * WTI + a * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
-            if (k < p.I && n < p.J) {
+            if (FULL || (k < p.I && n < p.J)) {
               const int off = sm.off[((k >> p.h.bk_shift) - w.tk0) * w.ntn + ((n >> p.h.bn_shift) - w.tn0)];
               float* dst = p.scatter + off + (k & (p.h.BK - 1)) * p.h.BN + (n & (p.h.BN - 1));
               unsafeAtomicAdd(dst, acc[a][b][e] * p.scale);
@@ -359,18 +443,18 @@ struct GemmKernel {
 #pragma unroll
           for (int e = 0; e < 16; e++) {
             const int row = i0 + wave_i * WTI + a * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
-            if (row < p.I && col < p.J) gC[(int64_t)row * p.ldc + col] = Tr::from_float(acc[a][b][e] * p.scale);
+            if (FULL || (row < p.I && col < p.J)) gC[(int64_t)row * p.ldc + col] = Tr::from_float(acc[a][b][e] * p.scale);
           }
         }
     }
   }
 };
 
-template <typename T, int OP, int TI, int TJ, int WI, int WJ>
+template <typename T, int OP, int TI, int TJ, int WI, int WJ, int NSTAGE, bool FULL>
 __global__ __launch_bounds__(64 * WI * WJ) void rz_gemm_kernel(GemmParams p) {
-  typedef GemmKernel<T, OP, TI, TJ, WI, WJ> K;
-  __shared__ typename K::Smem sm;
-  K::run(p, sm);
+  typedef GemmKernel<T, OP, TI, TJ, WI, WJ, NSTAGE, FULL> K;
+  extern __shared__ __attribute__((aligned(16))) unsigned char rz_smem_raw[];
+  K::run(p, *reinterpret_cast<typename K::Smem*>(rz_smem_raw));
 }
 
 }  // namespace rz
