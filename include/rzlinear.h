@@ -94,7 +94,10 @@ int rz_input_grad(const void* dY, const void* HW, void* dX, int M, int K, int N,
 
 /*
  * Bytes of device workspace rz_weight_grad needs for this problem (0 when none).
- * The 16-bit types reduce into an fp32 image of dHW kept in the workspace.
+ * When hashed_weight is small enough for an fp32 image of dHW to fit the LDS of a compute
+ * unit, every workgroup stores one partial image ([workgroups][H rounded up to 4] floats) that
+ * a second kernel adds up; otherwise the 16-bit types need an fp32 image of dHW (H floats)
+ * for the atomic adds and fp32 needs nothing.
  */
 size_t rz_weight_grad_workspace_bytes(int M, int K, int N, int H, int BK, int BN, int dtype);
 
@@ -103,8 +106,9 @@ size_t rz_weight_grad_workspace_bytes(int M, int K, int N, int H, int BK, int BN
  * off(tk,tn); dHW is zeroed and fully overwritten by the call (element type `dtype`).
  * Replaces rz_linear_backward_weight_grad_tl                          impl/RzLinearBackward.py:23-97
  * (kernel rz_linear_backward_weight_grad_core                         impl/RzLinearBackward.py:291-371).
- * Accumulation and the scatter are done in fp32 for every dtype; floating-point
- * summation order across tiles is not fixed (atomic adds), as in the reference.
+ * Accumulation and the scatter are done in fp32 for every dtype.  With the LDS-image path
+ * the only unordered sums are the LDS adds inside one workgroup; with global atomics the
+ * summation order across tiles is not fixed, as in the reference.
  */
 int rz_weight_grad(const void* X, const void* dY, void* dHW, void* workspace,
                    size_t workspace_bytes, int M, int K, int N, int H, int BK, int BN,

@@ -64,11 +64,12 @@ static int dtype_bytes(int dtype) {
   }
 }
 
-static hipError_t launch_gemm(int dtype, int op, const GemmParams& p, hipStream_t s) {
+static hipError_t launch_gemm(int dtype, int op, const GemmParams& p, const WeightGradPlan* plan,
+                              hipStream_t s) {
   switch (dtype) {
-    case RZ_F32: return launch_gemm_f32(op, p, s);
-    case RZ_BF16: return launch_gemm_bf16(op, p, s);
-    case RZ_F16: return launch_gemm_f16(op, p, s);
+    case RZ_F32: return launch_gemm_f32(op, p, plan, s);
+    case RZ_BF16: return launch_gemm_bf16(op, p, plan, s);
+    case RZ_F16: return launch_gemm_f16(op, p, plan, s);
     default: return hipErrorInvalidValue;
   }
 }
@@ -103,6 +104,38 @@ template <typename T>
 __global__ void convert_from_f32_kernel(const float* __restrict__ src, T* __restrict__ dst, int n) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i < n) dst[i] = ElemTraits<T>::from_float(src[i]);
+}
+
+// dHW[h] = sum over the partial images of part[p][h], converted to the element type.  A
+// workgroup of 256 threads owns 16 groups of four slots; 16 thread groups each add up every
+// 16th partial image, then the groups are combined through LDS in a fixed order, so the
+// result does not depend on scheduling.
+template <typename T>
+__global__ __launch_bounds__(256) void reduce_partials_kernel(const float* __restrict__ part,
+                                                              T* __restrict__ out, int H, int pitch,
+                                                              int nparts) {
+  __shared__ float4 sums[16][16];
+  const int q = threadIdx.x & 15, g = threadIdx.x >> 4;
+  const int slot = (blockIdx.x * 16 + q) * 4;
+  float4 s = {0.f, 0.f, 0.f, 0.f};
+  if (slot < pitch) {
+    for (int p = g; p < nparts; p += 16) {
+      const float4 v = *reinterpret_cast<const float4*>(part + (size_t)p * pitch + slot);
+      s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+    }
+  }
+  sums[g][q] = s;
+  __syncthreads();
+  if (g == 0 && slot < pitch) {
+    for (int i = 1; i < 16; i++) {
+      const float4 v = sums[i][q];
+      s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+    }
+    const float r[4] = {s.x, s.y, s.z, s.w};
+#pragma unroll
+    for (int e = 0; e < 4; e++)
+      if (slot + e < H) out[slot + e] = ElemTraits<T>::from_float(r[e]);
+  }
 }
 
 static hipError_t zero_words(void* p, size_t bytes, hipStream_t s) {
@@ -185,7 +218,7 @@ RZ_API int rz_forward(const void* X, const void* HW, void* Y, int M, int K, int 
   p.lda = ldx;
   p.ldc = ldy;
   p.scale = init_factor;
-  return launch_gemm(dtype, kForward, p, (hipStream_t)stream) == hipSuccess ? RZ_OK : RZ_ERR_LAUNCH;
+  return launch_gemm(dtype, kForward, p, nullptr, (hipStream_t)stream) == hipSuccess ? RZ_OK : RZ_ERR_LAUNCH;
 }
 
 RZ_API int rz_input_grad(const void* dY, const void* HW, void* dX, int M, int K, int N, int H,
@@ -206,14 +239,14 @@ RZ_API int rz_input_grad(const void* dY, const void* HW, void* dX, int M, int K,
   p.lda = lddy;
   p.ldc = lddx;
   p.scale = init_factor;
-  return launch_gemm(dtype, kInputGrad, p, (hipStream_t)stream) == hipSuccess ? RZ_OK : RZ_ERR_LAUNCH;
+  return launch_gemm(dtype, kInputGrad, p, nullptr, (hipStream_t)stream) == hipSuccess ? RZ_OK : RZ_ERR_LAUNCH;
 }
 
 RZ_API size_t rz_weight_grad_workspace_bytes(int M, int K, int N, int H, int BK, int BN, int dtype) {
-  (void)M; (void)K; (void)N; (void)BK; (void)BN;
-  if (H < 1) return 0;
-  // the 16-bit types reduce into an fp32 image of dHW
-  return (dtype == RZ_BF16 || dtype == RZ_F16) ? (size_t)H * sizeof(float) : 0;
+  (void)BK; (void)BN;
+  const int eb = dtype_bytes(dtype);
+  if (eb == 0 || M < 1 || K < 1 || N < 1 || H < 1) return 0;
+  return plan_weight_grad(M, K, N, H, eb).workspace_bytes;
 }
 
 RZ_API int rz_weight_grad(const void* X, const void* dY, void* dHW, void* workspace,
@@ -226,21 +259,41 @@ RZ_API int rz_weight_grad(const void* X, const void* dY, void* dHW, void* worksp
   GemmParams p = {};
   int st = make_hash(&p.h, K, N, H, BK, BN, R, 2);
   if (st != RZ_OK) return st;
-  const size_t need = rz_weight_grad_workspace_bytes(M, K, N, H, BK, BN, dtype);
-  if (need > 0 && (workspace == nullptr || workspace_bytes < need)) return RZ_ERR_WORKSPACE;
+  const WeightGradPlan plan = plan_weight_grad(M, K, N, H, dtype_bytes(dtype));
+  if (plan.workspace_bytes > 0 && (workspace == nullptr || workspace_bytes < plan.workspace_bytes))
+    return RZ_ERR_WORKSPACE;
   hipStream_t s = (hipStream_t)stream;
-  float* image = (dtype == RZ_F32) ? (float*)dHW : (float*)workspace;
-  if (zero_words(image, (size_t)H * sizeof(float), s) != hipSuccess) return RZ_ERR_LAUNCH;
   p.A = X;
   p.B = dY;
-  p.scatter = image;
   p.I = K;
   p.J = N;
   p.R = M;
   p.lda = ldx;
   p.ldb = lddy;
   p.scale = init_factor;
-  if (launch_gemm(dtype, kWeightGrad, p, s) != hipSuccess) return RZ_ERR_LAUNCH;
+  if (plan.image_pitch > 0) {
+    // every workgroup sums its tiles into an LDS image of dHW and stores it as a partial image;
+    // the partial images are then added up (no global atomics, fixed summation order)
+    p.scatter = (float*)workspace;
+    if (launch_gemm(dtype, kWeightGrad, p, &plan, s) != hipSuccess) return RZ_ERR_LAUNCH;
+    const int blocks = (plan.image_pitch / 4 + 15) / 16;
+    const int nparts = (int)plan.workgroups;
+    if (dtype == RZ_F32)
+      hipLaunchKernelGGL(reduce_partials_kernel<float>, dim3(blocks), dim3(256), 0, s, p.scatter,
+                         (float*)dHW, H, plan.image_pitch, nparts);
+    else if (dtype == RZ_BF16)
+      hipLaunchKernelGGL(reduce_partials_kernel<bf16_t>, dim3(blocks), dim3(256), 0, s, p.scatter,
+                         (bf16_t*)dHW, H, plan.image_pitch, nparts);
+    else
+      hipLaunchKernelGGL(reduce_partials_kernel<f16_t>, dim3(blocks), dim3(256), 0, s, p.scatter,
+                         (f16_t*)dHW, H, plan.image_pitch, nparts);
+    return hipGetLastError() == hipSuccess ? RZ_OK : RZ_ERR_LAUNCH;
+  }
+  // hashed_weight too large for an LDS image: tiles go to an fp32 image of dHW by global atomics
+  float* image = (dtype == RZ_F32) ? (float*)dHW : (float*)workspace;
+  if (zero_words(image, (size_t)H * sizeof(float), s) != hipSuccess) return RZ_ERR_LAUNCH;
+  p.scatter = image;
+  if (launch_gemm(dtype, kWeightGrad, p, &plan, s) != hipSuccess) return RZ_ERR_LAUNCH;
   if (dtype == RZ_BF16) {
     hipLaunchKernelGGL(convert_from_f32_kernel<bf16_t>, dim3((H + 255) / 256), dim3(256), 0, s, image,
                        (bf16_t*)dHW, H);

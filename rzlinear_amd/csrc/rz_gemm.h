@@ -11,9 +11,10 @@
 //
 // LDS layouts (X = I or J extent of the operand)
 //   16-bit, R contiguous in the source : [X][TR + 8]   fragment = one ds_read_b128 per lane
-//   16-bit, X contiguous in the source : [TR][X + 16]  fragment = two ds_read_b64_tr_b16
+//   16-bit, X contiguous in the source : [TR][X + 32]  fragment = two ds_read_b64_tr_b16
 //       (the LDS transpose read returns, to lane c of a 16-lane group, column c of a 4 x 16
-//        block whose rows the group's lanes address four-per-row)
+//        block whose rows the group's lanes address four-per-row; 32 lanes touch 4 rows x 64
+//        bytes, and the 64-byte row skew of this pitch keeps those on distinct banks)
 //   fp32                                : [TR][X + pad], one ds_read_b32 per lane; a source
 //       with R contiguous is transposed while it is written (pad 1), else copied (pad 4)
 #pragma once
@@ -113,7 +114,7 @@ struct GemmKernel {
   static_assert(WTI % 32 == 0 && WTJ % 32 == 0, "wavefront tile must be a multiple of 32");
 
   template <int LAYOUT, int TX> struct Lds {
-    static constexpr int kPitch = k16 ? (LAYOUT == kRContig ? TR + 8 : TX + 16)
+    static constexpr int kPitch = k16 ? (LAYOUT == kRContig ? TR + 8 : TX + 32)
                                       : (LAYOUT == kRContig ? TX + 1 : TX + 4);
     static constexpr int kRows = (k16 && LAYOUT == kRContig) ? TX : TR;
     static constexpr int kElems = ((kPitch * kRows + 7) / 8) * 8;
@@ -139,6 +140,9 @@ struct GemmKernel {
     alignas(16) T b[NSTAGE][LB::kElems];
     int off[kOffEntries];
   };
+  // after the last R step the operand stages are dead; weight-grad may keep an fp32 image of
+  // dHW there
+  static constexpr size_t kImageBytes = sizeof(T) * NSTAGE * (size_t)(LA::kElems + LB::kElems);
 
   // ---- LDS write of one staged piece -------------------------------------------------------
   template <int LAYOUT, typename L>
@@ -347,17 +351,21 @@ struct GemmKernel {
         // MFMAs (one read after each MFMA), so that their latency hides behind matrix work
         constexpr int kReads = (k16 && A_LAYOUT == kRStrided ? 2 : 1) * MI +
                                (k16 && B_LAYOUT == kRStrided ? 2 : 1) * MJ;
-        if constexpr (MI * MJ >= kReads) {
-          if (ks + 1 < NKS) {
+        constexpr int kMfmas = MI * MJ;
+        if (ks + 1 < NKS) {
 #pragma unroll
-            for (int i = 0; i < kReads; i++) {
-              __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // 1 MFMA
-              __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // 1 LDS read
-            }
-            __builtin_amdgcn_sched_group_barrier(0x008, MI * MJ - kReads, 0);
-          } else {
-            __builtin_amdgcn_sched_group_barrier(0x008, MI * MJ, 0);
+          for (int i = 0; i < kMfmas; i++) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // 1 MFMA
+            // its share of the LDS reads (compile-time: the loop is unrolled)
+            if ((kReads * (i + 1)) / kMfmas - (kReads * i) / kMfmas == 1)
+              __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            else if ((kReads * (i + 1)) / kMfmas - (kReads * i) / kMfmas == 2)
+              __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+            else if ((kReads * (i + 1)) / kMfmas - (kReads * i) / kMfmas == 3)
+              __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);
           }
+        } else {
+          __builtin_amdgcn_sched_group_barrier(0x008, kMfmas, 0);
         }
       }
     };
@@ -394,6 +402,9 @@ struct GemmKernel {
           commit((s + 1) & 1);
           fetch(s + 2);
           hash_step(s + 4);
+          // keep the global loads ahead of the MFMAs: their latency must hide behind this
+          // step's matrix work, not be met at the next step's LDS writes
+          __builtin_amdgcn_sched_barrier(0);
           compute(s & 1);
           __syncthreads();
         }
@@ -410,29 +421,98 @@ struct GemmKernel {
     // ---- epilogue ---------------------------------------------------------------------------
     // accumulator element e of a 32x32 block: row (e/4)*8 + (lane/32)*4 + e%4, column lane%32
     if constexpr (OP == kWeightGrad) {
-      if (steps <= 0) return;
-      OffWindow w = off_window(p.h, i0, TI, j0, TJ);
-      off_fill(sm.off, p.h, w, tid);
-      if (kThreads < w.count) {  // never true for the instantiated tiles; kept for safety
-        for (int t = tid + kThreads; t < w.count; t += kThreads)
-          sm.off[t] = (int)tile_offset(p.h, (uint32_t)(w.tk0 + t / w.ntn), (uint32_t)(w.tn0 + t % w.ntn));
+      const bool image_mode = p.image_pitch > 0;
+      float* image = reinterpret_cast<float*>(&sm);   // aliases the operand stages
+      __syncthreads();                                 // every wavefront is done reading them
+      if (image_mode) {
+        const float4 z = {0.f, 0.f, 0.f, 0.f};
+        for (int i = tid * 4; i < p.image_pitch; i += kThreads * 4) *reinterpret_cast<float4*>(image + i) = z;
       }
+      const OffWindow w = off_window(p.h, i0, TI, j0, TJ);
+      for (int t = tid; t < w.count; t += kThreads)
+        sm.off[t] = (int)tile_offset(p.h, (uint32_t)(w.tk0 + t / w.ntn), (uint32_t)(w.tn0 + t % w.ntn));
       __syncthreads();
+      // Scatter-add of the accumulators.  The four rows e&3 of a row group (e>>2) are adjacent
+      // rows of one hashed tile (tiles are at least 16 rows), so one table lookup per row
+      // group gives all four addresses; the lookups of a 32x32 block are issued together and
+      // the adds follow back to back.
+      auto scatter = [&](float* target) {
+        if (steps <= 0) return;
 #pragma unroll
-      for (int a = 0; a < MI; a++)
+        for (int a = 0; a < MI; a++)
 #pragma unroll
-        for (int b = 0; b < MJ; b++) {
-          const int n = j0 + wave_j * WTJ + b * 32 + (lane & 31);
+          for (int b = 0; b < MJ; b++) {
+            const int n = j0 + wave_j * WTJ + b * 32 + (lane & 31);
+            int base[4];
+            bool ok[4];
 #pragma unroll
-          for (int e = 0; e < 16; e++) {
-            const int k = i0 + wave_i * WTI + a * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
-            if (FULL || (k < p.I && n < p.J)) {
-              const int off = sm.off[((k >> p.h.bk_shift) - w.tk0) * w.ntn + ((n >> p.h.bn_shift) - w.tn0)];
-              float* dst = p.scatter + off + (k & (p.h.BK - 1)) * p.h.BN + (n & (p.h.BN - 1));
-              unsafeAtomicAdd(dst, acc[a][b][e] * p.scale);
+            for (int g = 0; g < 4; g++) {
+              const int k = i0 + wave_i * WTI + a * 32 + g * 8 + (lane >> 5) * 4;
+              ok[g] = FULL || (k < p.I && n < p.J);
+              base[g] = sm.off[((k >> p.h.bk_shift) - w.tk0) * w.ntn + ((n >> p.h.bn_shift) - w.tn0)] +
+                        (k & (p.h.BK - 1)) * p.h.BN + (n & (p.h.BN - 1));
+            }
+#pragma unroll
+            for (int e = 0; e < 16; e++) {
+              const int k = i0 + wave_i * WTI + a * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
+              if (FULL || (ok[e >> 2] && k < p.I))
+                unsafeAtomicAdd(target + base[e >> 2] + (e & 3) * p.h.BN, acc[a][b][e] * p.scale);
             }
           }
+      };
+      if (image_mode) {
+        // Tiles of one workgroup overlap in hashed_weight: sum them in an LDS image of dHW
+        // first, then store the image as this workgroup's partial result.
+        if (p.h.bk_shift >= 5 && p.h.bn_shift >= 5) {
+          // Every 32x32 accumulator block lies inside one hashed tile, whose BK*BN addresses
+          // are all distinct.  LDS float atomics are slow, so instead the tiles of the window
+          // take turns: in round t only the blocks of tile t are added, with plain
+          // read-add-write, and a barrier separates the rounds.
+          int blk_tile[MI][MJ], blk_base[MI][MJ];
+#pragma unroll
+          for (int a = 0; a < MI; a++)
+#pragma unroll
+            for (int b = 0; b < MJ; b++) {
+              const int k0 = i0 + wave_i * WTI + a * 32, n0 = j0 + wave_j * WTJ + b * 32;
+              const int t = __builtin_amdgcn_readfirstlane(((k0 >> p.h.bk_shift) - w.tk0) * w.ntn +
+                                                           ((n0 >> p.h.bn_shift) - w.tn0));
+              blk_tile[a][b] = t;
+              blk_base[a][b] = sm.off[t] + ((k0 & (p.h.BK - 1)) + (lane >> 5) * 4) * p.h.BN +
+                               ((n0 + (lane & 31)) & (p.h.BN - 1));
+            }
+          for (int t = 0; t < w.count; t++) {
+            if (steps > 0) {
+#pragma unroll
+              for (int a = 0; a < MI; a++)
+#pragma unroll
+                for (int b = 0; b < MJ; b++) {
+                  if (blk_tile[a][b] == t) {
+                    const int k0 = i0 + wave_i * WTI + a * 32 + (lane >> 5) * 4;
+                    const bool col_ok = FULL || (j0 + wave_j * WTJ + b * 32 + (lane & 31) < p.J);
+                    float cur[16];
+#pragma unroll
+                    for (int e = 0; e < 16; e++)
+                      cur[e] = image[blk_base[a][b] + ((e >> 2) * 8 + (e & 3)) * p.h.BN];
+#pragma unroll
+                    for (int e = 0; e < 16; e++)
+                      if (FULL || (col_ok && k0 + (e >> 2) * 8 + (e & 3) < p.I))
+                        image[blk_base[a][b] + ((e >> 2) * 8 + (e & 3)) * p.h.BN] =
+                            cur[e] + acc[a][b][e] * p.scale;
+                  }
+                }
+            }
+            __syncthreads();
+          }
+        } else {
+          scatter(image);
+          __syncthreads();
         }
+        float* dst = p.scatter + ((size_t)blockIdx.y * gridDim.x + blockIdx.x) * (size_t)p.image_pitch;
+        for (int i = tid * 4; i < p.image_pitch; i += kThreads * 4)
+          *reinterpret_cast<float4*>(dst + i) = *reinterpret_cast<const float4*>(image + i);
+      } else {
+        scatter(p.scatter);
+      }
     } else {
       T* __restrict__ gC = static_cast<T*>(p.C);
 #pragma unroll
