@@ -48,6 +48,9 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-dense", action="store_true")
     ap.add_argument("--cpu-budget", type=float, default=15.0, help="seconds of CPU-path timing")
+    ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MiB",
+                    help="only run a plain device-to-device copy of this many MiB (five launches) and exit: "
+                         "the known traffic against which rocprofv3's FETCH_SIZE / WRITE_SIZE are scaled")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (no collectives, no sharding); run with --gpus 1")
@@ -60,6 +63,17 @@ def main():
     lib = _lib.load()   # raises if librzlinear.so is not built: there is no fallback
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+
+    if args.calibrate_copy > 0:
+        n = args.calibrate_copy * 1024 * 1024
+        src = torch.empty((n,), dtype=torch.uint8, device=dev).random_(0, 255)
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"calibrate_copy_bytes_read": n, "calibrate_copy_bytes_written": n, "launches": 5}))
+        return
 
     M, K, N, H, dflt = WORKLOADS[args.workload]
     dname = args.dtype or dflt

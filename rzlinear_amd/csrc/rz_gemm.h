@@ -19,6 +19,8 @@
 //       with R contiguous is transposed while it is written (pad 1), else copied (pad 4)
 #pragma once
 
+#include <type_traits>
+
 #include "rz_common.h"
 
 namespace rz {
@@ -389,32 +391,96 @@ struct GemmKernel {
         __syncthreads();
       }
     } else {
-      // two LDS stages, one barrier per step: while stage s&1 feeds the MFMAs, the registers
-      // loaded during the previous step go into the other stage and the loads of step s+2
-      // are issued.  The steady-state loop carries no conditions; the last two steps are peeled.
+      // Two LDS stages and a software pipeline with ONE barrier per R step.  While the MFMAs
+      // of step s run out of stage s&1, the same instruction stream carries, between them:
+      //   sub-step 0      the LDS writes of step s+1 (registers loaded during step s-1)
+      //   sub-step 1      the global loads of step s+2 and the hashing of step s+4
+      //   every sub-step  the LDS reads of the next sub-step's fragments
+      // The barrier sits before the last sub-step: by then every wavefront has issued (and
+      // waited for) its last reads of stage s&1 and has written stage (s+1)&1, so the last
+      // sub-step can already read the first fragments of step s+1, and the next step's writes
+      // into stage s&1 are safe.
+      constexpr int NKS = TR / KS;
+      static_assert(NKS >= 3, "pipeline needs at least three sub-steps per R step");
+      Frag fa[2][MI], fb[2][MJ];
+      auto frags = [&](int st, int ks, int buf) {
+#pragma unroll
+        for (int a = 0; a < MI; a++)
+          fa[buf][a] = lds_frag<A_LAYOUT, LA>(sm.a[st], wave_i * WTI + a * 32, ks, lane);
+#pragma unroll
+        for (int b = 0; b < MJ; b++)
+          fb[buf][b] = lds_frag<B_LAYOUT, LB>(sm.b[st], wave_j * WTJ + b * 32, ks, lane);
+      };
+      auto mfmas = [&](int buf) {
+#pragma unroll
+        for (int a = 0; a < MI; a++)
+#pragma unroll
+          for (int b = 0; b < MJ; b++) acc[a][b] = Mfma<T>::run(fa[buf][a], fb[buf][b], acc[a][b]);
+      };
+      constexpr int kReads = (k16 && A_LAYOUT == kRStrided ? 2 : 1) * MI +
+                             (k16 && B_LAYOUT == kRStrided ? 2 : 1) * MJ;
+      constexpr int kMfmas = MI * MJ;
+      constexpr int kPieces = LA::kPieces + LB::kPieces;
+      // one R step; the flags say which of the side jobs still exist near the end of the loop
+      auto step = [&](int s, auto do_commit, auto do_fetch, auto has_next) {
+        const int st = s & 1;
+        // (its few threads branch, which ends a scheduling region: keep it out of the MFMA stream)
+        if constexpr (decltype(do_fetch)::value) hash_step(s + 4);
+#pragma unroll
+        for (int ks = 0; ks < NKS; ks++) {
+          if (ks + 1 < NKS) {
+            frags(st, ks + 1, (ks + 1) & 1);
+          } else {
+            __syncthreads();
+            if constexpr (decltype(has_next)::value) frags(st ^ 1, 0, (ks + 1) & 1);
+          }
+          if (ks == 0) {
+            if constexpr (decltype(do_commit)::value) commit(st ^ 1);
+          }
+          if (ks == 1) {
+            if constexpr (decltype(do_fetch)::value) fetch(s + 2);
+          }
+          mfmas(ks & 1);
+          // scheduling hints: after each MFMA, its share of this sub-step's other work
+          if (ks + 1 < NKS) {
+#pragma unroll
+            for (int i = 0; i < kMfmas; i++) {
+              __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // 1 MFMA
+              if ((kReads * (i + 1)) / kMfmas - (kReads * i) / kMfmas == 1)
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // LDS reads
+              else if ((kReads * (i + 1)) / kMfmas - (kReads * i) / kMfmas == 2)
+                __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+              else if ((kReads * (i + 1)) / kMfmas - (kReads * i) / kMfmas == 3)
+                __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);
+              if (ks == 0 && decltype(do_commit)::value) {
+                if ((kPieces * (i + 1)) / kMfmas - (kPieces * i) / kMfmas == 1)
+                  __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);  // LDS writes
+                else if ((kPieces * (i + 1)) / kMfmas - (kPieces * i) / kMfmas == 2)
+                  __builtin_amdgcn_sched_group_barrier(0x200, 2, 0);
+              }
+              if (ks == 1 && decltype(do_fetch)::value) {
+                if ((kPieces * (i + 1)) / kMfmas - (kPieces * i) / kMfmas == 1)
+                  __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // global loads
+                else if ((kPieces * (i + 1)) / kMfmas - (kPieces * i) / kMfmas == 2)
+                  __builtin_amdgcn_sched_group_barrier(0x020, 2, 0);
+              }
+            }
+          }
+        }
+      };
       if (steps > 0) {
         commit(0);
         if (steps > 1) fetch(1);
         hash_step(3);
         __syncthreads();
+        frags(0, 0, 0);
         int s = 0;
-        for (; s + 2 < steps; s++) {
-          commit((s + 1) & 1);
-          fetch(s + 2);
-          hash_step(s + 4);
-          // keep the global loads ahead of the MFMAs: their latency must hide behind this
-          // step's matrix work, not be met at the next step's LDS writes
-          __builtin_amdgcn_sched_barrier(0);
-          compute(s & 1);
-          __syncthreads();
-        }
+        for (; s + 2 < steps; s++) step(s, std::true_type{}, std::true_type{}, std::true_type{});
         if (s + 1 < steps) {
-          commit((s + 1) & 1);
-          compute(s & 1);
-          __syncthreads();
+          step(s, std::true_type{}, std::false_type{}, std::true_type{});
           s++;
         }
-        compute(s & 1);
+        step(s, std::false_type{}, std::false_type{}, std::false_type{});
       }
     }
 
