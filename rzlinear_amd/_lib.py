@@ -10,7 +10,8 @@ import os
 import torch
 
 _PKG_DIR = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_PKG_DIR, "librzlinear.so")
+# RZLINEAR_LIB selects another build of the same library (variant builds for tuning)
+LIB_PATH = os.environ.get("RZLINEAR_LIB") or os.path.join(_PKG_DIR, "librzlinear.so")
 
 RZ_F32, RZ_BF16, RZ_F16 = 0, 1, 2
 _DTYPES = {torch.float32: RZ_F32, torch.bfloat16: RZ_BF16, torch.float16: RZ_F16}

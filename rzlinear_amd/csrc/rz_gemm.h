@@ -126,6 +126,10 @@ struct GemmKernel {
     static constexpr int kCpr = kSrcCols / VEC;                 // 16-byte pieces per source row
     static constexpr int kPieces = kSrcRows * kCpr / kThreads;  // pieces per thread
     static_assert(kSrcRows * kCpr % kThreads == 0, "tile must split evenly over the threads");
+    // a thread's pieces are kPieces consecutive source rows (else: interleaved over the tile)
+    static constexpr bool kBlocked = (k16 || LAYOUT == kRStrided) && (kThreads % kCpr == 0) &&
+                                     (kPieces == 1 || kPieces == 2 || kPieces == 4 || kPieces == 8 ||
+                                      kPieces == 16);
   };
   typedef Lds<A_LAYOUT, TI> LA;
   typedef Lds<B_LAYOUT, TJ> LB;
@@ -276,12 +280,28 @@ struct GemmKernel {
         }
       }
     };
+    // Which 16-byte pieces of a source tile a thread moves.  A thread owns kPieces consecutive
+    // rows at one column position: the rows are a constant pitch apart (cheap addresses), and,
+    // being at most 16 rows aligned to their count, they lie in ONE hashed tile, so a hashed
+    // operand needs a single table lookup per thread and step.  (fp32 tiles whose source has R
+    // contiguous are transposed on their way into LDS; they keep the interleaved mapping, which
+    // spreads that scatter over the banks.)
+    auto piece_row = [&](auto L, int q) -> int {
+      typedef decltype(L) LL;
+      if constexpr (LL::kBlocked) return (tid / LL::kCpr) * LL::kPieces + q;
+      else return (tid + q * kThreads) / LL::kCpr;
+    };
+    auto piece_cc = [&](auto L, int q) -> int {
+      typedef decltype(L) LL;
+      if constexpr (LL::kBlocked) return tid % LL::kCpr;
+      else return (tid + q * kThreads) % LL::kCpr;
+    };
     // global -> registers for R step `step`
     auto fetch = [&](int step) {
       const int r0 = r_begin + step * TR;
 #pragma unroll
       for (int q = 0; q < LA::kPieces; q++) {
-        const int c = tid + q * kThreads, srow = c / LA::kCpr, scol = (c % LA::kCpr) * VEC;
+        const int srow = piece_row(LA{}, q), scol = piece_cc(LA{}, q) * VEC;
         if constexpr (A_LAYOUT == kRContig)
           ra[q] = load_plain<T, FULL>(gA, p.lda, i0 + srow, p.I, r0 + scol, r_end);
         else
@@ -290,24 +310,34 @@ struct GemmKernel {
       if constexpr (OP == kWeightGrad) {
 #pragma unroll
         for (int q = 0; q < LB::kPieces; q++) {
-          const int c = tid + q * kThreads, srow = c / LB::kCpr, scol = (c % LB::kCpr) * VEC;
+          const int srow = piece_row(LB{}, q), scol = piece_cc(LB{}, q) * VEC;
           rb[q] = load_plain<T, FULL>(gB, p.ldb, r0 + srow, r_end, j0 + scol, p.J);
         }
       } else {
-        // all table lookups first (one LDS round trip), then the loads
         const OffWindow w = window(step);
         const int* tab = sm.off + (step & (kOffSlots - 1)) * kOffWindow;
         int idx[LB::kPieces];
-#pragma unroll
-        for (int q = 0; q < LB::kPieces; q++) {
-          const int c = tid + q * kThreads, srow = c / LB::kCpr, scol = (c % LB::kCpr) * VEC;
+        if constexpr (LB::kBlocked) {
+          // one lookup: the thread's rows are consecutive rows k of one hashed tile
+          const int srow = piece_row(LB{}, 0), scol = piece_cc(LB{}, 0) * VEC;
           const int k = (OP == kForward) ? r0 + srow : j0 + srow;
           const int n = (OP == kForward) ? j0 + scol : r0 + scol;
-          idx[q] = hashed_index(p.h, tab, w, k, n);
+          const int idx0 = hashed_index(p.h, tab, w, k, n);
+#pragma unroll
+          for (int q = 0; q < LB::kPieces; q++) idx[q] = idx0 + q * p.h.BN;
+        } else {
+          // all table lookups first (one LDS round trip), then the loads
+#pragma unroll
+          for (int q = 0; q < LB::kPieces; q++) {
+            const int srow = piece_row(LB{}, q), scol = piece_cc(LB{}, q) * VEC;
+            const int k = (OP == kForward) ? r0 + srow : j0 + srow;
+            const int n = (OP == kForward) ? j0 + scol : r0 + scol;
+            idx[q] = hashed_index(p.h, tab, w, k, n);
+          }
         }
 #pragma unroll
         for (int q = 0; q < LB::kPieces; q++) {
-          const int c = tid + q * kThreads, srow = c / LB::kCpr, scol = (c % LB::kCpr) * VEC;
+          const int srow = piece_row(LB{}, q), scol = piece_cc(LB{}, q) * VEC;
           if constexpr (OP == kForward)
             rb[q] = load_hashed(gHW, idx[q], r0 + srow, r_end, j0 + scol, p.J);
           else
@@ -318,15 +348,11 @@ struct GemmKernel {
     // registers -> LDS stage `st`
     auto commit = [&](int st) {
 #pragma unroll
-      for (int q = 0; q < LA::kPieces; q++) {
-        const int c = tid + q * kThreads;
-        lds_put<A_LAYOUT, LA>(sm.a[st], c / LA::kCpr, c % LA::kCpr, ra[q]);
-      }
+      for (int q = 0; q < LA::kPieces; q++)
+        lds_put<A_LAYOUT, LA>(sm.a[st], piece_row(LA{}, q), piece_cc(LA{}, q), ra[q]);
 #pragma unroll
-      for (int q = 0; q < LB::kPieces; q++) {
-        const int c = tid + q * kThreads;
-        lds_put<B_LAYOUT, LB>(sm.b[st], c / LB::kCpr, c % LB::kCpr, rb[q]);
-      }
+      for (int q = 0; q < LB::kPieces; q++)
+        lds_put<B_LAYOUT, LB>(sm.b[st], piece_row(LB{}, q), piece_cc(LB{}, q), rb[q]);
     };
     // MFMAs of one R step out of LDS stage `st`; fragments are read one sub-step ahead
     auto compute = [&](int st) {
@@ -417,10 +443,6 @@ struct GemmKernel {
 #pragma unroll
           for (int b = 0; b < MJ; b++) acc[a][b] = Mfma<T>::run(fa[buf][a], fb[buf][b], acc[a][b]);
       };
-      constexpr int kReads = (k16 && A_LAYOUT == kRStrided ? 2 : 1) * MI +
-                             (k16 && B_LAYOUT == kRStrided ? 2 : 1) * MJ;
-      constexpr int kMfmas = MI * MJ;
-      constexpr int kPieces = LA::kPieces + LB::kPieces;
       // one R step; the flags say which of the side jobs still exist near the end of the loop
       auto step = [&](int s, auto do_commit, auto do_fetch, auto has_next) {
         const int st = s & 1;
@@ -441,31 +463,6 @@ struct GemmKernel {
             if constexpr (decltype(do_fetch)::value) fetch(s + 2);
           }
           mfmas(ks & 1);
-          // scheduling hints: after each MFMA, its share of this sub-step's other work
-          if (ks + 1 < NKS) {
-#pragma unroll
-            for (int i = 0; i < kMfmas; i++) {
-              __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // 1 MFMA
-              if ((kReads * (i + 1)) / kMfmas - (kReads * i) / kMfmas == 1)
-                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // LDS reads
-              else if ((kReads * (i + 1)) / kMfmas - (kReads * i) / kMfmas == 2)
-                __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-              else if ((kReads * (i + 1)) / kMfmas - (kReads * i) / kMfmas == 3)
-                __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);
-              if (ks == 0 && decltype(do_commit)::value) {
-                if ((kPieces * (i + 1)) / kMfmas - (kPieces * i) / kMfmas == 1)
-                  __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);  // LDS writes
-                else if ((kPieces * (i + 1)) / kMfmas - (kPieces * i) / kMfmas == 2)
-                  __builtin_amdgcn_sched_group_barrier(0x200, 2, 0);
-              }
-              if (ks == 1 && decltype(do_fetch)::value) {
-                if ((kPieces * (i + 1)) / kMfmas - (kPieces * i) / kMfmas == 1)
-                  __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // global loads
-                else if ((kPieces * (i + 1)) / kMfmas - (kPieces * i) / kMfmas == 2)
-                  __builtin_amdgcn_sched_group_barrier(0x020, 2, 0);
-              }
-            }
-          }
         }
       };
       if (steps > 0) {
