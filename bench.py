@@ -36,6 +36,16 @@ WORKLOADS = {
 }
 # dense MFMA peaks of MI355X, TFLOP/s
 PEAK = {"bf16": 2500.0, "fp16": 2500.0, "fp32": 157.3}
+# HBM bytes per launch, measured once with rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE (KiB per
+# dispatch) and scaled by what the same counters read for a plain 256 MiB copy (FETCH_SIZE x2.0,
+# WRITE_SIZE x1.0); the rocprof summary with the raw readings is committed with the profiles.
+TRAFFIC_BYTES = {
+    ("square4096", "bf16"): {
+        "forward": int((16628.8 * 2.0 + 32774.7) * 1024),       # algorithmic: 64.03 MiB
+        "input_grad": int((16624.4 * 2.0 + 32913.3) * 1024),
+        "weight_grad": int((98420.5 * 2.0 + 16784.5) * 1024),   # X, dY re-read by 3 XCD groups; + partial images
+    },
+}
 
 
 def main():
@@ -140,7 +150,7 @@ def main():
         "peak": peak,
         "unit": "TFLOP/s",
         "frac": round(leg_tflops[slowest] / peak, 4),
-        "traffic": None,
+        "traffic": TRAFFIC_BYTES.get((args.workload, dname), {}).get(slowest),
         "per_kernel_tflops": {k: round(v, 2) for k, v in leg_tflops.items()},
         "per_kernel_ms": {k: round(v, 4) for k, v in leg_ms.items()},
     }
