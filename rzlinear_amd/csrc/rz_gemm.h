@@ -444,7 +444,12 @@ struct GemmKernel {
           for (int b = 0; b < MJ; b++) acc[a][b] = Mfma<T>::run(fa[buf][a], fb[buf][b], acc[a][b]);
       };
       // one R step; the flags say which of the side jobs still exist near the end of the loop
-      auto step = [&](int s, auto do_commit, auto do_fetch, auto has_next) {
+      // `late` staggers the side jobs of the two wavefronts that share a SIMD: one does them
+      // during the first sub-steps, the other during the last ones, so that while one issues
+      // LDS writes and global loads the other keeps the MFMA pipe fed.
+      auto step = [&](int s, auto late, auto do_commit, auto do_fetch, auto has_next) {
+        constexpr int kCommitAt = decltype(late)::value ? NKS - 2 : 0;
+        constexpr int kFetchAt = decltype(late)::value ? NKS - 1 : 1;
         const int st = s & 1;
         // (its few threads branch, which ends a scheduling region: keep it out of the MFMA stream)
         if constexpr (decltype(do_fetch)::value) hash_step(s + 4);
@@ -456,14 +461,23 @@ struct GemmKernel {
             __syncthreads();
             if constexpr (decltype(has_next)::value) frags(st ^ 1, 0, (ks + 1) & 1);
           }
-          if (ks == 0) {
+          if (ks == kCommitAt) {
             if constexpr (decltype(do_commit)::value) commit(st ^ 1);
           }
-          if (ks == 1) {
+          if (ks == kFetchAt) {
             if constexpr (decltype(do_fetch)::value) fetch(s + 2);
           }
           mfmas(ks & 1);
         }
+      };
+      auto loop = [&](auto late) {
+        int s = 0;
+        for (; s + 2 < steps; s++) step(s, late, std::true_type{}, std::true_type{}, std::true_type{});
+        if (s + 1 < steps) {
+          step(s, late, std::true_type{}, std::false_type{}, std::true_type{});
+          s++;
+        }
+        step(s, late, std::false_type{}, std::false_type{}, std::false_type{});
       };
       if (steps > 0) {
         commit(0);
@@ -471,13 +485,9 @@ struct GemmKernel {
         hash_step(3);
         __syncthreads();
         frags(0, 0, 0);
-        int s = 0;
-        for (; s + 2 < steps; s++) step(s, std::true_type{}, std::true_type{}, std::true_type{});
-        if (s + 1 < steps) {
-          step(s, std::true_type{}, std::false_type{}, std::true_type{});
-          s++;
-        }
-        step(s, std::false_type{}, std::false_type{}, std::false_type{});
+        // wavefronts w and w + 4 of a workgroup share a SIMD
+        if (kThreads == 512 && wave >= 4) loop(std::true_type{});
+        else loop(std::false_type{});
       }
     }
 
@@ -491,9 +501,12 @@ struct GemmKernel {
         const float4 z = {0.f, 0.f, 0.f, 0.f};
         for (int i = tid * 4; i < p.image_pitch; i += kThreads * 4) *reinterpret_cast<float4*>(image + i) = z;
       }
+      // offset table of this C tile's hashed tiles: behind the image (which may be larger
+      // than the operand stages), else in its usual place
+      int* etab = image_mode ? reinterpret_cast<int*>(image + p.image_pitch) : sm.off;
       const OffWindow w = off_window(p.h, i0, TI, j0, TJ);
       for (int t = tid; t < w.count; t += kThreads)
-        sm.off[t] = (int)tile_offset(p.h, (uint32_t)(w.tk0 + t / w.ntn), (uint32_t)(w.tn0 + t % w.ntn));
+        etab[t] = (int)tile_offset(p.h, (uint32_t)(w.tk0 + t / w.ntn), (uint32_t)(w.tn0 + t % w.ntn));
       __syncthreads();
       // Scatter-add of the accumulators.  The four rows e&3 of a row group (e>>2) are adjacent
       // rows of one hashed tile (tiles are at least 16 rows), so one table lookup per row
@@ -512,7 +525,7 @@ struct GemmKernel {
             for (int g = 0; g < 4; g++) {
               const int k = i0 + wave_i * WTI + a * 32 + g * 8 + (lane >> 5) * 4;
               ok[g] = FULL || (k < p.I && n < p.J);
-              base[g] = sm.off[((k >> p.h.bk_shift) - w.tk0) * w.ntn + ((n >> p.h.bn_shift) - w.tn0)] +
+              base[g] = etab[((k >> p.h.bk_shift) - w.tk0) * w.ntn + ((n >> p.h.bn_shift) - w.tn0)] +
                         (k & (p.h.BK - 1)) * p.h.BN + (n & (p.h.BN - 1));
             }
 #pragma unroll
@@ -540,7 +553,7 @@ struct GemmKernel {
               const int t = __builtin_amdgcn_readfirstlane(((k0 >> p.h.bk_shift) - w.tk0) * w.ntn +
                                                            ((n0 >> p.h.bn_shift) - w.tn0));
               blk_tile[a][b] = t;
-              blk_base[a][b] = sm.off[t] + ((k0 & (p.h.BK - 1)) + (lane >> 5) * 4) * p.h.BN +
+              blk_base[a][b] = etab[t] + ((k0 & (p.h.BK - 1)) + (lane >> 5) * 4) * p.h.BN +
                                ((n0 + (lane & 31)) & (p.h.BN - 1));
             }
           for (int t = 0; t < w.count; t++) {

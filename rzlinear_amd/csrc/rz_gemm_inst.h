@@ -20,13 +20,18 @@ static hipError_t launch_one(GemmParams p, const WeightGradPlan* plan, hipStream
     splits = plan->splits;
     p.r_chunk = plan->r_chunk;
     p.image_pitch = plan->image_pitch;
-    if ((size_t)p.image_pitch * sizeof(float) > K::kImageBytes) return hipErrorInvalidValue;
+    if ((size_t)p.image_pitch * sizeof(float) > kMaxImageBytes) return hipErrorInvalidValue;
   } else {
     p.r_chunk = r_steps * K::TR;
   }
   auto kernel = rz_gemm_kernel<T, OP, TI, TJ, WI, WJ, NSTAGE, FULL>;
-  constexpr size_t smem = sizeof(typename K::Smem);
-  static_assert(smem <= 160 * 1024, "tile does not fit the 160 KB LDS of a compute unit");
+  size_t smem = sizeof(typename K::Smem);
+  static_assert(sizeof(typename K::Smem) <= 160 * 1024, "tile does not fit the 160 KB LDS of a compute unit");
+  if (OP == kWeightGrad && p.image_pitch > 0) {
+    // the dHW image and the scatter's offset table behind it may need more than the stages
+    const size_t need = (size_t)p.image_pitch * sizeof(float) + K::kOffEntries * sizeof(int);
+    if (need > smem) smem = need;
+  }
   if (smem > 64 * 1024) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
@@ -38,31 +43,41 @@ static hipError_t launch_one(GemmParams p, const WeightGradPlan* plan, hipStream
 }
 
 // FULL kernels carry no bounds checks: every tile and every R step must be complete.
-template <typename T, int OP, int TILE, int NSTAGE>
+template <typename T, int OP, int TILE, int WI, int WJ, int NSTAGE>
 static hipError_t launch_tile(GemmParams p, const WeightGradPlan* plan, hipStream_t stream) {
   constexpr int TR = 128 / ElemTraits<T>::kBytes;
-  // 256 x 256: eight wavefronts (two per SIMD) of 128 x 64; 128 x 128: four of 64 x 64
-  constexpr int WJ = (TILE == 256) ? 4 : 2;
   const bool full = (p.I % TILE == 0) && (p.J % TILE == 0) && (p.R % TR == 0);
-  if (full) return launch_one<T, OP, TILE, TILE, 2, WJ, NSTAGE, true>(p, plan, stream);
-  return launch_one<T, OP, TILE, TILE, 2, WJ, NSTAGE, false>(p, plan, stream);
+  if (full) return launch_one<T, OP, TILE, TILE, WI, WJ, NSTAGE, true>(p, plan, stream);
+  return launch_one<T, OP, TILE, TILE, WI, WJ, NSTAGE, false>(p, plan, stream);
 }
 
+template <typename T, int TILE, int WI, int WJ, int NSTAGE>
+static hipError_t launch_op(int op, GemmParams p, const WeightGradPlan* plan, hipStream_t stream) {
+  switch (op) {
+    case kForward: return launch_tile<T, kForward, TILE, WI, WJ, NSTAGE>(p, plan, stream);
+    case kInputGrad: return launch_tile<T, kInputGrad, TILE, WI, WJ, NSTAGE>(p, plan, stream);
+    case kWeightGrad: return launch_tile<T, kWeightGrad, TILE, WI, WJ, NSTAGE>(p, plan, stream);
+    default: return hipErrorInvalidValue;
+  }
+}
+
+// Tile shapes (all two LDS stages, software pipelined unless noted):
+//   256: 256 x 256, eight wavefronts of 128 x 64, one workgroup per compute unit
+//   128: 128 x 128, four wavefronts of 64 x 64, up to two workgroups per compute unit
+//    64:  64 x  64, four wavefronts of 32 x 32, for problems with few tiles
+// RZLINEAR_STAGES=1 selects a single-stage 128 x 128 form that leans on several workgroups
+// per compute unit instead of a pipeline (tuning aid).
 template <typename T>
 static hipError_t launch_gemm_t(int op, GemmParams p, const WeightGradPlan* plan, hipStream_t stream) {
   const int tile = (op == kWeightGrad && plan != nullptr) ? plan->tile : pick_tile(p.I, p.J);
-  if (tile == 256) {
-    switch (op) {
-      case kForward: return launch_tile<T, kForward, 256, 2>(p, plan, stream);
-      case kInputGrad: return launch_tile<T, kInputGrad, 256, 2>(p, plan, stream);
-      case kWeightGrad: return launch_tile<T, kWeightGrad, 256, 2>(p, plan, stream);
-      default: return hipErrorInvalidValue;
-    }
-  }
-  switch (op) {
-    case kForward: return launch_tile<T, kForward, 128, 1>(p, plan, stream);
-    case kInputGrad: return launch_tile<T, kInputGrad, 128, 1>(p, plan, stream);
-    case kWeightGrad: return launch_tile<T, kWeightGrad, 128, 1>(p, plan, stream);
+  const char* stages_env = getenv("RZLINEAR_STAGES");
+  const bool one_stage = stages_env != nullptr && atoi(stages_env) == 1;
+  switch (tile) {
+    case 256: return launch_op<T, 256, 2, 4, 2>(op, p, plan, stream);
+    case 64: return launch_op<T, 64, 2, 2, 2>(op, p, plan, stream);
+    case 128:
+      if (one_stage) return launch_op<T, 128, 2, 2, 1>(op, p, plan, stream);
+      return launch_op<T, 128, 2, 2, 2>(op, p, plan, stream);
     default: return hipErrorInvalidValue;
   }
 }

@@ -11,17 +11,23 @@ static constexpr int kComputeUnits = 256;
 // Number of workgroups of the small tile that fills the compute units a few times over.
 static constexpr int kTargetWorkgroups = 1024;
 
-// Large tile (256 x 256, one workgroup of eight wavefronts per compute unit, two LDS stages)
-// when it still yields enough workgroups to occupy the chip; else the 128 x 128 tile with
-// several workgroups per compute unit.  RZLINEAR_TILE=128|256 forces one of them (tuning aid).
+// C-tile edge for a contraction with an I x J result: the largest of 256, 128, 64 that still
+// yields about one workgroup per compute unit; RZLINEAR_TILE=64|128|256 forces one (tuning aid).
+static inline int forced_tile() {
+  const char* e = getenv("RZLINEAR_TILE");   // read per call, so a test can switch it
+  const int v = e ? atoi(e) : 0;
+  return (v == 64 || v == 128 || v == 256) ? v : 0;
+}
+
+static inline long long tile_count(int I, int J, int t) {
+  return (long long)((I + t - 1) / t) * ((J + t - 1) / t);
+}
+
 static inline int pick_tile(int I, int J) {
-  static const int forced = []() {
-    const char* e = getenv("RZLINEAR_TILE");
-    return e ? atoi(e) : 0;
-  }();
-  if (forced == 128 || forced == 256) return forced;
-  const long long big = (long long)((I + 255) / 256) * ((J + 255) / 256);
-  return big >= kComputeUnits / 2 ? 256 : 128;
+  if (forced_tile()) return forced_tile();
+  if (tile_count(I, J, 256) >= kComputeUnits / 2) return 256;
+  if (tile_count(I, J, 128) >= kComputeUnits * 3 / 4) return 128;
+  return 64;
 }
 
 // How the weight-grad contraction C[K,N] = X^T.dY over M is cut into workgroups, and how the
@@ -37,33 +43,44 @@ struct WeightGradPlan {
   size_t workspace_bytes;
 };
 
-// LDS bytes that the weight-grad kernel's operand stages occupy (and its dHW image may reuse).
-static inline size_t weight_grad_stage_bytes(int tile, int elem_bytes) {
-  const int TR = 128 / elem_bytes;
-  const size_t pitch = (elem_bytes == 2) ? (size_t)tile + 32 : (size_t)tile + 4;
-  const size_t one = ((pitch * TR + 7) / 8) * 8 * elem_bytes;   // one operand, one stage
-  return one * 2 * (tile == 256 ? 2 : 1);
+// LDS bytes of a compute unit that an fp32 image of dHW may take (the rest holds the small
+// offset table of the scatter); the image reuses the operand stages, which are dead by then.
+static constexpr size_t kMaxImageBytes = 147456;
+
+static inline long long tile_cover(int K, int N, int t) {
+  return (long long)((K + t - 1) / t) * ((N + t - 1) / t) * t * t;
 }
 
 static inline WeightGradPlan plan_weight_grad(int M, int K, int N, int H, int elem_bytes) {
   WeightGradPlan pl;
-  pl.tile = pick_tile(K, N);
   const int TR = 128 / elem_bytes;
+  const int pitch = (H + 3) & ~3;
+  const bool no_image = getenv("RZLINEAR_NO_LDS_IMAGE") != nullptr;   // tuning aid
+  const bool image = !no_image && (size_t)pitch * sizeof(float) <= kMaxImageBytes;
+  if (forced_tile()) {
+    pl.tile = forced_tile();
+  } else if (image) {
+    // with the LDS image the M loop can be cut freely (a slice costs one partial image), so
+    // the pipelined 256 tile is used unless it would mostly compute padding
+    pl.tile = 64;
+    if (tile_cover(K, N, 128) * 10 <= tile_cover(K, N, 64) * 13) pl.tile = 128;
+    if (tile_cover(K, N, 256) * 10 <= tile_cover(K, N, pl.tile) * 13) pl.tile = 256;
+  } else {
+    pl.tile = pick_tile(K, N);
+  }
   const long long tiles = (long long)((K + pl.tile - 1) / pl.tile) * ((N + pl.tile - 1) / pl.tile);
   const int r_steps = (M + TR - 1) / TR;
   // split the reduction over M when there are too few W tiles to fill the chip
-  const long long target = (pl.tile >= 256) ? kComputeUnits : kTargetWorkgroups;
+  const long long target = (pl.tile >= 256) ? kComputeUnits : (pl.tile == 128 ? 2 * kComputeUnits : kTargetWorkgroups);
   long long want = (target + tiles - 1) / tiles;
+  if (!image && want > 8) want = 8;   // every slice repeats the K*N global atomics
   if (want > r_steps) want = r_steps;
   if (want < 1) want = 1;
   const int steps_per = (int)((r_steps + want - 1) / want);
   pl.splits = (r_steps + steps_per - 1) / steps_per;
   pl.r_chunk = steps_per * TR;
   pl.workgroups = tiles * pl.splits;
-  const int pitch = (H + 3) & ~3;
-  static const bool no_image = getenv("RZLINEAR_NO_LDS_IMAGE") != nullptr;   // tuning aid
-  const bool fits = (size_t)pitch * sizeof(float) <= weight_grad_stage_bytes(pl.tile, elem_bytes);
-  pl.image_pitch = (fits && !no_image) ? pitch : 0;
+  pl.image_pitch = image ? pitch : 0;
   size_t ws = 0;
   if (pl.image_pitch > 0) ws = (size_t)pl.workgroups * pl.image_pitch * sizeof(float);
   else if (elem_bytes == 2) ws = (size_t)H * sizeof(float);   // fp32 image for the atomics

@@ -116,3 +116,35 @@ def test_materialize_both_hashes(oracle, dtype):
     assert np.array_equal(w1.double().cpu().numpy(), oracle.materialize(hw64, K, N, BK, BN, R, 1))
     w2 = rz_linear_weight_tl(hw, 1000, 900, H, *rargs(R), BLOCK_SIZE_K=BK, BLOCK_SIZE_N=BN)
     assert np.array_equal(w2.double().cpu().numpy(), oracle.materialize(hw64, 1000, 900, BK, BN, R, 2))
+
+
+TILE_CASES = [
+    # (M, K, N, H, BK, BN): complete tiles for every C-tile size, ragged, and both scatter paths
+    (512, 512, 512, 9000, 64, 64),
+    (300, 200, 330, 9000, 32, 64),
+    (256, 256, 512, 70000, 64, 64),      # H too large for the LDS image: global atomics
+    (130, 70, 90, 2000, 16, 16),         # 16-wide tiles: LDS atomics inside the image
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=lambda d: str(d).split(".")[-1])
+@pytest.mark.parametrize("env", [{"RZLINEAR_TILE": "64"}, {"RZLINEAR_TILE": "128"}, {"RZLINEAR_TILE": "256"},
+                                 {"RZLINEAR_TILE": "128", "RZLINEAR_STAGES": "1"},
+                                 {"RZLINEAR_TILE": "256", "RZLINEAR_NO_LDS_IMAGE": "1"}],
+                         ids=lambda e: "-".join("%s=%s" % (k.replace("RZLINEAR_", ""), v) for k, v in e.items()))
+@pytest.mark.parametrize("shape", TILE_CASES, ids=lambda s: "x".join(map(str, s)))
+def test_every_tile_shape_and_scatter_mode(oracle, monkeypatch, shape, env, dtype):
+    """The library picks its C tile and scatter path from the problem size; force each one."""
+    from rzlinear_amd.impl.RzLinearBackward import rz_linear_backward_tl
+    from rzlinear_amd.impl.RzLinearForward import rz_linear_forward_tl
+    for k, v in env.items():
+        monkeypatch.setenv(k, v)
+    M, K, N, H, BK, BN = shape
+    _say("tiles", shape, env, dtype)
+    (x, hw, dy), (x64, hw64, dy64) = make_inputs(M, K, N, H, dtype, seed=4)
+    y = rz_linear_forward_tl(x, hw, 1.0, M, K, N, H, *rargs(R1024), BLOCK_SIZE_K=BK, BLOCK_SIZE_N=BN)
+    dx, dhw = rz_linear_backward_tl(x, hw, dy, 1.0, M, K, N, H, *rargs(R1024), BLOCK_SIZE_K=BK, BLOCK_SIZE_N=BN)
+    torch.cuda.synchronize()
+    assert rel_err(y.float().cpu().numpy(), oracle.forward(x64, hw64, N, BK, BN, R1024)) <= TOL[dtype]
+    assert rel_err(dx.float().cpu().numpy(), oracle.input_grad(dy64, hw64, K, BK, BN, R1024)) <= TOL[dtype]
+    assert rel_err(dhw.float().cpu().numpy(), oracle.weight_grad(x64, dy64, H, BK, BN, R1024)) <= TOL[dtype]
