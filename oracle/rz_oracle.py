@@ -12,9 +12,11 @@ module; the product package never does.  Two independent restatements live here:
   * ``c_*`` functions: ctypes calls into oracle/librz_oracle.so (rz_oracle.c), which follows
     the loop structure of the device kernels instead.
 
-Parity status: no golden vectors for the two-level hash exist in the reference, so these
-functions are pinned by the known-answer and invariant tests in tests/test_oracle.py, which
-also check the two restatements against each other.
+Parity status: pinned.  The reference holds no golden vectors for the two-level hash, so they
+were produced once by running its own Triton kernels under Triton's CPU interpreter
+(tests/golden/make_reference_vectors.py -> tests/golden/reference_vectors.npz); both
+restatements agree with them to fp32 rounding, and tests/test_oracle.py adds known-answer and
+invariant tests and checks the two restatements against each other.
 """
 import ctypes
 import os

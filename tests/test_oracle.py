@@ -247,3 +247,25 @@ def test_linearity_and_adjointness(oracle):
     s = (Y * dY).sum()
     np.testing.assert_allclose((X * dX).sum(), s, rtol=1e-11)
     np.testing.assert_allclose((hw * dHW).sum(), s, rtol=1e-11)
+
+
+# ------------------------------------------------------------------ vectors made by the reference itself
+def test_oracle_matches_vectors_produced_by_the_reference_kernels(oracle):
+    """tests/golden/reference_vectors.npz holds inputs and outputs of the reference's own Triton
+    kernels (run under Triton's CPU interpreter by tests/golden/make_reference_vectors.py).  This
+    is what pins the transcription of the two-level hash, the masks and the scale."""
+    d = np.load(os.path.join(GOLDEN, "reference_vectors.npz"))
+    R = d["R"].tolist()
+    assert R == R1024
+    for name in "abc":
+        M, K, N, H, BK, BN = [int(v) for v in d[name + "_shape"]]
+        f = float(d[name + "_f"])
+        x, hw, dy = d[name + "_x"], d[name + "_hw"], d[name + "_dy"]
+        for fwd, ig, wg in ((oracle.forward, oracle.input_grad, oracle.weight_grad),
+                            (oracle.c_forward, oracle.c_input_grad, oracle.c_weight_grad)):
+            for ref, got in ((d[name + "_y"], fwd(x, hw, N, BK, BN, R, f)),
+                             (d[name + "_dx"], ig(dy, hw, K, BK, BN, R, f)),
+                             (d[name + "_dhw"], wg(x, dy, H, BK, BN, R, f))):
+                assert ref.shape == got.shape
+                # the reference accumulates in fp32: allow its rounding, nothing more
+                assert np.abs(ref - got).max() <= 2e-6 * np.abs(got).max()
