@@ -449,7 +449,7 @@ struct GemmKernel {
       // LDS writes and global loads the other keeps the MFMA pipe fed.
       auto step = [&](int s, auto late, auto do_commit, auto do_fetch, auto has_next) {
         constexpr int kCommitAt = decltype(late)::value ? NKS - 2 : 0;
-        constexpr int kFetchAt = decltype(late)::value ? NKS - 1 : 1;
+        constexpr int kFetchAt = kCommitAt;   // right behind the LDS writes that free the registers
         const int st = s & 1;
         // (its few threads branch, which ends a scheduling region: keep it out of the MFMA stream)
         if constexpr (decltype(do_fetch)::value) hash_step(s + 4);
