@@ -84,6 +84,16 @@ int rz_forward(const void* X, const void* HW, void* Y, int M, int K, int N, int 
                void* stream);
 
 /*
+ * Forward with the layer's bias fused into the store: Y = (X . W) * init_factor + bias[N]
+ * (bias of element type `dtype`, may be NULL = rz_forward).  The sum is formed in fp32 and
+ * rounded once.  Replaces the launcher above plus the separate `x + self._bias` of the module,
+ * python/rz_linear/RzLinear.py:93-94.
+ */
+int rz_forward_bias(const void* X, const void* HW, const void* bias, void* Y, int M, int K, int N,
+                    int H, int BK, int BN, const int32_t R[8], float init_factor, int64_t ldx,
+                    int64_t ldy, int dtype, void* stream);
+
+/*
  * Input gradient: dX[M,K] = (dY[M,N] . W^T) * init_factor.
  * Replaces rz_linear_backward_input_grad_tl                           impl/RzLinearBackward.py:374-449
  * (kernel rz_linear_backward_input_grad_core                          impl/RzLinearBackward.py:642-727).

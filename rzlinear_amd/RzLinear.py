@@ -91,11 +91,11 @@ class RzLinear(torch.nn.Module):
         if (dim_gt_2):
             shape = x.shape
             x = x.reshape(-1, shape[-1]).contiguous()
+        # the bias is added inside the forward kernel's store (one rounding, no extra pass)
+        bias = self._bias if isinstance(self._bias, torch.Tensor) else None
         x = RzLinearFunction.apply(
             x, self._hashed_weight, self._random_numbers, self._output_dim, self._chunk_size,
-            self._init_factor, self._block_size_k, self._block_size_n)
-        if isinstance(self._bias, torch.Tensor):
-            x = x + self._bias
+            self._init_factor, self._block_size_k, self._block_size_n, bias)
         if (dim_gt_2):
             x = x.view(*shape[:-1], x.shape[-1])
         return x

@@ -1,7 +1,7 @@
 """autograd.Function of the compressed linear layer (host side of the drop-in boundary)."""
 import torch
 
-from .impl.RzLinearForward import rz_linear_forward_tl
+from .impl.RzLinearForward import rz_linear_forward_bias_tl
 from .impl.RzLinearBackward import (rz_linear_backward_input_grad_tl,
                                     rz_linear_backward_weight_grad_tl)
 
@@ -21,7 +21,7 @@ class RzLinearFunction(torch.autograd.Function):
     @staticmethod
     def forward(ctx, input: torch.Tensor, hashed_weight: torch.Tensor,
                 random_numbers: torch.Tensor, output_dim, chunk_size, init_factor,
-                block_size_k=None, block_size_n=None) -> torch.Tensor:
+                block_size_k=None, block_size_n=None, bias=None) -> torch.Tensor:
         '''
             Same six leading arguments and result as the reference
             (python/rz_linear/RzLinearFunction.py:13-43).
@@ -34,6 +34,7 @@ class RzLinearFunction(torch.autograd.Function):
                 chunk_size (int): carried, unused (as in the reference)
                 init_factor (float): scale applied to every result
                 block_size_k, block_size_n (int, optional): hashed tile; default controls[...]
+                bias (Tensor, optional): (output_dim), added inside the kernel's store
 
             Returns:
                 output (Tensor): (M, output_dim)
@@ -43,17 +44,18 @@ class RzLinearFunction(torch.autograd.Function):
         BK = int(block_size_k if block_size_k is not None else controls['block_size_k'])
         BN = int(block_size_n if block_size_n is not None else controls['block_size_n'])
         M, K, N, H = input.shape[0], input.shape[1], output_dim, hashed_weight.shape[0]
-        output = rz_linear_forward_tl(input, hashed_weight.data, init_factor, M, K, N, H,
-                                      R[7], R[6], R[5], R[4], R[3], R[2], R[1], R[0],
-                                      allow_tf32=controls['triton_allow_tf32'],
-                                      allow_autotune=controls['triton_allow_autotune'],
-                                      BLOCK_SIZE_K=BK, BLOCK_SIZE_N=BN)
+        output = rz_linear_forward_bias_tl(input, hashed_weight.data, None if bias is None else bias.data,
+                                           init_factor, M, K, N, H,
+                                           R[7], R[6], R[5], R[4], R[3], R[2], R[1], R[0],
+                                           allow_tf32=controls['triton_allow_tf32'],
+                                           allow_autotune=controls['triton_allow_autotune'],
+                                           BLOCK_SIZE_K=BK, BLOCK_SIZE_N=BN)
         ctx.save_for_backward(input, hashed_weight, random_numbers)
         ctx.output_dim = output_dim
         ctx.chunk_size = chunk_size
         ctx.init_factor = init_factor
         ctx.block_sizes = (BK, BN)
-        ctx.n_extra = (block_size_k is not None) + (block_size_n is not None)
+        ctx.has_bias = bias is not None
         return output
 
     @staticmethod
@@ -79,4 +81,8 @@ class RzLinearFunction(torch.autograd.Function):
                 R[7], R[6], R[5], R[4], R[3], R[2], R[1], R[0],
                 allow_tf32=controls['triton_allow_tf32'], allow_autotune=controls['triton_allow_autotune'],
                 BLOCK_SIZE_K=BK, BLOCK_SIZE_N=BN)
-        return (input_grad, weight_grad, None, None, None, None) + (None,) * ctx.n_extra
+        bias_grad = None
+        if ctx.has_bias and ctx.needs_input_grad[8]:
+            bias_grad = grad.sum(dim=0)
+        # autograd takes one value per argument that apply() was given (6 to 9 of them)
+        return (input_grad, weight_grad, None, None, None, None, None, None, bias_grad)

@@ -19,7 +19,7 @@ _DTYPES = {torch.float32: RZ_F32, torch.bfloat16: RZ_BF16, torch.float16: RZ_F16
 # every symbol that include/rzlinear.h declares
 EXPORTS = (
     "rz_version", "rz_status_string", "rz_tile_offsets", "rz_tile_offsets_device", "rz_forward",
-    "rz_input_grad", "rz_weight_grad_workspace_bytes", "rz_weight_grad", "rz_materialize",
+    "rz_forward_bias", "rz_input_grad", "rz_weight_grad_workspace_bytes", "rz_weight_grad", "rz_materialize",
 )
 
 _lib = None
@@ -56,6 +56,9 @@ def load():
     lib.rz_forward.restype = c_int
     lib.rz_forward.argtypes = [c_vp, c_vp, c_vp, c_int, c_int, c_int, c_int, c_int, c_int, i32p, c_f,
                                c_i64, c_i64, c_int, c_vp]
+    lib.rz_forward_bias.restype = c_int
+    lib.rz_forward_bias.argtypes = [c_vp, c_vp, c_vp, c_vp, c_int, c_int, c_int, c_int, c_int, c_int, i32p,
+                                    c_f, c_i64, c_i64, c_int, c_vp]
     lib.rz_input_grad.restype = c_int
     lib.rz_input_grad.argtypes = lib.rz_forward.argtypes
     lib.rz_weight_grad_workspace_bytes.restype = c_sz

@@ -200,9 +200,9 @@ RZ_API int rz_tile_offsets_device(int32_t* d_out, int K, int N, int H, int BK, i
   return hipGetLastError() == hipSuccess ? RZ_OK : RZ_ERR_LAUNCH;
 }
 
-RZ_API int rz_forward(const void* X, const void* HW, void* Y, int M, int K, int N, int H, int BK,
-                      int BN, const int32_t R[8], float init_factor, int64_t ldx, int64_t ldy,
-                      int dtype, void* stream) {
+RZ_API int rz_forward_bias(const void* X, const void* HW, const void* bias, void* Y, int M, int K,
+                           int N, int H, int BK, int BN, const int32_t R[8], float init_factor,
+                           int64_t ldx, int64_t ldy, int dtype, void* stream) {
   if (X == nullptr || HW == nullptr || Y == nullptr) return RZ_ERR_NULL_POINTER;
   if (dtype_bytes(dtype) == 0) return RZ_ERR_BAD_DTYPE;
   if (M < 1 || ldx < K || ldy < N) return RZ_ERR_BAD_SHAPE;
@@ -212,6 +212,7 @@ RZ_API int rz_forward(const void* X, const void* HW, void* Y, int M, int K, int 
   p.A = X;
   p.HW = HW;
   p.C = Y;
+  p.bias = bias;
   p.I = M;
   p.J = N;
   p.R = K;
@@ -219,6 +220,12 @@ RZ_API int rz_forward(const void* X, const void* HW, void* Y, int M, int K, int 
   p.ldc = ldy;
   p.scale = init_factor;
   return launch_gemm(dtype, kForward, p, nullptr, (hipStream_t)stream) == hipSuccess ? RZ_OK : RZ_ERR_LAUNCH;
+}
+
+RZ_API int rz_forward(const void* X, const void* HW, void* Y, int M, int K, int N, int H, int BK,
+                      int BN, const int32_t R[8], float init_factor, int64_t ldx, int64_t ldy,
+                      int dtype, void* stream) {
+  return rz_forward_bias(X, HW, nullptr, Y, M, K, N, H, BK, BN, R, init_factor, ldx, ldy, dtype, stream);
 }
 
 RZ_API int rz_input_grad(const void* dY, const void* HW, void* dX, int M, int K, int N, int H,

@@ -94,6 +94,7 @@ struct GemmParams {
   const void* B;      // plain B operand (weight-grad) — else unused
   const void* HW;     // hashed weight (forward, input-grad)
   void* C;            // plain output (forward, input-grad)
+  const void* bias;   // optional [J] vector added to every row of C (forward), or null
   float* scatter;     // weight-grad target: fp32 image of dHW (direct atomics), or the
                       // per-workgroup partial images [workgroups][image_pitch] (LDS mode)
   int image_pitch;    // > 0 selects the LDS mode: floats per partial image (H rounded up to 4)

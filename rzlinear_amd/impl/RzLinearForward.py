@@ -19,15 +19,37 @@ def rz_linear_forward_tl(input: torch.Tensor, hashed_weight: torch.Tensor, init_
     accepted and ignored (fp32 always runs on true-fp32 MFMA).  Returns a new [M, N] tensor of
     input's dtype on input's device.
     """
+    return rz_linear_forward_bias_tl(input, hashed_weight, None, init_factor, M, K, N, H,
+                                     R7, R6, R5, R4, R3, R2, R1, R0, allow_tf32=allow_tf32,
+                                     allow_autotune=allow_autotune, BLOCK_SIZE_M=BLOCK_SIZE_M,
+                                     BLOCK_SIZE_N=BLOCK_SIZE_N, BLOCK_SIZE_K=BLOCK_SIZE_K,
+                                     GROUP_SIZE=GROUP_SIZE)
+
+
+def rz_linear_forward_bias_tl(input: torch.Tensor, hashed_weight: torch.Tensor, bias, init_factor: float,
+                              M: int, K: int, N: int, H: int,
+                              R7: int, R6: int, R5: int, R4: int,
+                              R3: int, R2: int, R1: int, R0: int,
+                              allow_tf32: bool = True, allow_autotune: bool = True,
+                              BLOCK_SIZE_M: int = 64, BLOCK_SIZE_N: int = 64, BLOCK_SIZE_K: int = 32,
+                              GROUP_SIZE: int = 4) -> torch.Tensor:
+    """rz_linear_forward_tl with the module's bias (a [N] tensor or None) added inside the
+    kernel's store, instead of by the separate ``x + self._bias`` of the reference module
+    (python/rz_linear/RzLinear.py:93-94)."""
     assert (H > (BLOCK_SIZE_K * BLOCK_SIZE_N))
-    stream = _lib.require_gpu(input, hashed_weight)
+    stream = _lib.require_gpu(input, hashed_weight, *([bias] if bias is not None else []))
     if hashed_weight.dtype != input.dtype:
         raise TypeError("input is %s but hashed_weight is %s" % (input.dtype, hashed_weight.dtype))
+    if bias is not None:
+        if bias.dtype != input.dtype or bias.numel() != N:
+            raise TypeError("bias must be a [%d] tensor of %s" % (N, input.dtype))
+        bias = bias.contiguous()
     x, ldx = _lib.rows(input)
     hw = hashed_weight.contiguous()
     output = torch.empty((M, N), device=input.device, dtype=input.dtype)
-    _lib.check(_lib.load().rz_forward(
-        x.data_ptr(), hw.data_ptr(), output.data_ptr(), M, K, N, H, BLOCK_SIZE_K, BLOCK_SIZE_N,
+    _lib.check(_lib.load().rz_forward_bias(
+        x.data_ptr(), hw.data_ptr(), bias.data_ptr() if bias is not None else None, output.data_ptr(),
+        M, K, N, H, BLOCK_SIZE_K, BLOCK_SIZE_N,
         _lib.hash_constants(R7, R6, R5, R4, R3, R2, R1, R0), float(init_factor), ldx, N,
         _lib.dtype_code(input), stream))
     return output

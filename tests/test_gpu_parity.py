@@ -171,3 +171,62 @@ def test_kernels_match_vectors_produced_by_the_reference_kernels():
         assert rel_err(y.cpu().numpy(), d[name + "_y"]) <= 1e-4
         assert rel_err(dx.cpu().numpy(), d[name + "_dx"]) <= 1e-4
         assert rel_err(dhw.cpu().numpy(), d[name + "_dhw"]) <= 1e-4
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=lambda d: str(d).split(".")[-1])
+def test_module_forward_backward_with_fused_bias(oracle, dtype):
+    """The nn.Module end to end: N-D input, bias fused into the forward kernel, all gradients."""
+    from rzlinear_amd import RzLinear
+    B, S, K, N, BK, BN = 3, 50, 192, 130, 32, 64
+    _say("module", dtype)
+    g = torch.Generator().manual_seed(9)
+    layer = RzLinear(K, N, seed=0, dtype=dtype, compress_ratio=0.5, init_factor=0.25, block_size_k=BK,
+                     block_size_n=BN)
+    H = layer._hashed_weight.shape[0]
+    with torch.no_grad():
+        layer._hashed_weight.copy_(((torch.rand(H, generator=g) * 2 - 1) / K ** 0.5).to(dtype))
+        layer._bias.copy_(torch.randn(N, generator=g).to(dtype))
+    layer = layer.cuda()
+    x = torch.randn((B, S, K), generator=g).to(dtype).cuda().requires_grad_(True)
+    dy = torch.randn((B, S, N), generator=g).to(dtype).cuda()
+    y = layer(x)
+    assert y.shape == (B, S, N) and y.dtype == dtype
+    y.backward(dy)
+    torch.cuda.synchronize()
+    R = layer._random_numbers.tolist()
+    assert R == SEED_CONSTANTS[0]
+    x64 = x.detach().double().cpu().numpy().reshape(-1, K)
+    dy64 = dy.double().cpu().numpy().reshape(-1, N)
+    hw64 = layer._hashed_weight.detach().double().cpu().numpy()
+    b64 = layer._bias.detach().double().cpu().numpy()
+    tol = TOL[dtype]
+    assert rel_err(y.detach().float().cpu().numpy().reshape(-1, N), oracle.forward(x64, hw64, N, BK, BN, R, 0.25) + b64) <= tol
+    assert rel_err(x.grad.float().cpu().numpy().reshape(-1, K), oracle.input_grad(dy64, hw64, K, BK, BN, R, 0.25)) <= tol
+    assert rel_err(layer._hashed_weight.grad.float().cpu().numpy(), oracle.weight_grad(x64, dy64, H, BK, BN, R, 0.25)) <= tol
+    assert rel_err(layer._bias.grad.float().cpu().numpy(), dy64.sum(0)) <= tol
+
+
+def test_function_apply_with_the_reference_six_arguments(oracle):
+    """RzLinearFunction.apply(input, hashed_weight, random_numbers, output_dim, chunk_size, init_factor)
+    as reference code calls it: default tile from `controls`, no bias, and a gradient that is not
+    needed is not computed."""
+    from rzlinear_amd import RzLinearFunction, controls
+    M, K, N, H = 70, 96, 128, 9000
+    BK, BN = controls["block_size_k"], controls["block_size_n"]
+    (x, hw, dy), (x64, hw64, dy64) = make_inputs(M, K, N, H, torch.float32, seed=6)
+    rnd = torch.tensor(R1024, dtype=torch.int32)
+    hw.requires_grad_(True)
+    y = RzLinearFunction.apply(x, hw, rnd, N, 1, 2.0)
+    y.backward(dy)
+    torch.cuda.synchronize()
+    assert x.grad is None
+    assert rel_err(y.detach().cpu().numpy(), oracle.forward(x64, hw64, N, BK, BN, R1024, 2.0)) <= 1e-4
+    assert rel_err(hw.grad.cpu().numpy(), oracle.weight_grad(x64, dy64, H, BK, BN, R1024, 2.0)) <= 1e-4
+    # shared hashed_weight: two layers, autograd adds their weight gradients
+    hw2 = hw.detach().clone().requires_grad_(True)
+    x2 = x.detach().clone().requires_grad_(True)
+    out = RzLinearFunction.apply(x2, hw2, rnd, N, 1, 1.0) + RzLinearFunction.apply(x2, hw2, rnd, N, 1, 1.0)
+    out.backward(dy)
+    torch.cuda.synchronize()
+    assert rel_err(hw2.grad.cpu().numpy(), 2 * oracle.weight_grad(x64, dy64, H, BK, BN, R1024, 1.0)) <= 1e-4
+    assert rel_err(x2.grad.cpu().numpy(), 2 * oracle.input_grad(dy64, hw64, K, BK, BN, R1024, 1.0)) <= 1e-4
