@@ -33,6 +33,14 @@ WORKLOADS = {
     "rec_mlp": (16384, 512, 1024, 5243, "bf16"),
     "ffn": (8192, 4096, 16384, 67109, "bf16"),
     "collision": (32768, 2048, 2048, 32768, "fp32"),
+    # the shape grid of the reference's own benchmark script (python/bench/bench.py:10-11),
+    # with its default compress_ratio 0.0625
+    "grid_32_1024": (32, 1024, 1024, 65536, "fp32"),
+    "grid_128_1024": (128, 1024, 1024, 65536, "fp32"),
+    "grid_1024_1024": (1024, 1024, 1024, 65536, "fp32"),
+    "grid_32_10240": (32, 10240, 10240, 6553600, "fp32"),
+    "grid_128_10240": (128, 10240, 10240, 6553600, "fp32"),
+    "grid_1024_10240": (1024, 10240, 10240, 6553600, "fp32"),
 }
 # dense MFMA peaks of MI355X, TFLOP/s
 PEAK = {"bf16": 2500.0, "fp16": 2500.0, "fp32": 157.3}

@@ -119,6 +119,8 @@ __global__ __launch_bounds__(256) void reduce_partials_kernel(const float* __res
   const int slot = (blockIdx.x * 16 + q) * 4;
   float4 s = {0.f, 0.f, 0.f, 0.f};
   if (slot < pitch) {
+    // eight loads in flight per thread; the order of the additions stays fixed
+#pragma unroll 8
     for (int p = g; p < nparts; p += 16) {
       const float4 v = *reinterpret_cast<const float4*>(part + (size_t)p * pitch + slot);
       s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;

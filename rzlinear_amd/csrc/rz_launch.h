@@ -23,11 +23,46 @@ static inline long long tile_count(int I, int J, int t) {
   return (long long)((I + t - 1) / t) * ((J + t - 1) / t);
 }
 
+// Relative throughput of a tile shape at a given number of workgroups, from bf16 measurements
+// on MI355X (256 tile at one workgroup per compute unit = 1): the 128 tile reaches 0.51 with one
+// workgroup per compute unit and 0.75 with two or more, the 64 tile 0.16 and 0.33 (four or
+// more); below one workgroup per compute unit the rate falls with the idle compute units, and
+// a last, partly filled round of workgroups costs a full one.
+static inline double tile_score_full(int I, int J, int t);
+// ... times the share of a tile grid's MFMA work that is not padding
+static inline double tile_score(int I, int J, int t) {
+  const double wgs = (double)tile_count(I, J, t);
+  return tile_score_full(I, J, t) * ((double)I * (double)J) / (wgs * t * t);
+}
+static inline double tile_score_full(int I, int J, int t) {
+  const double wgs = (double)tile_count(I, J, t);
+  const double per_cu = wgs / kComputeUnits;
+  const int slots = (t == 256) ? 1 : (t == 128 ? 2 : 4);          // resident workgroups per CU
+  const double lo = (t == 256) ? 1.0 : (t == 128 ? 0.51 : 0.16);  // at one workgroup per CU
+  const double hi = (t == 256) ? 1.0 : (t == 128 ? 0.75 : 0.33);  // at `slots` per CU
+  if (per_cu <= 1.0) return lo * per_cu;
+  const double cap = (double)kComputeUnits * slots;
+  const double rounds = (double)((long long)((wgs + cap - 1) / cap));
+  const double util = wgs / (rounds * cap);                        // tail effect
+  const double fill = per_cu >= slots ? 1.0 : (per_cu - 1.0) / (slots - 1.0);
+  const double e = lo + (hi - lo) * fill;
+  // between one and `slots` workgroups per CU every CU is busy: no tail penalty yet
+  return per_cu >= slots ? e * util : e;
+}
+
 static inline int pick_tile(int I, int J) {
   if (forced_tile()) return forced_tile();
-  if (tile_count(I, J, 256) >= kComputeUnits / 2) return 256;
-  if (tile_count(I, J, 128) >= kComputeUnits * 3 / 4) return 128;
-  return 64;
+  int best = 256;
+  double best_score = tile_score(I, J, 256);
+  const int others[2] = {128, 64};
+  for (int t : others) {
+    const double sc = tile_score(I, J, t);
+    if (sc > best_score * 1.02) {   // prefer the larger tile on a near tie
+      best = t;
+      best_score = sc;
+    }
+  }
+  return best;
 }
 
 // How the weight-grad contraction C[K,N] = X^T.dY over M is cut into workgroups, and how the
