@@ -592,19 +592,26 @@ struct GemmKernel {
     } else {
       T* __restrict__ gC = static_cast<T*>(p.C);
       const T* __restrict__ gBias = static_cast<const T*>(p.bias);
+      // optional bias of this lane's columns, added in fp32 before the single rounding
+      float bias[MJ];
 #pragma unroll
       for (int b = 0; b < MJ; b++) {
         const int col = j0 + wave_j * WTJ + b * 32 + (lane & 31);
-        // optional bias of this column, added in fp32 before the single rounding of the result
-        float bias = 0.f;
-        if (gBias != nullptr && (FULL || col < p.J)) bias = Tr::to_float(gBias[col]);
+        bias[b] = 0.f;
+        if (gBias != nullptr && (FULL || col < p.J)) bias[b] = Tr::to_float(gBias[col]);
+      }
+      // the column blocks of a row go out back to back, so that the halves of a cache line
+      // reach L2 together
 #pragma unroll
-        for (int a = 0; a < MI; a++) {
+      for (int a = 0; a < MI; a++) {
 #pragma unroll
-          for (int e = 0; e < 16; e++) {
-            const int row = i0 + wave_i * WTI + a * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
+        for (int e = 0; e < 16; e++) {
+          const int row = i0 + wave_i * WTI + a * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
+#pragma unroll
+          for (int b = 0; b < MJ; b++) {
+            const int col = j0 + wave_j * WTJ + b * 32 + (lane & 31);
             if (FULL || (row < p.I && col < p.J))
-              gC[(int64_t)row * p.ldc + col] = Tr::from_float(acc[a][b][e] * p.scale + bias);
+              gC[(int64_t)row * p.ldc + col] = Tr::from_float(acc[a][b][e] * p.scale + bias[b]);
           }
         }
       }
