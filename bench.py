@@ -109,15 +109,20 @@ def main():
     dhw = torch.empty((H,), dtype=dtype, device=dev)
     ws_bytes = lib.rz_weight_grad_workspace_bytes(M, K, N, H, BK, BN, code)
     ws = torch.empty((max(ws_bytes, 16),), dtype=torch.uint8, device=dev)
+    # skinny workloads split the contraction of forward / input-grad (0 bytes = no split)
+    fws_bytes = lib.rz_forward_workspace_bytes(M, K, N, H, BK, BN, code)
+    iws_bytes = lib.rz_input_grad_workspace_bytes(M, K, N, H, BK, BN, code)
+    fws = torch.empty((max(fws_bytes, 16),), dtype=torch.uint8, device=dev)
+    iws = torch.empty((max(iws_bytes, 16),), dtype=torch.uint8, device=dev)
     stream = torch.cuda.current_stream(dev).cuda_stream
 
     def fwd():
-        _lib.check(lib.rz_forward(x.data_ptr(), hw.data_ptr(), y.data_ptr(), M, K, N, H, BK, BN, R, 1.0, K, N,
-                                  code, stream))
+        _lib.check(lib.rz_forward_ws(x.data_ptr(), hw.data_ptr(), None, y.data_ptr(), fws.data_ptr(), fws_bytes,
+                                     M, K, N, H, BK, BN, R, 1.0, K, N, code, stream))
 
     def igrad():
-        _lib.check(lib.rz_input_grad(dy.data_ptr(), hw.data_ptr(), dx.data_ptr(), M, K, N, H, BK, BN, R, 1.0,
-                                     N, K, code, stream))
+        _lib.check(lib.rz_input_grad_ws(dy.data_ptr(), hw.data_ptr(), dx.data_ptr(), iws.data_ptr(), iws_bytes,
+                                        M, K, N, H, BK, BN, R, 1.0, N, K, code, stream))
 
     def wgrad():
         _lib.check(lib.rz_weight_grad(x.data_ptr(), dy.data_ptr(), dhw.data_ptr(), ws.data_ptr(), ws_bytes,

@@ -103,6 +103,26 @@ int rz_input_grad(const void* dY, const void* HW, void* dX, int M, int K, int N,
                   int dtype, void* stream);
 
 /*
+ * Forward / input-grad that may split the contraction: with few output tiles and a long
+ * contracted dimension (skinny batches such as M = 32 against K = N = 10240) the work is cut
+ * into slices that write fp32 partial results to `workspace`, and a second kernel adds them
+ * (plus bias) into the output.  *_workspace_bytes returns the size needed (0 = no split; then
+ * these calls equal rz_forward_bias / rz_input_grad and workspace may be NULL).  No
+ * counterpart in the reference, whose kernels never split (impl/RzLinearForward.py:37-40,
+ * impl/RzLinearBackward.py:407-410).
+ */
+size_t rz_forward_workspace_bytes(int M, int K, int N, int H, int BK, int BN, int dtype);
+int rz_forward_ws(const void* X, const void* HW, const void* bias, void* Y, void* workspace,
+                  size_t workspace_bytes, int M, int K, int N, int H, int BK, int BN,
+                  const int32_t R[8], float init_factor, int64_t ldx, int64_t ldy, int dtype,
+                  void* stream);
+size_t rz_input_grad_workspace_bytes(int M, int K, int N, int H, int BK, int BN, int dtype);
+int rz_input_grad_ws(const void* dY, const void* HW, void* dX, void* workspace,
+                     size_t workspace_bytes, int M, int K, int N, int H, int BK, int BN,
+                     const int32_t R[8], float init_factor, int64_t lddy, int64_t lddx, int dtype,
+                     void* stream);
+
+/*
  * Bytes of device workspace rz_weight_grad needs for this problem (0 when none).
  * When hashed_weight is small enough for an fp32 image of dHW to fit the LDS of a compute
  * unit, every workgroup stores one partial image ([workgroups][H rounded up to 4] floats) that

@@ -19,7 +19,8 @@ _DTYPES = {torch.float32: RZ_F32, torch.bfloat16: RZ_BF16, torch.float16: RZ_F16
 # every symbol that include/rzlinear.h declares
 EXPORTS = (
     "rz_version", "rz_status_string", "rz_tile_offsets", "rz_tile_offsets_device", "rz_forward",
-    "rz_forward_bias", "rz_input_grad", "rz_weight_grad_workspace_bytes", "rz_weight_grad", "rz_materialize",
+    "rz_forward_bias", "rz_forward_workspace_bytes", "rz_forward_ws", "rz_input_grad",
+    "rz_input_grad_workspace_bytes", "rz_input_grad_ws", "rz_weight_grad_workspace_bytes", "rz_weight_grad", "rz_materialize",
 )
 
 _lib = None
@@ -61,6 +62,16 @@ def load():
                                     c_f, c_i64, c_i64, c_int, c_vp]
     lib.rz_input_grad.restype = c_int
     lib.rz_input_grad.argtypes = lib.rz_forward.argtypes
+    lib.rz_forward_workspace_bytes.restype = c_sz
+    lib.rz_forward_workspace_bytes.argtypes = [c_int] * 7
+    lib.rz_input_grad_workspace_bytes.restype = c_sz
+    lib.rz_input_grad_workspace_bytes.argtypes = [c_int] * 7
+    lib.rz_forward_ws.restype = c_int
+    lib.rz_forward_ws.argtypes = [c_vp, c_vp, c_vp, c_vp, c_vp, c_sz, c_int, c_int, c_int, c_int, c_int, c_int,
+                                  i32p, c_f, c_i64, c_i64, c_int, c_vp]
+    lib.rz_input_grad_ws.restype = c_int
+    lib.rz_input_grad_ws.argtypes = [c_vp, c_vp, c_vp, c_vp, c_sz, c_int, c_int, c_int, c_int, c_int, c_int,
+                                     i32p, c_f, c_i64, c_i64, c_int, c_vp]
     lib.rz_weight_grad_workspace_bytes.restype = c_sz
     lib.rz_weight_grad_workspace_bytes.argtypes = [c_int] * 7
     lib.rz_weight_grad.restype = c_int
@@ -107,6 +118,11 @@ def rows(t):
         t = t.contiguous()
     ld = t.stride(0) if t.shape[0] > 1 else max(t.shape[1], 1)
     return t, ld
+
+
+def workspace(nbytes, device):
+    """A scratch buffer of nbytes on `device` (None when nbytes is 0)."""
+    return torch.empty((nbytes,), device=device, dtype=torch.uint8) if nbytes else None
 
 
 def tile_offsets(K, N, H, BLOCK_SIZE_K, BLOCK_SIZE_N, random_numbers, hash_levels=2):

@@ -65,11 +65,11 @@ static int dtype_bytes(int dtype) {
 }
 
 static hipError_t launch_gemm(int dtype, int op, const GemmParams& p, const WeightGradPlan* plan,
-                              hipStream_t s) {
+                              const SplitPlan* split, hipStream_t s) {
   switch (dtype) {
-    case RZ_F32: return launch_gemm_f32(op, p, plan, s);
-    case RZ_BF16: return launch_gemm_bf16(op, p, plan, s);
-    case RZ_F16: return launch_gemm_f16(op, p, plan, s);
+    case RZ_F32: return launch_gemm_f32(op, p, plan, split, s);
+    case RZ_BF16: return launch_gemm_bf16(op, p, plan, split, s);
+    case RZ_F16: return launch_gemm_f16(op, p, plan, split, s);
     default: return hipErrorInvalidValue;
   }
 }
@@ -140,6 +140,61 @@ __global__ __launch_bounds__(256) void reduce_partials_kernel(const float* __res
   }
 }
 
+// C[i][j] = sum over the slices of part[s][i][j] (+ bias[j]), converted to the element type.
+template <typename T>
+__global__ __launch_bounds__(256) void reduce_slices_kernel(const float* __restrict__ part,
+                                                            T* __restrict__ C, const T* __restrict__ bias,
+                                                            int I, int J, int64_t ldc, int slices) {
+  const size_t plane = (size_t)I * (size_t)J;
+  const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= plane) return;
+  const int i = (int)(idx / J), j = (int)(idx % J);
+  float s = 0.f;
+  for (int k = 0; k < slices; k++) s += part[(size_t)k * plane + idx];
+  if (bias != nullptr) s += ElemTraits<T>::to_float(bias[j]);
+  C[(int64_t)i * ldc + j] = ElemTraits<T>::from_float(s);
+}
+
+template <typename T>
+static hipError_t reduce_slices(const float* part, void* C, const void* bias, int I, int J, int64_t ldc,
+                                int slices, hipStream_t s) {
+  const size_t plane = (size_t)I * (size_t)J;
+  const size_t blocks = (plane + 255) / 256;
+  if (blocks > 0x7fffffffULL) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(reduce_slices_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, s, part, (T*)C,
+                     (const T*)bias, I, J, ldc, slices);
+  return hipGetLastError();
+}
+
+static hipError_t reduce_slices_dtype(int dtype, const float* part, void* C, const void* bias, int I, int J,
+                                      int64_t ldc, int slices, hipStream_t s) {
+  switch (dtype) {
+    case RZ_F32: return reduce_slices<float>(part, C, bias, I, J, ldc, slices, s);
+    case RZ_BF16: return reduce_slices<bf16_t>(part, C, bias, I, J, ldc, slices, s);
+    case RZ_F16: return reduce_slices<f16_t>(part, C, bias, I, J, ldc, slices, s);
+    default: return hipErrorInvalidValue;
+  }
+}
+
+// Forward (op kForward) or input-grad through one code path: p holds the operands; with a
+// workspace the contraction may be split over R (skinny problems).
+static int run_plain_op(int op, int dtype, GemmParams p, const void* bias, void* workspace,
+                        size_t workspace_bytes, bool may_split, hipStream_t s) {
+  if (may_split) {
+    const SplitPlan sp = plan_split(p.I, p.J, p.R, dtype_bytes(dtype));
+    if (sp.splits > 1) {
+      if (workspace == nullptr || workspace_bytes < sp.workspace_bytes) return RZ_ERR_WORKSPACE;
+      p.partial = (float*)workspace;
+      p.bias = nullptr;
+      if (launch_gemm(dtype, op, p, nullptr, &sp, s) != hipSuccess) return RZ_ERR_LAUNCH;
+      return reduce_slices_dtype(dtype, p.partial, p.C, bias, p.I, p.J, p.ldc, sp.splits, s) == hipSuccess
+                 ? RZ_OK : RZ_ERR_LAUNCH;
+    }
+  }
+  p.bias = bias;
+  return launch_gemm(dtype, op, p, nullptr, nullptr, s) == hipSuccess ? RZ_OK : RZ_ERR_LAUNCH;
+}
+
 static hipError_t zero_words(void* p, size_t bytes, hipStream_t s) {
   // bytes is a multiple of 4 for every caller (fp32 images)
   const size_t words = bytes / 4;
@@ -202,9 +257,10 @@ RZ_API int rz_tile_offsets_device(int32_t* d_out, int K, int N, int H, int BK, i
   return hipGetLastError() == hipSuccess ? RZ_OK : RZ_ERR_LAUNCH;
 }
 
-RZ_API int rz_forward_bias(const void* X, const void* HW, const void* bias, void* Y, int M, int K,
-                           int N, int H, int BK, int BN, const int32_t R[8], float init_factor,
-                           int64_t ldx, int64_t ldy, int dtype, void* stream) {
+static int forward_impl(const void* X, const void* HW, const void* bias, void* Y, void* workspace,
+                        size_t workspace_bytes, bool may_split, int M, int K, int N, int H, int BK, int BN,
+                        const int32_t R[8], float init_factor, int64_t ldx, int64_t ldy, int dtype,
+                        void* stream) {
   if (X == nullptr || HW == nullptr || Y == nullptr) return RZ_ERR_NULL_POINTER;
   if (dtype_bytes(dtype) == 0) return RZ_ERR_BAD_DTYPE;
   if (M < 1 || ldx < K || ldy < N) return RZ_ERR_BAD_SHAPE;
@@ -214,25 +270,18 @@ RZ_API int rz_forward_bias(const void* X, const void* HW, const void* bias, void
   p.A = X;
   p.HW = HW;
   p.C = Y;
-  p.bias = bias;
   p.I = M;
   p.J = N;
   p.R = K;
   p.lda = ldx;
   p.ldc = ldy;
   p.scale = init_factor;
-  return launch_gemm(dtype, kForward, p, nullptr, (hipStream_t)stream) == hipSuccess ? RZ_OK : RZ_ERR_LAUNCH;
+  return run_plain_op(kForward, dtype, p, bias, workspace, workspace_bytes, may_split, (hipStream_t)stream);
 }
 
-RZ_API int rz_forward(const void* X, const void* HW, void* Y, int M, int K, int N, int H, int BK,
-                      int BN, const int32_t R[8], float init_factor, int64_t ldx, int64_t ldy,
-                      int dtype, void* stream) {
-  return rz_forward_bias(X, HW, nullptr, Y, M, K, N, H, BK, BN, R, init_factor, ldx, ldy, dtype, stream);
-}
-
-RZ_API int rz_input_grad(const void* dY, const void* HW, void* dX, int M, int K, int N, int H,
-                         int BK, int BN, const int32_t R[8], float init_factor, int64_t lddy,
-                         int64_t lddx, int dtype, void* stream) {
+static int input_grad_impl(const void* dY, const void* HW, void* dX, void* workspace, size_t workspace_bytes,
+                           bool may_split, int M, int K, int N, int H, int BK, int BN, const int32_t R[8],
+                           float init_factor, int64_t lddy, int64_t lddx, int dtype, void* stream) {
   if (dY == nullptr || HW == nullptr || dX == nullptr) return RZ_ERR_NULL_POINTER;
   if (dtype_bytes(dtype) == 0) return RZ_ERR_BAD_DTYPE;
   if (M < 1 || lddy < N || lddx < K) return RZ_ERR_BAD_SHAPE;
@@ -248,7 +297,59 @@ RZ_API int rz_input_grad(const void* dY, const void* HW, void* dX, int M, int K,
   p.lda = lddy;
   p.ldc = lddx;
   p.scale = init_factor;
-  return launch_gemm(dtype, kInputGrad, p, nullptr, (hipStream_t)stream) == hipSuccess ? RZ_OK : RZ_ERR_LAUNCH;
+  return run_plain_op(kInputGrad, dtype, p, nullptr, workspace, workspace_bytes, may_split,
+                      (hipStream_t)stream);
+}
+
+RZ_API int rz_forward_bias(const void* X, const void* HW, const void* bias, void* Y, int M, int K,
+                           int N, int H, int BK, int BN, const int32_t R[8], float init_factor,
+                           int64_t ldx, int64_t ldy, int dtype, void* stream) {
+  return forward_impl(X, HW, bias, Y, nullptr, 0, false, M, K, N, H, BK, BN, R, init_factor, ldx, ldy, dtype,
+                      stream);
+}
+
+RZ_API int rz_forward(const void* X, const void* HW, void* Y, int M, int K, int N, int H, int BK,
+                      int BN, const int32_t R[8], float init_factor, int64_t ldx, int64_t ldy,
+                      int dtype, void* stream) {
+  return forward_impl(X, HW, nullptr, Y, nullptr, 0, false, M, K, N, H, BK, BN, R, init_factor, ldx, ldy,
+                      dtype, stream);
+}
+
+RZ_API size_t rz_forward_workspace_bytes(int M, int K, int N, int H, int BK, int BN, int dtype) {
+  (void)H; (void)BK; (void)BN;
+  const int eb = dtype_bytes(dtype);
+  if (eb == 0 || M < 1 || K < 1 || N < 1) return 0;
+  return plan_split(M, N, K, eb).workspace_bytes;
+}
+
+RZ_API int rz_forward_ws(const void* X, const void* HW, const void* bias, void* Y, void* workspace,
+                         size_t workspace_bytes, int M, int K, int N, int H, int BK, int BN,
+                         const int32_t R[8], float init_factor, int64_t ldx, int64_t ldy, int dtype,
+                         void* stream) {
+  return forward_impl(X, HW, bias, Y, workspace, workspace_bytes, true, M, K, N, H, BK, BN, R, init_factor,
+                      ldx, ldy, dtype, stream);
+}
+
+RZ_API int rz_input_grad(const void* dY, const void* HW, void* dX, int M, int K, int N, int H,
+                         int BK, int BN, const int32_t R[8], float init_factor, int64_t lddy,
+                         int64_t lddx, int dtype, void* stream) {
+  return input_grad_impl(dY, HW, dX, nullptr, 0, false, M, K, N, H, BK, BN, R, init_factor, lddy, lddx,
+                         dtype, stream);
+}
+
+RZ_API size_t rz_input_grad_workspace_bytes(int M, int K, int N, int H, int BK, int BN, int dtype) {
+  (void)H; (void)BK; (void)BN;
+  const int eb = dtype_bytes(dtype);
+  if (eb == 0 || M < 1 || K < 1 || N < 1) return 0;
+  return plan_split(M, K, N, eb).workspace_bytes;
+}
+
+RZ_API int rz_input_grad_ws(const void* dY, const void* HW, void* dX, void* workspace,
+                            size_t workspace_bytes, int M, int K, int N, int H, int BK, int BN,
+                            const int32_t R[8], float init_factor, int64_t lddy, int64_t lddx, int dtype,
+                            void* stream) {
+  return input_grad_impl(dY, HW, dX, workspace, workspace_bytes, true, M, K, N, H, BK, BN, R, init_factor,
+                         lddy, lddx, dtype, stream);
 }
 
 RZ_API size_t rz_weight_grad_workspace_bytes(int M, int K, int N, int H, int BK, int BN, int dtype) {
@@ -284,7 +385,7 @@ RZ_API int rz_weight_grad(const void* X, const void* dY, void* dHW, void* worksp
     // every workgroup sums its tiles into an LDS image of dHW and stores it as a partial image;
     // the partial images are then added up (no global atomics, fixed summation order)
     p.scatter = (float*)workspace;
-    if (launch_gemm(dtype, kWeightGrad, p, &plan, s) != hipSuccess) return RZ_ERR_LAUNCH;
+    if (launch_gemm(dtype, kWeightGrad, p, &plan, nullptr, s) != hipSuccess) return RZ_ERR_LAUNCH;
     const int blocks = (plan.image_pitch / 4 + 15) / 16;
     const int nparts = (int)plan.workgroups;
     if (dtype == RZ_F32)
@@ -302,7 +403,7 @@ RZ_API int rz_weight_grad(const void* X, const void* dY, void* dHW, void* worksp
   float* image = (dtype == RZ_F32) ? (float*)dHW : (float*)workspace;
   if (zero_words(image, (size_t)H * sizeof(float), s) != hipSuccess) return RZ_ERR_LAUNCH;
   p.scatter = image;
-  if (launch_gemm(dtype, kWeightGrad, p, &plan, s) != hipSuccess) return RZ_ERR_LAUNCH;
+  if (launch_gemm(dtype, kWeightGrad, p, &plan, nullptr, s) != hipSuccess) return RZ_ERR_LAUNCH;
   if (dtype == RZ_BF16) {
     hipLaunchKernelGGL(convert_from_f32_kernel<bf16_t>, dim3((H + 255) / 256), dim3(256), 0, s, image,
                        (bf16_t*)dHW, H);

@@ -95,6 +95,8 @@ struct GemmParams {
   const void* HW;     // hashed weight (forward, input-grad)
   void* C;            // plain output (forward, input-grad)
   const void* bias;   // optional [J] vector added to every row of C (forward), or null
+  float* partial;     // forward/input-grad with R split over blockIdx.y: fp32 partial results
+                      // [slices][I][J] (scaled, no bias) instead of C; null = no split
   float* scatter;     // weight-grad target: fp32 image of dHW (direct atomics), or the
                       // per-workgroup partial images [workgroups][image_pitch] (LDS mode)
   int image_pitch;    // > 0 selects the LDS mode: floats per partial image (H rounded up to 4)

@@ -590,6 +590,24 @@ struct GemmKernel {
         scatter(p.scatter);
       }
     } else {
+      if (p.partial != nullptr) {
+        // R is split over blockIdx.y (few C tiles, long R): this slice's scaled fp32 partial
+        // result goes to its own [I][J] plane; a second kernel adds the planes up
+        float* __restrict__ gP = p.partial + (size_t)blockIdx.y * (size_t)p.I * (size_t)p.J;
+#pragma unroll
+        for (int a = 0; a < MI; a++) {
+#pragma unroll
+          for (int e = 0; e < 16; e++) {
+            const int row = i0 + wave_i * WTI + a * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
+#pragma unroll
+            for (int b = 0; b < MJ; b++) {
+              const int col = j0 + wave_j * WTJ + b * 32 + (lane & 31);
+              if (FULL || (row < p.I && col < p.J)) gP[(size_t)row * p.J + col] = acc[a][b][e] * p.scale;
+            }
+          }
+        }
+        return;
+      }
       T* __restrict__ gC = static_cast<T*>(p.C);
       const T* __restrict__ gBias = static_cast<const T*>(p.bias);
       // optional bias of this lane's columns, added in fp32 before the single rounding

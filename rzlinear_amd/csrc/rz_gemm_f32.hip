@@ -2,7 +2,8 @@
 #include "rz_gemm_inst.h"
 
 namespace rz {
-hipError_t launch_gemm_f32(int op, GemmParams p, const WeightGradPlan* plan, hipStream_t stream) {
-  return launch_gemm_t<float>(op, p, plan, stream);
+hipError_t launch_gemm_f32(int op, GemmParams p, const WeightGradPlan* plan, const SplitPlan* split,
+                           hipStream_t stream) {
+  return launch_gemm_t<float>(op, p, plan, split, stream);
 }
 }  // namespace rz

@@ -7,7 +7,8 @@
 namespace rz {
 
 template <typename T, int OP, int TI, int TJ, int WI, int WJ, int NSTAGE, bool FULL>
-static hipError_t launch_one(GemmParams p, const WeightGradPlan* plan, hipStream_t stream) {
+static hipError_t launch_one(GemmParams p, const WeightGradPlan* plan, const SplitPlan* split,
+                             hipStream_t stream) {
   typedef GemmKernel<T, OP, TI, TJ, WI, WJ, NSTAGE, FULL> K;
   p.tiles_i = (p.I + TI - 1) / TI;
   p.tiles_j = (p.J + TJ - 1) / TJ;
@@ -21,8 +22,13 @@ static hipError_t launch_one(GemmParams p, const WeightGradPlan* plan, hipStream
     p.r_chunk = plan->r_chunk;
     p.image_pitch = plan->image_pitch;
     if ((size_t)p.image_pitch * sizeof(float) > kMaxImageBytes) return hipErrorInvalidValue;
+  } else if (split != nullptr && split->splits > 1) {
+    if (split->tile != TI || p.partial == nullptr) return hipErrorInvalidValue;
+    splits = split->splits;
+    p.r_chunk = split->r_chunk;
   } else {
     p.r_chunk = r_steps * K::TR;
+    p.partial = nullptr;
   }
   auto kernel = rz_gemm_kernel<T, OP, TI, TJ, WI, WJ, NSTAGE, FULL>;
   size_t smem = sizeof(typename K::Smem);
@@ -44,19 +50,21 @@ static hipError_t launch_one(GemmParams p, const WeightGradPlan* plan, hipStream
 
 // FULL kernels carry no bounds checks: every tile and every R step must be complete.
 template <typename T, int OP, int TILE, int WI, int WJ, int NSTAGE>
-static hipError_t launch_tile(GemmParams p, const WeightGradPlan* plan, hipStream_t stream) {
+static hipError_t launch_tile(GemmParams p, const WeightGradPlan* plan, const SplitPlan* split,
+                              hipStream_t stream) {
   constexpr int TR = 128 / ElemTraits<T>::kBytes;
   const bool full = (p.I % TILE == 0) && (p.J % TILE == 0) && (p.R % TR == 0);
-  if (full) return launch_one<T, OP, TILE, TILE, WI, WJ, NSTAGE, true>(p, plan, stream);
-  return launch_one<T, OP, TILE, TILE, WI, WJ, NSTAGE, false>(p, plan, stream);
+  if (full) return launch_one<T, OP, TILE, TILE, WI, WJ, NSTAGE, true>(p, plan, split, stream);
+  return launch_one<T, OP, TILE, TILE, WI, WJ, NSTAGE, false>(p, plan, split, stream);
 }
 
 template <typename T, int TILE, int WI, int WJ, int NSTAGE>
-static hipError_t launch_op(int op, GemmParams p, const WeightGradPlan* plan, hipStream_t stream) {
+static hipError_t launch_op(int op, GemmParams p, const WeightGradPlan* plan, const SplitPlan* split,
+                            hipStream_t stream) {
   switch (op) {
-    case kForward: return launch_tile<T, kForward, TILE, WI, WJ, NSTAGE>(p, plan, stream);
-    case kInputGrad: return launch_tile<T, kInputGrad, TILE, WI, WJ, NSTAGE>(p, plan, stream);
-    case kWeightGrad: return launch_tile<T, kWeightGrad, TILE, WI, WJ, NSTAGE>(p, plan, stream);
+    case kForward: return launch_tile<T, kForward, TILE, WI, WJ, NSTAGE>(p, plan, split, stream);
+    case kInputGrad: return launch_tile<T, kInputGrad, TILE, WI, WJ, NSTAGE>(p, plan, split, stream);
+    case kWeightGrad: return launch_tile<T, kWeightGrad, TILE, WI, WJ, NSTAGE>(p, plan, split, stream);
     default: return hipErrorInvalidValue;
   }
 }
@@ -68,16 +76,18 @@ static hipError_t launch_op(int op, GemmParams p, const WeightGradPlan* plan, hi
 // RZLINEAR_STAGES=1 selects a single-stage 128 x 128 form that leans on several workgroups
 // per compute unit instead of a pipeline (tuning aid).
 template <typename T>
-static hipError_t launch_gemm_t(int op, GemmParams p, const WeightGradPlan* plan, hipStream_t stream) {
-  const int tile = (op == kWeightGrad && plan != nullptr) ? plan->tile : pick_tile(p.I, p.J);
+static hipError_t launch_gemm_t(int op, GemmParams p, const WeightGradPlan* plan, const SplitPlan* split,
+                                hipStream_t stream) {
+  const int tile = (op == kWeightGrad && plan != nullptr) ? plan->tile
+                   : (split != nullptr ? split->tile : pick_tile(p.I, p.J));
   const char* stages_env = getenv("RZLINEAR_STAGES");
   const bool one_stage = stages_env != nullptr && atoi(stages_env) == 1;
   switch (tile) {
-    case 256: return launch_op<T, 256, 2, 4, 2>(op, p, plan, stream);
-    case 64: return launch_op<T, 64, 2, 2, 2>(op, p, plan, stream);
+    case 256: return launch_op<T, 256, 2, 4, 2>(op, p, plan, split, stream);
+    case 64: return launch_op<T, 64, 2, 2, 2>(op, p, plan, split, stream);
     case 128:
-      if (one_stage) return launch_op<T, 128, 2, 2, 1>(op, p, plan, stream);
-      return launch_op<T, 128, 2, 2, 2>(op, p, plan, stream);
+      if (one_stage) return launch_op<T, 128, 2, 2, 1>(op, p, plan, split, stream);
+      return launch_op<T, 128, 2, 2, 2>(op, p, plan, split, stream);
     default: return hipErrorInvalidValue;
   }
 }

@@ -123,10 +123,44 @@ static inline WeightGradPlan plan_weight_grad(int M, int K, int N, int H, int el
   return pl;
 }
 
+// Forward / input-grad with few C tiles and a long contraction (skinny batches): R is cut into
+// slices over blockIdx.y, every slice writes an fp32 partial result, a second kernel adds them.
+struct SplitPlan {
+  int tile;
+  int splits;        // 1 = no split, no workspace
+  int r_chunk;
+  size_t workspace_bytes;
+};
+
+static inline SplitPlan plan_split(int I, int J, int R, int elem_bytes) {
+  SplitPlan pl;
+  const int TR = 128 / elem_bytes;
+  pl.tile = pick_tile(I, J);
+  const long long tiles = tile_count(I, J, pl.tile);
+  const int r_steps = (R + TR - 1) / TR;
+  const int slots = (pl.tile == 256) ? 1 : (pl.tile == 128 ? 2 : 4);
+  long long want = ((long long)kComputeUnits * slots + tiles - 1) / tiles;   // fill every CU slot
+  // a slice should run at least 16 steps (8 when most compute units would otherwise sit idle)
+  const int min_steps = (tiles * 2 < kComputeUnits) ? 8 : 16;
+  if (want > r_steps / min_steps) want = r_steps / min_steps;
+  if (want > 16) want = 16;
+  if (tiles * 2 >= (long long)kComputeUnits * slots || want < 2 || getenv("RZLINEAR_NO_SPLIT") != nullptr)
+    want = 1;
+  const int steps_per = (int)((r_steps + want - 1) / want);
+  pl.splits = (r_steps + steps_per - 1) / steps_per;
+  pl.r_chunk = steps_per * TR;
+  pl.workspace_bytes = pl.splits > 1 ? (size_t)pl.splits * (size_t)I * (size_t)J * sizeof(float) : 0;
+  return pl;
+}
+
 // Fills in the tiling fields of `p` and enqueues the kernel for `op` on `stream`; weight-grad
 // takes its plan (tile, split of M, scatter mode) from `plan`, the others ignore it.
-hipError_t launch_gemm_f32(int op, GemmParams p, const WeightGradPlan* plan, hipStream_t stream);
-hipError_t launch_gemm_bf16(int op, GemmParams p, const WeightGradPlan* plan, hipStream_t stream);
-hipError_t launch_gemm_f16(int op, GemmParams p, const WeightGradPlan* plan, hipStream_t stream);
+// (forward / input-grad take tile and split from `split`, or pick a tile and do not split).
+hipError_t launch_gemm_f32(int op, GemmParams p, const WeightGradPlan* plan, const SplitPlan* split,
+                           hipStream_t stream);
+hipError_t launch_gemm_bf16(int op, GemmParams p, const WeightGradPlan* plan, const SplitPlan* split,
+                            hipStream_t stream);
+hipError_t launch_gemm_f16(int op, GemmParams p, const WeightGradPlan* plan, const SplitPlan* split,
+                           hipStream_t stream);
 
 }  // namespace rz

@@ -75,8 +75,12 @@ def rz_linear_backward_input_grad_tl(output_grad: torch.Tensor, hashed_weight: t
     dy, lddy = _lib.rows(output_grad)
     hw = hashed_weight.contiguous()
     input_grad = torch.empty((M, K), device=output_grad.device, dtype=output_grad.dtype)
-    _lib.check(_lib.load().rz_input_grad(
-        dy.data_ptr(), hw.data_ptr(), input_grad.data_ptr(), M, K, N, H, BLOCK_SIZE_K, BLOCK_SIZE_N,
-        _lib.hash_constants(R7, R6, R5, R4, R3, R2, R1, R0), float(init_factor), lddy, K,
-        _lib.dtype_code(output_grad), stream))
+    lib = _lib.load()
+    code = _lib.dtype_code(output_grad)
+    need = lib.rz_input_grad_workspace_bytes(M, K, N, H, BLOCK_SIZE_K, BLOCK_SIZE_N, code)
+    ws = _lib.workspace(need, output_grad.device)
+    _lib.check(lib.rz_input_grad_ws(
+        dy.data_ptr(), hw.data_ptr(), input_grad.data_ptr(), ws.data_ptr() if need else None, need,
+        M, K, N, H, BLOCK_SIZE_K, BLOCK_SIZE_N,
+        _lib.hash_constants(R7, R6, R5, R4, R3, R2, R1, R0), float(init_factor), lddy, K, code, stream))
     return input_grad

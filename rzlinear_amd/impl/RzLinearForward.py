@@ -47,9 +47,13 @@ def rz_linear_forward_bias_tl(input: torch.Tensor, hashed_weight: torch.Tensor, 
     x, ldx = _lib.rows(input)
     hw = hashed_weight.contiguous()
     output = torch.empty((M, N), device=input.device, dtype=input.dtype)
-    _lib.check(_lib.load().rz_forward_bias(
+    lib = _lib.load()
+    code = _lib.dtype_code(input)
+    # skinny problems split the contraction and need a scratch buffer for the partial results
+    need = lib.rz_forward_workspace_bytes(M, K, N, H, BLOCK_SIZE_K, BLOCK_SIZE_N, code)
+    ws = _lib.workspace(need, input.device)
+    _lib.check(lib.rz_forward_ws(
         x.data_ptr(), hw.data_ptr(), bias.data_ptr() if bias is not None else None, output.data_ptr(),
-        M, K, N, H, BLOCK_SIZE_K, BLOCK_SIZE_N,
-        _lib.hash_constants(R7, R6, R5, R4, R3, R2, R1, R0), float(init_factor), ldx, N,
-        _lib.dtype_code(input), stream))
+        ws.data_ptr() if need else None, need, M, K, N, H, BLOCK_SIZE_K, BLOCK_SIZE_N,
+        _lib.hash_constants(R7, R6, R5, R4, R3, R2, R1, R0), float(init_factor), ldx, N, code, stream))
     return output

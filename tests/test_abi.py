@@ -80,6 +80,14 @@ def test_status_codes(lib):
     assert lib.rz_weight_grad(one, one, one, None, 0, 8, 128, 128, 65536, 64, 64, _R(R1024), 1.0, 128, 128, 1,
                               None) == -7                         # bf16 needs the fp32 workspace
     assert lib.rz_materialize(one, one, 128, 128, 65536, 64, 64, _R(R1024), 2, 64, 0, None) == -2
+    # a skinny problem splits its contraction and then needs the workspace
+    need = lib.rz_forward_workspace_bytes(32, 10240, 1024, 65536, 64, 64, 0)
+    assert need > 0 and need % (32 * 1024 * 4) == 0
+    assert lib.rz_forward_workspace_bytes(4096, 4096, 4096, 65536, 64, 64, 1) == 0
+    assert lib.rz_forward_ws(one, one, None, one, None, 0, 32, 10240, 1024, 65536, 64, 64, _R(R1024), 1.0,
+                             10240, 1024, 0, None) == -7
+    assert lib.rz_input_grad_ws(one, one, one, None, 0, 32, 1024, 10240, 65536, 64, 64, _R(R1024), 1.0,
+                                10240, 1024, 0, None) == -7
     assert lib.rz_weight_grad_workspace_bytes(8, 128, 128, 65536, 64, 64, 0) == 0
     assert lib.rz_weight_grad_workspace_bytes(8, 128, 128, 65536, 64, 64, 1) == 65536 * 4
     for code in range(0, -10, -1):

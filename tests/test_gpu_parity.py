@@ -230,3 +230,27 @@ def test_function_apply_with_the_reference_six_arguments(oracle):
     torch.cuda.synchronize()
     assert rel_err(hw2.grad.cpu().numpy(), 2 * oracle.weight_grad(x64, dy64, H, BK, BN, R1024, 1.0)) <= 1e-4
     assert rel_err(x2.grad.cpu().numpy(), 2 * oracle.input_grad(dy64, hw64, K, BK, BN, R1024, 1.0)) <= 1e-4
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=lambda d: str(d).split(".")[-1])
+@pytest.mark.parametrize("shape", [(32, 2048, 1024, 70000, 32, 64), (100, 4096, 300, 20000, 64, 64),
+                                   (7, 2100, 520, 9000, 16, 32)], ids=lambda s: "x".join(map(str, s)))
+def test_skinny_problems_split_the_contraction(oracle, shape, dtype):
+    """Few output tiles and a long contraction: forward / input-grad cut it into slices with fp32
+    partial results (workspace) that a second kernel adds up, bias included."""
+    from rzlinear_amd import _lib
+    from rzlinear_amd.impl.RzLinearBackward import rz_linear_backward_input_grad_tl
+    from rzlinear_amd.impl.RzLinearForward import rz_linear_forward_bias_tl
+    M, K, N, H, BK, BN = shape
+    _say("split", shape, dtype)
+    lib = _lib.load()
+    code = _lib.dtype_code(torch.empty(0, dtype=dtype))
+    assert lib.rz_forward_workspace_bytes(M, K, N, H, BK, BN, code) > 0      # these shapes do split
+    (x, hw, dy), (x64, hw64, dy64) = make_inputs(M, K, N, H, dtype, seed=8)
+    bias = torch.randn(N, generator=torch.Generator().manual_seed(1)).to(dtype).cuda()
+    y = rz_linear_forward_bias_tl(x, hw, bias, 0.5, M, K, N, H, *rargs(R1024), BLOCK_SIZE_K=BK, BLOCK_SIZE_N=BN)
+    dx = rz_linear_backward_input_grad_tl(dy, hw, 0.5, M, K, N, H, *rargs(R1024), BLOCK_SIZE_K=BK, BLOCK_SIZE_N=BN)
+    torch.cuda.synchronize()
+    ref_y = oracle.forward(x64, hw64, N, BK, BN, R1024, 0.5) + bias.double().cpu().numpy()
+    assert rel_err(y.float().cpu().numpy(), ref_y) <= TOL[dtype]
+    assert rel_err(dx.float().cpu().numpy(), oracle.input_grad(dy64, hw64, K, BK, BN, R1024, 0.5)) <= TOL[dtype]
