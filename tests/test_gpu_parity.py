@@ -254,3 +254,34 @@ def test_skinny_problems_split_the_contraction(oracle, shape, dtype):
     ref_y = oracle.forward(x64, hw64, N, BK, BN, R1024, 0.5) + bias.double().cpu().numpy()
     assert rel_err(y.float().cpu().numpy(), ref_y) <= TOL[dtype]
     assert rel_err(dx.float().cpu().numpy(), oracle.input_grad(dy64, hw64, K, BK, BN, R1024, 0.5)) <= TOL[dtype]
+
+
+def _random_cases(n, seed):
+    rng = np.random.default_rng(seed)
+    cases = []
+    for _ in range(n):
+        BK, BN = (int(2 ** rng.integers(4, 9)) for _ in range(2))
+        M, K, N = (int(rng.integers(1, 700)) for _ in range(3))
+        if rng.random() < 0.3:      # complete tiles now and then, so the unchecked kernels run too
+            M, K, N = (int(rng.choice([64, 128, 256, 512])) for _ in range(3))
+        H = BK * BN + int(rng.integers(1, 60000))
+        cases.append((M, K, N, H, BK, BN))
+    return cases
+
+
+@pytest.mark.parametrize("shape", _random_cases(40, 2024), ids=lambda s: "x".join(map(str, s)))
+def test_random_shapes_fp32(oracle, shape):
+    """Seeded random shapes, tiles and hashed sizes: every tile family, checked and unchecked
+    kernels, split and unsplit contractions, LDS-image and atomic scatters get hit."""
+    from rzlinear_amd.impl.RzLinearBackward import rz_linear_backward_tl
+    from rzlinear_amd.impl.RzLinearForward import rz_linear_forward_tl
+    M, K, N, H, BK, BN = shape
+    _say("random", shape)
+    (x, hw, dy), (x64, hw64, dy64) = make_inputs(M, K, N, H, torch.float32, seed=M + K + N)
+    R = SEED_CONSTANTS[0]
+    y = rz_linear_forward_tl(x, hw, 1.5, M, K, N, H, *rargs(R), BLOCK_SIZE_K=BK, BLOCK_SIZE_N=BN)
+    dx, dhw = rz_linear_backward_tl(x, hw, dy, 1.5, M, K, N, H, *rargs(R), BLOCK_SIZE_K=BK, BLOCK_SIZE_N=BN)
+    torch.cuda.synchronize()
+    assert rel_err(y.cpu().numpy(), oracle.forward(x64, hw64, N, BK, BN, R, 1.5)) <= 1e-4
+    assert rel_err(dx.cpu().numpy(), oracle.input_grad(dy64, hw64, K, BK, BN, R, 1.5)) <= 1e-4
+    assert rel_err(dhw.cpu().numpy(), oracle.weight_grad(x64, dy64, H, BK, BN, R, 1.5)) <= 1e-4
