@@ -71,7 +71,8 @@ static hipError_t launch_op(int op, GemmParams p, const WeightGradPlan* plan, co
 
 // Tile shapes (all two LDS stages, software pipelined unless noted):
 //   256: 256 x 256, eight wavefronts of 128 x 64, one workgroup per compute unit
-//   128: 128 x 128, four wavefronts of 64 x 64, up to two workgroups per compute unit
+//   128: 128 x 128, four wavefronts of 64 x 64 (up to two workgroups per compute unit) or
+//        eight of 64 x 32 when there is about one workgroup per compute unit
 //    64:  64 x  64, four wavefronts of 32 x 32, for problems with few tiles
 // RZLINEAR_STAGES=1 selects a single-stage 128 x 128 form that leans on several workgroups
 // per compute unit instead of a pipeline (tuning aid).
@@ -87,6 +88,12 @@ static hipError_t launch_gemm_t(int op, GemmParams p, const WeightGradPlan* plan
     case 64: return launch_op<T, 64, 2, 2, 2>(op, p, plan, split, stream);
     case 128:
       if (one_stage) return launch_op<T, 128, 2, 2, 1>(op, p, plan, split, stream);
+      // with about one workgroup per compute unit, eight wavefronts (two per SIMD, 64 x 32
+      // each) hide latency better than four of 64 x 64; with more workgroups resident the
+      // four-wavefront form does less LDS traffic per flop
+      if (tile_count(p.I, p.J, 128) * (op == kWeightGrad && plan != nullptr ? plan->splits : 1) <=
+          kComputeUnits * 3 / 2)
+        return launch_op<T, 128, 2, 4, 2>(op, p, plan, split, stream);
       return launch_op<T, 128, 2, 2, 2>(op, p, plan, split, stream);
     default: return hipErrorInvalidValue;
   }

@@ -124,6 +124,7 @@ TILE_CASES = [
     (300, 200, 330, 9000, 32, 64),
     (256, 256, 512, 70000, 64, 64),      # H too large for the LDS image: global atomics
     (130, 70, 90, 2000, 16, 16),         # 16-wide tiles: LDS atomics inside the image
+    (2688, 192, 2432, 30000, 64, 64),    # > 384 tiles of 128: the four-wavefront 128 form
 ]
 
 
