@@ -146,6 +146,34 @@ int rz_weight_grad(const void* X, const void* dY, void* dHW, void* workspace,
                    void* stream);
 
 /*
+ * Weight gradient for training loops that own their gradient buffers, optionally with the
+ * bias gradient from the same pass over dY.
+ *   flags (bitwise or):
+ *     RZ_WG_ACCUMULATE  dHW += gradient instead of dHW = gradient.  Several layers may share one
+ *                       hashed_weight (python/rz_linear/RzLinear.py:54-58); accumulating here
+ *                       saves autograd's separate add over H and the clearing of dHW.
+ *     RZ_WG_DHW_F32     dHW is fp32 whatever `dtype` is (fp32 master gradients).
+ *     RZ_WG_DBIAS_F32   dbias is fp32 whatever `dtype` is.
+ *   dbias (may be NULL): dbias[N] = column sums of dY — the gradient of the bias that
+ *     python/rz_linear/RzLinear.py:93-94 adds, which autograd otherwise computes with a second
+ *     pass over dY.  Always overwritten; not scaled by init_factor (the bias is added after it).
+ *     The sums come from the dY tiles that the contraction stages anyway, in a fixed order.
+ * With flags = 0 and dbias = NULL this is rz_weight_grad.  The workspace size depends on the
+ * options: ask rz_weight_grad_ex_workspace_bytes with the same flags and with_dbias = (dbias != NULL).
+ * Extends rz_linear_backward_weight_grad_tl                           impl/RzLinearBackward.py:23-97,
+ * which always overwrites a fresh buffer of the input's dtype.
+ */
+#define RZ_WG_ACCUMULATE 1u
+#define RZ_WG_DHW_F32 2u
+#define RZ_WG_DBIAS_F32 4u
+size_t rz_weight_grad_ex_workspace_bytes(int M, int K, int N, int H, int BK, int BN, int dtype,
+                                         unsigned flags, int with_dbias);
+int rz_weight_grad_ex(const void* X, const void* dY, void* dHW, void* dbias, void* workspace,
+                      size_t workspace_bytes, int M, int K, int N, int H, int BK, int BN,
+                      const int32_t R[8], float init_factor, int64_t ldx, int64_t lddy, int dtype,
+                      unsigned flags, void* stream);
+
+/*
  * Materialise W[K,N] (row pitch ldw) from hashed_weight; edge tiles are clipped.
  * Replaces rz_linear_idx_tl                                           impl/RzLinearIdx.py:6-45
  * (kernel rz_linear_idx_kernel                                        impl/RzLinearIdx.py:48-77),

@@ -8,6 +8,7 @@ random_numbers, output_dim, chunk_size, init_factor)`` and a backward that hands
 import torch
 
 from .impl.RzLinearBackward import (rz_linear_backward_input_grad_tl,
+                                    rz_linear_backward_weight_bias_grad_tl,
                                     rz_linear_backward_weight_grad_tl)
 from .impl.RzLinearForward import rz_linear_forward_bias_tl
 
@@ -79,9 +80,12 @@ class RzLinearFunction(torch.autograd.Function):
         if need_input:      # enqueued first, like the reference's rz_linear_backward_tl
             input_grad = rz_linear_backward_input_grad_tl(grad, hashed_weight.data, ctx.init_factor,
                                                           M, K, N, H, *consts, **kwargs)
-        if need_weight:
+        if need_weight and need_bias:   # one pass over grad yields both
+            weight_grad, bias_grad = rz_linear_backward_weight_bias_grad_tl(input, grad, ctx.init_factor,
+                                                                            M, K, N, H, *consts, **kwargs)
+        elif need_weight:
             weight_grad = rz_linear_backward_weight_grad_tl(input, grad, ctx.init_factor,
                                                             M, K, N, H, *consts, **kwargs)
-        if need_bias:
+        elif need_bias:
             bias_grad = grad.sum(dim=0)
         return input_grad, weight_grad, None, None, None, None, None, None, bias_grad

@@ -20,7 +20,8 @@ _DTYPES = {torch.float32: RZ_F32, torch.bfloat16: RZ_BF16, torch.float16: RZ_F16
 EXPORTS = (
     "rz_version", "rz_status_string", "rz_tile_offsets", "rz_tile_offsets_device", "rz_forward",
     "rz_forward_bias", "rz_forward_workspace_bytes", "rz_forward_ws", "rz_input_grad",
-    "rz_input_grad_workspace_bytes", "rz_input_grad_ws", "rz_weight_grad_workspace_bytes", "rz_weight_grad", "rz_materialize",
+    "rz_input_grad_workspace_bytes", "rz_input_grad_ws", "rz_weight_grad_workspace_bytes", "rz_weight_grad", "rz_weight_grad_ex_workspace_bytes",
+    "rz_weight_grad_ex", "rz_materialize",
 )
 
 _lib = None
@@ -77,11 +78,20 @@ def load():
     lib.rz_weight_grad.restype = c_int
     lib.rz_weight_grad.argtypes = [c_vp, c_vp, c_vp, c_vp, c_sz, c_int, c_int, c_int, c_int, c_int, c_int,
                                    i32p, c_f, c_i64, c_i64, c_int, c_vp]
+    lib.rz_weight_grad_ex_workspace_bytes.restype = c_sz
+    lib.rz_weight_grad_ex_workspace_bytes.argtypes = [c_int] * 7 + [ctypes.c_uint, c_int]
+    lib.rz_weight_grad_ex.restype = c_int
+    lib.rz_weight_grad_ex.argtypes = [c_vp, c_vp, c_vp, c_vp, c_vp, c_sz, c_int, c_int, c_int, c_int, c_int, c_int,
+                                      i32p, c_f, c_i64, c_i64, c_int, ctypes.c_uint, c_vp]
     lib.rz_materialize.restype = c_int
     lib.rz_materialize.argtypes = [c_vp, c_vp, c_int, c_int, c_int, c_int, c_int, i32p, c_int, c_i64,
                                    c_int, c_vp]
     _lib = lib
     return lib
+
+
+# options of rz_weight_grad_ex
+WG_ACCUMULATE, WG_DHW_F32, WG_DBIAS_F32 = 1, 2, 4
 
 
 def check(status):

@@ -100,17 +100,18 @@ __global__ void fill_zero_kernel(uint32_t* p, size_t words) {
   for (; i < words; i += stride) p[i] = 0u;
 }
 
-template <typename T>
+// dst[i] = src[i] (+ dst[i] when ACC), converted to the element type.
+template <typename T, bool ACC>
 __global__ void convert_from_f32_kernel(const float* __restrict__ src, T* __restrict__ dst, int n) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < n) dst[i] = ElemTraits<T>::from_float(src[i]);
+  if (i < n) dst[i] = ElemTraits<T>::from_float(src[i] + (ACC ? ElemTraits<T>::to_float(dst[i]) : 0.f));
 }
 
-// dHW[h] = sum over the partial images of part[p][h], converted to the element type.  A
-// workgroup of 256 threads owns 16 groups of four slots; 16 thread groups each add up every
-// 16th partial image, then the groups are combined through LDS in a fixed order, so the
-// result does not depend on scheduling.
-template <typename T>
+// dHW[h] = sum over the partial images of part[p][h] (+ dHW[h] when ACC), converted to the
+// element type.  A workgroup of 256 threads owns 16 groups of four slots; 16 thread groups each
+// add up every 16th partial image, then the groups are combined through LDS in a fixed order,
+// so the result does not depend on scheduling.
+template <typename T, bool ACC>
 __global__ __launch_bounds__(256) void reduce_partials_kernel(const float* __restrict__ part,
                                                               T* __restrict__ out, int H, int pitch,
                                                               int nparts) {
@@ -136,8 +137,28 @@ __global__ __launch_bounds__(256) void reduce_partials_kernel(const float* __res
     const float r[4] = {s.x, s.y, s.z, s.w};
 #pragma unroll
     for (int e = 0; e < 4; e++)
-      if (slot + e < H) out[slot + e] = ElemTraits<T>::from_float(r[e]);
+      if (slot + e < H)
+        out[slot + e] = ElemTraits<T>::from_float(r[e] + (ACC ? ElemTraits<T>::to_float(out[slot + e]) : 0.f));
   }
+}
+
+// dbias[n] = sum over the rows of part[row][n], converted to the element type.  A workgroup owns
+// 64 columns; four thread groups each add up every fourth row (eight loads in flight), then
+// the groups are combined through LDS in a fixed order.
+template <typename T>
+__global__ __launch_bounds__(256) void reduce_colsum_kernel(const float* __restrict__ part,
+                                                            T* __restrict__ out, int N, int pitch, int rows) {
+  __shared__ float sums[4][64];
+  const int c = threadIdx.x & 63, g = threadIdx.x >> 6;
+  const int n = blockIdx.x * 64 + c;
+  float s = 0.f;
+  if (n < N) {
+#pragma unroll 8
+    for (int r = g; r < rows; r += 4) s += part[(size_t)r * pitch + n];
+  }
+  sums[g][c] = s;
+  __syncthreads();
+  if (g == 0 && n < N) out[n] = ElemTraits<T>::from_float((sums[0][c] + sums[1][c]) + (sums[2][c] + sums[3][c]));
 }
 
 // C[i][j] = sum over the slices of part[s][i][j] (+ bias[j]), converted to the element type.
@@ -203,6 +224,113 @@ static hipError_t zero_words(void* p, size_t bytes, hipStream_t s) {
   if (blocks > 4096) blocks = 4096;
   hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)blocks), dim3(256), 0, s, (uint32_t*)p, words);
   return hipGetLastError();
+}
+
+// Launchers over the output element type (an rz_dtype code) of the weight-grad tail kernels.
+template <bool ACC>
+static void launch_reduce_partials(int out_dtype, const float* part, void* out, int H, int pitch, int nparts,
+                                   hipStream_t s) {
+  const dim3 grid((pitch / 4 + 15) / 16), block(256);
+  if (out_dtype == RZ_F32)
+    hipLaunchKernelGGL((reduce_partials_kernel<float, ACC>), grid, block, 0, s, part, (float*)out, H, pitch, nparts);
+  else if (out_dtype == RZ_BF16)
+    hipLaunchKernelGGL((reduce_partials_kernel<bf16_t, ACC>), grid, block, 0, s, part, (bf16_t*)out, H, pitch, nparts);
+  else
+    hipLaunchKernelGGL((reduce_partials_kernel<f16_t, ACC>), grid, block, 0, s, part, (f16_t*)out, H, pitch, nparts);
+}
+
+template <bool ACC>
+static void launch_convert(int out_dtype, const float* src, void* dst, int n, hipStream_t s) {
+  const dim3 grid((n + 255) / 256), block(256);
+  if (out_dtype == RZ_BF16)
+    hipLaunchKernelGGL((convert_from_f32_kernel<bf16_t, ACC>), grid, block, 0, s, src, (bf16_t*)dst, n);
+  else if (out_dtype == RZ_F16)
+    hipLaunchKernelGGL((convert_from_f32_kernel<f16_t, ACC>), grid, block, 0, s, src, (f16_t*)dst, n);
+  else
+    hipLaunchKernelGGL((convert_from_f32_kernel<float, ACC>), grid, block, 0, s, src, (float*)dst, n);
+}
+
+static void launch_reduce_colsum(int out_dtype, const float* part, void* out, int N, int pitch, int rows,
+                                 hipStream_t s) {
+  const dim3 grid((N + 63) / 64), block(256);
+  if (out_dtype == RZ_F32)
+    hipLaunchKernelGGL(reduce_colsum_kernel<float>, grid, block, 0, s, part, (float*)out, N, pitch, rows);
+  else if (out_dtype == RZ_BF16)
+    hipLaunchKernelGGL(reduce_colsum_kernel<bf16_t>, grid, block, 0, s, part, (bf16_t*)out, N, pitch, rows);
+  else
+    hipLaunchKernelGGL(reduce_colsum_kernel<f16_t>, grid, block, 0, s, part, (f16_t*)out, N, pitch, rows);
+}
+
+static inline size_t round256(size_t b) { return (b + 255) & ~(size_t)255; }
+
+// Workspace layout of a weight-grad call: [main][column sums].  main = the partial images (LDS
+// image mode) or, for the atomic scatter into a 16-bit dHW, its fp32 image.
+struct WeightGradWorkspace {
+  size_t main_bytes, total_bytes;
+};
+static WeightGradWorkspace weight_grad_workspace(const WeightGradPlan& plan, int H, bool dhw_f32, bool with_dbias) {
+  WeightGradWorkspace w;
+  if (plan.image_pitch > 0) w.main_bytes = plan.workspace_bytes;
+  else w.main_bytes = dhw_f32 ? 0 : round256((size_t)H * sizeof(float));
+  w.total_bytes = w.main_bytes + (with_dbias ? plan.colsum_bytes : 0);
+  return w;
+}
+
+// dHW (and optionally dbias) of one layer; see rz_weight_grad_ex in the header.
+static int weight_grad_impl(const void* X, const void* dY, void* dHW, void* dbias, void* workspace,
+                            size_t workspace_bytes, int M, int K, int N, int H, int BK, int BN,
+                            const int32_t R[8], float init_factor, int64_t ldx, int64_t lddy, int dtype,
+                            unsigned flags, void* stream) {
+  if (X == nullptr || dY == nullptr || dHW == nullptr) return RZ_ERR_NULL_POINTER;
+  if (dtype_bytes(dtype) == 0) return RZ_ERR_BAD_DTYPE;
+  if (M < 1 || ldx < K || lddy < N) return RZ_ERR_BAD_SHAPE;
+  if (flags & ~(unsigned)(RZ_WG_ACCUMULATE | RZ_WG_DHW_F32 | RZ_WG_DBIAS_F32)) return RZ_ERR_BAD_ARGUMENT;
+  GemmParams p = {};
+  int st = make_hash(&p.h, K, N, H, BK, BN, R, 2);
+  if (st != RZ_OK) return st;
+  const bool accumulate = (flags & RZ_WG_ACCUMULATE) != 0;
+  const int dhw_dtype = (flags & RZ_WG_DHW_F32) ? RZ_F32 : dtype;
+  const int dbias_dtype = (flags & RZ_WG_DBIAS_F32) ? RZ_F32 : dtype;
+  const WeightGradPlan plan = plan_weight_grad(M, K, N, H, dtype_bytes(dtype));
+  const WeightGradWorkspace ws = weight_grad_workspace(plan, H, dhw_dtype == RZ_F32, dbias != nullptr);
+  if (ws.total_bytes > 0 && (workspace == nullptr || workspace_bytes < ws.total_bytes)) return RZ_ERR_WORKSPACE;
+  hipStream_t s = (hipStream_t)stream;
+  p.A = X;
+  p.B = dY;
+  p.I = K;
+  p.J = N;
+  p.R = M;
+  p.lda = ldx;
+  p.ldb = lddy;
+  p.scale = init_factor;
+  if (dbias != nullptr) p.colsum = reinterpret_cast<float*>(static_cast<char*>(workspace) + ws.main_bytes);
+  if (plan.image_pitch > 0) {
+    // every workgroup sums its tiles into an LDS image of dHW and stores it as a partial image;
+    // the partial images are then added up (no global atomics, fixed summation order)
+    p.scatter = (float*)workspace;
+    if (launch_gemm(dtype, kWeightGrad, p, &plan, nullptr, s) != hipSuccess) return RZ_ERR_LAUNCH;
+    if (accumulate) launch_reduce_partials<true>(dhw_dtype, p.scatter, dHW, H, plan.image_pitch, (int)plan.workgroups, s);
+    else launch_reduce_partials<false>(dhw_dtype, p.scatter, dHW, H, plan.image_pitch, (int)plan.workgroups, s);
+  } else {
+    // hashed_weight too large for an LDS image: tiles go to an fp32 image of dHW by global
+    // atomics; an fp32 dHW is its own image (and, accumulating, needs no clearing)
+    float* image = (dhw_dtype == RZ_F32) ? (float*)dHW : (float*)workspace;
+    if (!(accumulate && dhw_dtype == RZ_F32) &&
+        zero_words(image, (size_t)H * sizeof(float), s) != hipSuccess)
+      return RZ_ERR_LAUNCH;
+    p.scatter = image;
+    if (launch_gemm(dtype, kWeightGrad, p, &plan, nullptr, s) != hipSuccess) return RZ_ERR_LAUNCH;
+    if (dhw_dtype != RZ_F32) {
+      if (accumulate) launch_convert<true>(dhw_dtype, image, dHW, H, s);
+      else launch_convert<false>(dhw_dtype, image, dHW, H, s);
+    }
+  }
+  if (hipGetLastError() != hipSuccess) return RZ_ERR_LAUNCH;
+  if (dbias != nullptr) {
+    launch_reduce_colsum(dbias_dtype, p.colsum, dbias, N, plan.colsum_pitch, plan.colsum_rows, s);
+    if (hipGetLastError() != hipSuccess) return RZ_ERR_LAUNCH;
+  }
+  return RZ_OK;
 }
 
 }  // namespace rz
@@ -353,65 +481,33 @@ RZ_API int rz_input_grad_ws(const void* dY, const void* HW, void* dX, void* work
 }
 
 RZ_API size_t rz_weight_grad_workspace_bytes(int M, int K, int N, int H, int BK, int BN, int dtype) {
-  (void)BK; (void)BN;
-  const int eb = dtype_bytes(dtype);
-  if (eb == 0 || M < 1 || K < 1 || N < 1 || H < 1) return 0;
-  return plan_weight_grad(M, K, N, H, eb).workspace_bytes;
+  return rz_weight_grad_ex_workspace_bytes(M, K, N, H, BK, BN, dtype, 0u, 0);
 }
 
 RZ_API int rz_weight_grad(const void* X, const void* dY, void* dHW, void* workspace,
                           size_t workspace_bytes, int M, int K, int N, int H, int BK, int BN,
                           const int32_t R[8], float init_factor, int64_t ldx, int64_t lddy,
                           int dtype, void* stream) {
-  if (X == nullptr || dY == nullptr || dHW == nullptr) return RZ_ERR_NULL_POINTER;
-  if (dtype_bytes(dtype) == 0) return RZ_ERR_BAD_DTYPE;
-  if (M < 1 || ldx < K || lddy < N) return RZ_ERR_BAD_SHAPE;
-  GemmParams p = {};
-  int st = make_hash(&p.h, K, N, H, BK, BN, R, 2);
-  if (st != RZ_OK) return st;
-  const WeightGradPlan plan = plan_weight_grad(M, K, N, H, dtype_bytes(dtype));
-  if (plan.workspace_bytes > 0 && (workspace == nullptr || workspace_bytes < plan.workspace_bytes))
-    return RZ_ERR_WORKSPACE;
-  hipStream_t s = (hipStream_t)stream;
-  p.A = X;
-  p.B = dY;
-  p.I = K;
-  p.J = N;
-  p.R = M;
-  p.lda = ldx;
-  p.ldb = lddy;
-  p.scale = init_factor;
-  if (plan.image_pitch > 0) {
-    // every workgroup sums its tiles into an LDS image of dHW and stores it as a partial image;
-    // the partial images are then added up (no global atomics, fixed summation order)
-    p.scatter = (float*)workspace;
-    if (launch_gemm(dtype, kWeightGrad, p, &plan, nullptr, s) != hipSuccess) return RZ_ERR_LAUNCH;
-    const int blocks = (plan.image_pitch / 4 + 15) / 16;
-    const int nparts = (int)plan.workgroups;
-    if (dtype == RZ_F32)
-      hipLaunchKernelGGL(reduce_partials_kernel<float>, dim3(blocks), dim3(256), 0, s, p.scatter,
-                         (float*)dHW, H, plan.image_pitch, nparts);
-    else if (dtype == RZ_BF16)
-      hipLaunchKernelGGL(reduce_partials_kernel<bf16_t>, dim3(blocks), dim3(256), 0, s, p.scatter,
-                         (bf16_t*)dHW, H, plan.image_pitch, nparts);
-    else
-      hipLaunchKernelGGL(reduce_partials_kernel<f16_t>, dim3(blocks), dim3(256), 0, s, p.scatter,
-                         (f16_t*)dHW, H, plan.image_pitch, nparts);
-    return hipGetLastError() == hipSuccess ? RZ_OK : RZ_ERR_LAUNCH;
-  }
-  // hashed_weight too large for an LDS image: tiles go to an fp32 image of dHW by global atomics
-  float* image = (dtype == RZ_F32) ? (float*)dHW : (float*)workspace;
-  if (zero_words(image, (size_t)H * sizeof(float), s) != hipSuccess) return RZ_ERR_LAUNCH;
-  p.scatter = image;
-  if (launch_gemm(dtype, kWeightGrad, p, &plan, nullptr, s) != hipSuccess) return RZ_ERR_LAUNCH;
-  if (dtype == RZ_BF16) {
-    hipLaunchKernelGGL(convert_from_f32_kernel<bf16_t>, dim3((H + 255) / 256), dim3(256), 0, s, image,
-                       (bf16_t*)dHW, H);
-  } else if (dtype == RZ_F16) {
-    hipLaunchKernelGGL(convert_from_f32_kernel<f16_t>, dim3((H + 255) / 256), dim3(256), 0, s, image,
-                       (f16_t*)dHW, H);
-  }
-  return hipGetLastError() == hipSuccess ? RZ_OK : RZ_ERR_LAUNCH;
+  return weight_grad_impl(X, dY, dHW, nullptr, workspace, workspace_bytes, M, K, N, H, BK, BN, R,
+                          init_factor, ldx, lddy, dtype, 0u, stream);
+}
+
+RZ_API size_t rz_weight_grad_ex_workspace_bytes(int M, int K, int N, int H, int BK, int BN, int dtype,
+                                                unsigned flags, int with_dbias) {
+  (void)BK; (void)BN;
+  const int eb = dtype_bytes(dtype);
+  if (eb == 0 || M < 1 || K < 1 || N < 1 || H < 1) return 0;
+  const WeightGradPlan plan = plan_weight_grad(M, K, N, H, eb);
+  const bool dhw_f32 = (flags & RZ_WG_DHW_F32) != 0 || dtype == RZ_F32;
+  return weight_grad_workspace(plan, H, dhw_f32, with_dbias != 0).total_bytes;
+}
+
+RZ_API int rz_weight_grad_ex(const void* X, const void* dY, void* dHW, void* dbias, void* workspace,
+                             size_t workspace_bytes, int M, int K, int N, int H, int BK, int BN,
+                             const int32_t R[8], float init_factor, int64_t ldx, int64_t lddy,
+                             int dtype, unsigned flags, void* stream) {
+  return weight_grad_impl(X, dY, dHW, dbias, workspace, workspace_bytes, M, K, N, H, BK, BN, R,
+                          init_factor, ldx, lddy, dtype, flags, stream);
 }
 
 RZ_API int rz_materialize(const void* HW, void* W, int K, int N, int H, int BK, int BN,

@@ -100,6 +100,9 @@ struct GemmParams {
   float* scatter;     // weight-grad target: fp32 image of dHW (direct atomics), or the
                       // per-workgroup partial images [workgroups][image_pitch] (LDS mode)
   int image_pitch;    // > 0 selects the LDS mode: floats per partial image (H rounded up to 4)
+  float* colsum;      // weight-grad that also yields the bias gradient: partial column sums of B
+                      // (dY), one row per (slice, tile row): [slices * tiles_i][colsum_pitch]
+  int colsum_pitch;   // floats per row of colsum (J rounded up to the tile)
   int I, J, R;
   int64_t lda, ldb, ldc;
   int tiles_i, tiles_j;

@@ -100,8 +100,10 @@ __device__ __forceinline__ u32x4_t mask_tail(u32x4_t v, int col, int col_lim) {
   return v;
 }
 
-template <typename T, int OP, int TI, int TJ, int WI, int WJ, int NSTAGE, bool FULL>
+// COLSUM (weight-grad only): also sum the columns of B (dY) for the bias gradient.
+template <typename T, int OP, int TI, int TJ, int WI, int WJ, int NSTAGE, bool FULL, bool COLSUM = false>
 struct GemmKernel {
+  static_assert(!COLSUM || OP == kWeightGrad, "column sums belong to the weight-grad contraction");
   typedef ElemTraits<T> Tr;
   typedef typename Mfma<T>::Frag Frag;
   static constexpr int kThreads = 64 * WI * WJ;
@@ -266,6 +268,16 @@ struct GemmKernel {
 
     u32x4_t ra[LA::kPieces], rb[LB::kPieces];
 
+    // Bias gradient (COLSUM): the tiles_i workgroups of one tile column and slice stage the same
+    // rows of dY, so they take turns: the workgroup whose turn it is adds the rows of that R
+    // step, from the registers on their way into LDS, into per-thread column sums.  A thread's
+    // pieces sit in one 16-byte column position, so VEC sums per thread suffice.
+    static_assert(!COLSUM || kThreads % LB::kCpr == 0, "a thread's pieces must share their columns");
+    float colsum[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; e++) colsum[e] = 0.f;
+    int colsum_turn = COLSUM ? (r_begin / TR) % p.tiles_i : 0;
+
     auto window = [&](int step) -> OffWindow {
       const int r0 = r_begin + step * TR;
       if constexpr (OP == kForward) return off_window(p.h, r0, TR, j0, TJ);
@@ -353,6 +365,19 @@ struct GemmKernel {
 #pragma unroll
       for (int q = 0; q < LB::kPieces; q++)
         lds_put<B_LAYOUT, LB>(sm.b[st], piece_row(LB{}, q), piece_cc(LB{}, q), rb[q]);
+      if constexpr (COLSUM) {
+        // commits happen once per R step, in step order
+        if (colsum_turn == ti) {
+#pragma unroll
+          for (int q = 0; q < LB::kPieces; q++) {
+            T elems[VEC];
+            __builtin_memcpy(elems, &rb[q], 16);
+#pragma unroll
+            for (int e = 0; e < VEC; e++) colsum[e] += Tr::to_float(elems[e]);
+          }
+        }
+        colsum_turn = (colsum_turn + 1 == p.tiles_i) ? 0 : colsum_turn + 1;
+      }
     };
     // MFMAs of one R step out of LDS stage `st`; fragments are read one sub-step ahead
     auto compute = [&](int st) {
@@ -497,6 +522,20 @@ struct GemmKernel {
       const bool image_mode = p.image_pitch > 0;
       float* image = reinterpret_cast<float*>(&sm);   // aliases the operand stages
       __syncthreads();                                 // every wavefront is done reading them
+      if constexpr (COLSUM) {
+        // combine the threads that share columns (fixed order), one row of partial sums out
+        constexpr int kGroups = kThreads / LB::kCpr;
+        static_assert(sizeof(float) * kGroups * TJ <= sizeof(Smem), "column sums must fit the stages");
+#pragma unroll
+        for (int e = 0; e < VEC; e++) image[(tid / LB::kCpr) * TJ + (tid % LB::kCpr) * VEC + e] = colsum[e];
+        __syncthreads();
+        for (int c = tid; c < TJ; c += kThreads) {
+          float s = 0.f;
+          for (int g = 0; g < kGroups; g++) s += image[g * TJ + c];
+          p.colsum[((size_t)blockIdx.y * p.tiles_i + ti) * (size_t)p.colsum_pitch + j0 + c] = s;
+        }
+        __syncthreads();
+      }
       if (image_mode) {
         const float4 z = {0.f, 0.f, 0.f, 0.f};
         for (int i = tid * 4; i < p.image_pitch; i += kThreads * 4) *reinterpret_cast<float4*>(image + i) = z;
@@ -637,9 +676,9 @@ struct GemmKernel {
   }
 };
 
-template <typename T, int OP, int TI, int TJ, int WI, int WJ, int NSTAGE, bool FULL>
+template <typename T, int OP, int TI, int TJ, int WI, int WJ, int NSTAGE, bool FULL, bool COLSUM>
 __global__ __launch_bounds__(64 * WI * WJ) void rz_gemm_kernel(GemmParams p) {
-  typedef GemmKernel<T, OP, TI, TJ, WI, WJ, NSTAGE, FULL> K;
+  typedef GemmKernel<T, OP, TI, TJ, WI, WJ, NSTAGE, FULL, COLSUM> K;
   extern __shared__ __attribute__((aligned(16))) unsigned char rz_smem_raw[];
   K::run(p, *reinterpret_cast<typename K::Smem*>(rz_smem_raw));
 }

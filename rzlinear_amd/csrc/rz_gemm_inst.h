@@ -6,10 +6,10 @@
 
 namespace rz {
 
-template <typename T, int OP, int TI, int TJ, int WI, int WJ, int NSTAGE, bool FULL>
+template <typename T, int OP, int TI, int TJ, int WI, int WJ, int NSTAGE, bool FULL, bool COLSUM>
 static hipError_t launch_one(GemmParams p, const WeightGradPlan* plan, const SplitPlan* split,
                              hipStream_t stream) {
-  typedef GemmKernel<T, OP, TI, TJ, WI, WJ, NSTAGE, FULL> K;
+  typedef GemmKernel<T, OP, TI, TJ, WI, WJ, NSTAGE, FULL, COLSUM> K;
   p.tiles_i = (p.I + TI - 1) / TI;
   p.tiles_j = (p.J + TJ - 1) / TJ;
   const long long tiles = (long long)p.tiles_i * p.tiles_j;
@@ -22,6 +22,12 @@ static hipError_t launch_one(GemmParams p, const WeightGradPlan* plan, const Spl
     p.r_chunk = plan->r_chunk;
     p.image_pitch = plan->image_pitch;
     if ((size_t)p.image_pitch * sizeof(float) > kMaxImageBytes) return hipErrorInvalidValue;
+    if (COLSUM) {
+      if (p.colsum == nullptr || plan->colsum_pitch != p.tiles_j * TJ ||
+          plan->colsum_rows != plan->splits * p.tiles_i)
+        return hipErrorInvalidValue;
+      p.colsum_pitch = plan->colsum_pitch;
+    }
   } else if (split != nullptr && split->splits > 1) {
     if (split->tile != TI || p.partial == nullptr) return hipErrorInvalidValue;
     splits = split->splits;
@@ -30,7 +36,7 @@ static hipError_t launch_one(GemmParams p, const WeightGradPlan* plan, const Spl
     p.r_chunk = r_steps * K::TR;
     p.partial = nullptr;
   }
-  auto kernel = rz_gemm_kernel<T, OP, TI, TJ, WI, WJ, NSTAGE, FULL>;
+  auto kernel = rz_gemm_kernel<T, OP, TI, TJ, WI, WJ, NSTAGE, FULL, COLSUM>;
   size_t smem = sizeof(typename K::Smem);
   static_assert(sizeof(typename K::Smem) <= 160 * 1024, "tile does not fit the 160 KB LDS of a compute unit");
   if (OP == kWeightGrad && p.image_pitch > 0) {
@@ -49,13 +55,13 @@ static hipError_t launch_one(GemmParams p, const WeightGradPlan* plan, const Spl
 }
 
 // FULL kernels carry no bounds checks: every tile and every R step must be complete.
-template <typename T, int OP, int TILE, int WI, int WJ, int NSTAGE>
+template <typename T, int OP, int TILE, int WI, int WJ, int NSTAGE, bool COLSUM = false>
 static hipError_t launch_tile(GemmParams p, const WeightGradPlan* plan, const SplitPlan* split,
                               hipStream_t stream) {
   constexpr int TR = 128 / ElemTraits<T>::kBytes;
   const bool full = (p.I % TILE == 0) && (p.J % TILE == 0) && (p.R % TR == 0);
-  if (full) return launch_one<T, OP, TILE, TILE, WI, WJ, NSTAGE, true>(p, plan, split, stream);
-  return launch_one<T, OP, TILE, TILE, WI, WJ, NSTAGE, false>(p, plan, split, stream);
+  if (full) return launch_one<T, OP, TILE, TILE, WI, WJ, NSTAGE, true, COLSUM>(p, plan, split, stream);
+  return launch_one<T, OP, TILE, TILE, WI, WJ, NSTAGE, false, COLSUM>(p, plan, split, stream);
 }
 
 template <typename T, int TILE, int WI, int WJ, int NSTAGE>
@@ -64,7 +70,10 @@ static hipError_t launch_op(int op, GemmParams p, const WeightGradPlan* plan, co
   switch (op) {
     case kForward: return launch_tile<T, kForward, TILE, WI, WJ, NSTAGE>(p, plan, split, stream);
     case kInputGrad: return launch_tile<T, kInputGrad, TILE, WI, WJ, NSTAGE>(p, plan, split, stream);
-    case kWeightGrad: return launch_tile<T, kWeightGrad, TILE, WI, WJ, NSTAGE>(p, plan, split, stream);
+    case kWeightGrad:
+      // with a column-sum target the kernel also produces the bias gradient's partial sums
+      if (p.colsum != nullptr) return launch_tile<T, kWeightGrad, TILE, WI, WJ, NSTAGE, true>(p, plan, split, stream);
+      return launch_tile<T, kWeightGrad, TILE, WI, WJ, NSTAGE>(p, plan, split, stream);
     default: return hipErrorInvalidValue;
   }
 }

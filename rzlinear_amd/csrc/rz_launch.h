@@ -75,7 +75,11 @@ struct WeightGradPlan {
   int image_pitch;   // > 0: every workgroup first sums its tiles into an fp32 image of dHW held
                      // in LDS and stores it as one partial image; a second kernel adds the
                      // partial images up.  0: tiles go to dHW by global atomics.
-  size_t workspace_bytes;
+  size_t workspace_bytes;   // partial images, or the fp32 image for the atomics (16-bit dHW)
+  // bias gradient computed in the same pass: partial column sums of dY, one row per
+  // (slice, tile row), stored behind the first `workspace_bytes` of the workspace
+  int colsum_rows, colsum_pitch;
+  size_t colsum_bytes;
 };
 
 // LDS bytes of a compute unit that an fp32 image of dHW may take (the rest holds the small
@@ -119,7 +123,10 @@ static inline WeightGradPlan plan_weight_grad(int M, int K, int N, int H, int el
   size_t ws = 0;
   if (pl.image_pitch > 0) ws = (size_t)pl.workgroups * pl.image_pitch * sizeof(float);
   else if (elem_bytes == 2) ws = (size_t)H * sizeof(float);   // fp32 image for the atomics
-  pl.workspace_bytes = ws;
+  pl.workspace_bytes = (ws + 255) & ~(size_t)255;
+  pl.colsum_rows = pl.splits * ((K + pl.tile - 1) / pl.tile);
+  pl.colsum_pitch = ((N + pl.tile - 1) / pl.tile) * pl.tile;
+  pl.colsum_bytes = (size_t)pl.colsum_rows * pl.colsum_pitch * sizeof(float);
   return pl;
 }
 

@@ -27,19 +27,9 @@ def rz_linear_backward_tl(input: torch.Tensor, hashed_weight: torch.Tensor, outp
     return input_grad, weight_grad
 
 
-def rz_linear_backward_weight_grad_tl(input: torch.Tensor, output_grad: torch.Tensor, init_factor: float,
-                                      M: int, K: int, N: int, H: int,
-                                      R7: int, R6: int, R5: int, R4: int,
-                                      R3: int, R2: int, R1: int, R0: int,
-                                      allow_tf32: bool = True, allow_autotune: bool = True,
-                                      BLOCK_SIZE_M: int = 64, BLOCK_SIZE_N: int = 64, BLOCK_SIZE_K: int = 32,
-                                      GROUP_SIZE: int = 8) -> torch.Tensor:
-    """hashed_weight_grad[H] = scatter_add over W tiles of (input^T . output_grad) * init_factor.
-
-    Same signature as the reference launcher (python/rz_linear/impl/RzLinearBackward.py:23-97);
-    the result has output_grad's dtype.  The tiles are reduced and scattered in fp32 whatever the
-    dtype (the reference adds atomically in output_grad's dtype), then converted once.
-    """
+def _weight_grad(input, output_grad, init_factor, M, K, N, H, R, BLOCK_SIZE_K, BLOCK_SIZE_N,
+                 out=None, accumulate=False, with_bias_grad=False):
+    """One rz_weight_grad_ex call; returns (hashed_weight_grad, bias_grad or None)."""
     stream = _lib.require_gpu(input, output_grad)
     if input.dtype != output_grad.dtype:
         raise TypeError("input is %s but output_grad is %s" % (input.dtype, output_grad.dtype))
@@ -47,14 +37,73 @@ def rz_linear_backward_weight_grad_tl(input: torch.Tensor, output_grad: torch.Te
     x, ldx = _lib.rows(input)
     dy, lddy = _lib.rows(output_grad)
     code = _lib.dtype_code(output_grad)
-    hashed_weight_grad = torch.empty((H,), device=output_grad.device, dtype=output_grad.dtype)
-    need = lib.rz_weight_grad_workspace_bytes(M, K, N, H, BLOCK_SIZE_K, BLOCK_SIZE_N, code)
-    workspace = torch.empty((max(need, 1),), device=output_grad.device, dtype=torch.uint8) if need else None
-    _lib.check(lib.rz_weight_grad(
-        x.data_ptr(), dy.data_ptr(), hashed_weight_grad.data_ptr(),
-        workspace.data_ptr() if need else None, need, M, K, N, H, BLOCK_SIZE_K, BLOCK_SIZE_N,
-        _lib.hash_constants(R7, R6, R5, R4, R3, R2, R1, R0), float(init_factor), ldx, lddy, code, stream))
-    return hashed_weight_grad
+    flags = 0
+    if out is None:
+        if accumulate:
+            raise ValueError("accumulate=True needs the buffer to add into (out=...)")
+        out = torch.empty((H,), device=output_grad.device, dtype=output_grad.dtype)
+    else:
+        _lib.require_gpu(output_grad, out)
+        if out.shape != (H,) or not out.is_contiguous():
+            raise ValueError("out must be a contiguous tensor of %d elements" % H)
+        if out.dtype == torch.float32:
+            flags |= _lib.WG_DHW_F32
+        elif out.dtype != output_grad.dtype:
+            raise TypeError("out must be float32 or %s, got %s" % (output_grad.dtype, out.dtype))
+        if accumulate:
+            flags |= _lib.WG_ACCUMULATE
+    bias_grad = torch.empty((N,), device=output_grad.device, dtype=output_grad.dtype) if with_bias_grad else None
+    need = lib.rz_weight_grad_ex_workspace_bytes(M, K, N, H, BLOCK_SIZE_K, BLOCK_SIZE_N, code, flags,
+                                                 int(with_bias_grad))
+    ws = _lib.workspace(need, output_grad.device)
+    _lib.check(lib.rz_weight_grad_ex(
+        x.data_ptr(), dy.data_ptr(), out.data_ptr(), bias_grad.data_ptr() if with_bias_grad else None,
+        ws.data_ptr() if need else None, need, M, K, N, H, BLOCK_SIZE_K, BLOCK_SIZE_N, R,
+        float(init_factor), ldx, lddy, code, flags, stream))
+    return out, bias_grad
+
+
+def rz_linear_backward_weight_grad_tl(input: torch.Tensor, output_grad: torch.Tensor, init_factor: float,
+                                      M: int, K: int, N: int, H: int,
+                                      R7: int, R6: int, R5: int, R4: int,
+                                      R3: int, R2: int, R1: int, R0: int,
+                                      allow_tf32: bool = True, allow_autotune: bool = True,
+                                      BLOCK_SIZE_M: int = 64, BLOCK_SIZE_N: int = 64, BLOCK_SIZE_K: int = 32,
+                                      GROUP_SIZE: int = 8, out: torch.Tensor = None,
+                                      accumulate: bool = False) -> torch.Tensor:
+    """hashed_weight_grad[H] = scatter_add over W tiles of (input^T . output_grad) * init_factor.
+
+    Same signature as the reference launcher (python/rz_linear/impl/RzLinearBackward.py:23-97);
+    the result has output_grad's dtype.  The tiles are reduced and scattered in fp32 whatever the
+    dtype (the reference adds atomically in output_grad's dtype), then converted once.
+
+    Beyond the reference: ``out`` (a [H] tensor of output_grad's dtype or float32) receives the
+    result instead of a new tensor, and with ``accumulate=True`` the gradient is added to what
+    ``out`` holds — for layers that share one hashed_weight and for fp32 master gradients.
+    """
+    R = _lib.hash_constants(R7, R6, R5, R4, R3, R2, R1, R0)
+    return _weight_grad(input, output_grad, init_factor, M, K, N, H, R, BLOCK_SIZE_K, BLOCK_SIZE_N,
+                        out=out, accumulate=accumulate)[0]
+
+
+def rz_linear_backward_weight_bias_grad_tl(input: torch.Tensor, output_grad: torch.Tensor, init_factor: float,
+                                           M: int, K: int, N: int, H: int,
+                                           R7: int, R6: int, R5: int, R4: int,
+                                           R3: int, R2: int, R1: int, R0: int,
+                                           allow_tf32: bool = True, allow_autotune: bool = True,
+                                           BLOCK_SIZE_M: int = 64, BLOCK_SIZE_N: int = 64, BLOCK_SIZE_K: int = 32,
+                                           GROUP_SIZE: int = 8, out: torch.Tensor = None,
+                                           accumulate: bool = False) -> Tuple[torch.Tensor, torch.Tensor]:
+    """(hashed_weight_grad[H], bias_grad[N]) from one pass over output_grad.
+
+    bias_grad = output_grad.sum(0): the gradient of the bias that the reference module adds after
+    the product (python/rz_linear/RzLinear.py:93-94) and leaves to autograd.  Here the
+    weight-grad kernel sums the output_grad tiles it stages anyway.  No counterpart launcher in
+    the reference; arguments as rz_linear_backward_weight_grad_tl.
+    """
+    R = _lib.hash_constants(R7, R6, R5, R4, R3, R2, R1, R0)
+    return _weight_grad(input, output_grad, init_factor, M, K, N, H, R, BLOCK_SIZE_K, BLOCK_SIZE_N,
+                        out=out, accumulate=accumulate, with_bias_grad=True)
 
 
 def rz_linear_backward_input_grad_tl(output_grad: torch.Tensor, hashed_weight: torch.Tensor, init_factor: float,

@@ -1,0 +1,122 @@
+"""GPU parity of rz_weight_grad_ex: bias gradient from the same pass, accumulation into an
+existing buffer, fp32 gradient buffers for 16-bit operands.  Checked against the CPU oracle's
+weight-grad and against the column sums of dY in float64."""
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import SEED_CONSTANTS, TOL, make_inputs, rargs, rel_err
+
+pytestmark = pytest.mark.gpu
+
+R1024 = SEED_CONSTANTS[1024]
+
+# (M, K, N, H, BK, BN)
+CASES = [
+    (512, 512, 512, 9000, 64, 64),       # complete tiles, LDS image
+    (300, 200, 330, 9000, 32, 64),       # ragged
+    (256, 256, 512, 70000, 64, 64),      # H too large for the LDS image: global atomics
+    (130, 70, 90, 2000, 16, 16),         # 16-wide tiles
+    (4100, 192, 160, 30000, 64, 64),     # long M: the reduction is cut into slices
+    (40, 1500, 140, 9000, 64, 64),       # more tile rows than R steps: some workgroups never sum
+]
+ENVS = [{}, {"RZLINEAR_TILE": "64"}, {"RZLINEAR_TILE": "128"}, {"RZLINEAR_TILE": "256"},
+        {"RZLINEAR_TILE": "128", "RZLINEAR_STAGES": "1"}, {"RZLINEAR_NO_LDS_IMAGE": "1"}]
+_env_id = lambda e: "-".join("%s=%s" % (k.replace("RZLINEAR_", ""), v) for k, v in e.items()) or "auto"
+_dt_id = lambda d: str(d).split(".")[-1]
+_shape_id = lambda s: "x".join(map(str, s))
+
+
+def _say(*a):
+    print(*a, flush=True)
+    sys.stdout.flush()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16], ids=_dt_id)
+@pytest.mark.parametrize("env", ENVS, ids=_env_id)
+@pytest.mark.parametrize("shape", CASES, ids=_shape_id)
+def test_bias_grad_from_the_weight_grad_pass(oracle, monkeypatch, shape, env, dtype):
+    from rzlinear_amd.impl.RzLinearBackward import rz_linear_backward_weight_bias_grad_tl
+    for k, v in env.items():
+        monkeypatch.setenv(k, v)
+    M, K, N, H, BK, BN = shape
+    _say("weight+bias grad", shape, env, dtype)
+    (x, _, dy), (x64, _, dy64) = make_inputs(M, K, N, H, dtype, seed=11)
+    dhw, dbias = rz_linear_backward_weight_bias_grad_tl(x, dy, 0.5, M, K, N, H, *rargs(R1024),
+                                                        BLOCK_SIZE_K=BK, BLOCK_SIZE_N=BN)
+    torch.cuda.synchronize()
+    assert dhw.shape == (H,) and dhw.dtype == dtype
+    assert dbias.shape == (N,) and dbias.dtype == dtype
+    assert rel_err(dhw.float().cpu().numpy(), oracle.weight_grad(x64, dy64, H, BK, BN, R1024, 0.5)) <= TOL[dtype]
+    # the bias gradient is not scaled by init_factor
+    assert rel_err(dbias.float().cpu().numpy(), dy64.sum(axis=0)) <= TOL[dtype]
+
+
+@pytest.mark.parametrize("out_dtype", ["same", "f32"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=_dt_id)
+@pytest.mark.parametrize("env", [{}, {"RZLINEAR_NO_LDS_IMAGE": "1"}], ids=_env_id)
+@pytest.mark.parametrize("shape", CASES[:4], ids=_shape_id)
+def test_accumulate_into_an_existing_gradient(oracle, monkeypatch, shape, env, dtype, out_dtype):
+    from rzlinear_amd.impl.RzLinearBackward import (rz_linear_backward_weight_bias_grad_tl,
+                                                    rz_linear_backward_weight_grad_tl)
+    for k, v in env.items():
+        monkeypatch.setenv(k, v)
+    M, K, N, H, BK, BN = shape
+    _say("accumulate", shape, env, dtype, out_dtype)
+    (x, _, dy), (x64, _, dy64) = make_inputs(M, K, N, H, dtype, seed=12)
+    odt = torch.float32 if out_dtype == "f32" else dtype
+    ref = oracle.weight_grad(x64, dy64, H, BK, BN, R1024, 1.0)
+    g = torch.Generator().manual_seed(5)
+    start = (torch.randn((H,), generator=g) * float(np.abs(ref).max())).to(odt)
+    # overwrite into a caller-owned buffer
+    buf = start.clone().cuda()
+    out = rz_linear_backward_weight_grad_tl(x, dy, 1.0, M, K, N, H, *rargs(R1024), BLOCK_SIZE_K=BK,
+                                            BLOCK_SIZE_N=BN, out=buf)
+    torch.cuda.synchronize()
+    assert out.data_ptr() == buf.data_ptr() and out.dtype == odt
+    assert rel_err(buf.float().cpu().numpy(), ref) <= TOL[dtype]
+    # add to what the buffer holds; twice, with the bias gradient the second time
+    buf = start.clone().cuda()
+    rz_linear_backward_weight_grad_tl(x, dy, 1.0, M, K, N, H, *rargs(R1024), BLOCK_SIZE_K=BK,
+                                      BLOCK_SIZE_N=BN, out=buf, accumulate=True)
+    torch.cuda.synchronize()
+    want = start.double().numpy() + ref
+    assert rel_err(buf.float().cpu().numpy(), want) <= TOL[odt if odt != torch.float32 else dtype]
+    _, dbias = rz_linear_backward_weight_bias_grad_tl(x, dy, 1.0, M, K, N, H, *rargs(R1024), BLOCK_SIZE_K=BK,
+                                                      BLOCK_SIZE_N=BN, out=buf, accumulate=True)
+    torch.cuda.synchronize()
+    want = start.double().numpy() + 2 * ref
+    assert rel_err(buf.float().cpu().numpy(), want) <= 2 * TOL[odt if odt != torch.float32 else dtype]
+    assert rel_err(dbias.float().cpu().numpy(), dy64.sum(axis=0)) <= TOL[dtype]
+
+
+def test_ex_argument_checks():
+    import ctypes
+    from rzlinear_amd import _lib
+    from rzlinear_amd.impl.RzLinearBackward import rz_linear_backward_weight_grad_tl
+    lib = _lib.load()
+    M, K, N, H = 64, 64, 64, 5000
+    x = torch.zeros((M, K), device="cuda")
+    dy = torch.zeros((M, N), device="cuda")
+    dhw = torch.zeros((H,), device="cuda")
+    R = (ctypes.c_int32 * 8)(*R1024)
+    s = torch.cuda.current_stream().cuda_stream
+    need = lib.rz_weight_grad_ex_workspace_bytes(M, K, N, H, 64, 64, 0, 0, 1)
+    assert need > lib.rz_weight_grad_ex_workspace_bytes(M, K, N, H, 64, 64, 0, 0, 0)
+    assert lib.rz_weight_grad_ex_workspace_bytes(M, K, N, H, 64, 64, 0, 0, 0) == \
+        lib.rz_weight_grad_workspace_bytes(M, K, N, H, 64, 64, 0)
+    # unknown flag bit, workspace too small for the column sums
+    assert lib.rz_weight_grad_ex(x.data_ptr(), dy.data_ptr(), dhw.data_ptr(), None, None, 0, M, K, N, H, 64, 64,
+                                 R, 1.0, K, N, 0, 8, s) == -9
+    ws = torch.empty((need,), dtype=torch.uint8, device="cuda")
+    dbias = torch.zeros((N,), device="cuda")
+    assert lib.rz_weight_grad_ex(x.data_ptr(), dy.data_ptr(), dhw.data_ptr(), dbias.data_ptr(), ws.data_ptr(),
+                                 need - 1, M, K, N, H, 64, 64, R, 1.0, K, N, 0, 0, s) == -7
+    with pytest.raises(ValueError):
+        rz_linear_backward_weight_grad_tl(x, dy, 1.0, M, K, N, H, *rargs(R1024), BLOCK_SIZE_K=64,
+                                          BLOCK_SIZE_N=64, accumulate=True)
+    with pytest.raises(TypeError):
+        rz_linear_backward_weight_grad_tl(x, dy, 1.0, M, K, N, H, *rargs(R1024), BLOCK_SIZE_K=64,
+                                          BLOCK_SIZE_N=64, out=torch.zeros((H,), device="cuda", dtype=torch.float16))

@@ -74,7 +74,11 @@ def test_launcher_signatures_are_the_reference_ones():
     dims = ["M", "K", "N", "H"]
     assert names(rz_linear_forward_tl) == ["input", "hashed_weight", "init_factor"] + dims + consts + tail
     assert names(rz_linear_backward_tl) == ["input", "hashed_weight", "output_grad", "init_factor"] + dims + consts + tail
-    assert names(rz_linear_backward_weight_grad_tl) == ["input", "output_grad", "init_factor"] + dims + consts + tail
+    # the reference's arguments first, then this build's optional gradient-buffer arguments
+    assert names(rz_linear_backward_weight_grad_tl) == (["input", "output_grad", "init_factor"] + dims + consts + tail +
+                                                        ["out", "accumulate"])
+    extra = inspect.signature(rz_linear_backward_weight_grad_tl).parameters
+    assert extra["out"].default is None and extra["accumulate"].default is False
     assert names(rz_linear_backward_input_grad_tl) == ["output_grad", "hashed_weight", "init_factor"] + dims + consts + tail
     assert names(rz_linear_idx_tl) == ["hashed_weight", "K", "N", "H", "R3", "R2", "R1", "R0", "BLOCK_SIZE_K", "BLOCK_SIZE_N"]
     d = {k: v.default for k, v in inspect.signature(rz_linear_forward_tl).parameters.items()}
