@@ -56,7 +56,7 @@ def build(keep_asm=False, jobs=None, verbose=True, extra_flags=(), out=None):
     extra_flags / out build a variant (e.g. with -D tuning switches) next to the default one;
     RZLINEAR_LIB=<path> makes the package load it."""
     out = out or LIB_PATH
-    obj_dir = OBJ_DIR if out == LIB_PATH else OBJ_DIR + "_" + os.path.basename(out).replace(".", "_")
+    obj_dir = OBJ_DIR if out == LIB_PATH else os.path.join(OBJ_DIR, "variant_" + os.path.basename(out).replace(".", "_"))
     os.makedirs(obj_dir, exist_ok=True)
     srcs = sources()
     jobs = jobs or min(len(srcs), os.cpu_count() or 1, 16)

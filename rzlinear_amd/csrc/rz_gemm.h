@@ -17,6 +17,15 @@
 //        bytes, and the 64-byte row skew of this pitch keeps those on distinct banks)
 //   fp32                                : [TR][X + pad], one ds_read_b32 per lane; a source
 //       with R contiguous is transposed while it is written (pad 1), else copied (pad 4)
+//
+// Direct staging (16-bit types, complete tiles, two stages): the tiles go global -> LDS with
+// direct-to-LDS loads, no registers and no LDS write instructions in between.  Such a load
+// puts the 64 lanes' 16-byte pieces at consecutive LDS addresses, so rows cannot be padded;
+// the stages are unpadded and swizzled instead, and the swizzle is applied on the global side
+// (each lane fetches the piece that belongs at its LDS slot):
+//   R contiguous : [X][TR], row = 8 pieces; piece p of row x sits at slot p ^ ((x >> 1) & 7)
+//   X contiguous : [TR][X], row = X/32 chunks of 64 bytes; chunk c of row r sits at c ^ (r & 3)
+// Both keep the fragment reads above free of bank conflicts.
 #pragma once
 
 #include <type_traits>
@@ -117,9 +126,13 @@ struct GemmKernel {
   static constexpr int MI = WTI / 32, MJ = WTJ / 32;   // 32x32 MFMA blocks per wavefront
   static_assert(WTI % 32 == 0 && WTJ % 32 == 0, "wavefront tile must be a multiple of 32");
 
+  // direct-to-LDS staging (see the head of this file)
+  static constexpr bool kDirect = k16 && FULL && NSTAGE == 2 && !COLSUM && TI >= 128 && TJ >= 128;
+
   template <int LAYOUT, int TX> struct Lds {
-    static constexpr int kPitch = k16 ? (LAYOUT == kRContig ? TR + 8 : TX + 32)
-                                      : (LAYOUT == kRContig ? TX + 1 : TX + 4);
+    static constexpr int kPitch = kDirect ? (LAYOUT == kRContig ? TR : TX)
+                                  : k16   ? (LAYOUT == kRContig ? TR + 8 : TX + 32)
+                                          : (LAYOUT == kRContig ? TX + 1 : TX + 4);
     static constexpr int kRows = (k16 && LAYOUT == kRContig) ? TX : TR;
     static constexpr int kElems = ((kPitch * kRows + 7) / 8) * 8;
     // source tile as seen by the global loads
@@ -172,12 +185,16 @@ struct GemmKernel {
       return reinterpret_cast<const float*>(lds)[(ks * 2 + (lane >> 5)) * L::kPitch + x_base +
                                                  (lane & 31)];
     } else if constexpr (LAYOUT == kRContig) {
-      return *reinterpret_cast<const u32x4_t*>(lds + (x_base + (lane & 31)) * L::kPitch + ks * 16 +
-                                               8 * (lane >> 5));
+      const int row = x_base + (lane & 31), piece = ks * 2 + (lane >> 5);
+      if constexpr (kDirect)
+        return *reinterpret_cast<const u32x4_t*>(lds + row * L::kPitch + ((piece ^ ((row >> 1) & 7)) << 3));
+      return *reinterpret_cast<const u32x4_t*>(lds + row * L::kPitch + piece * 8);
     } else {
       const int g = lane >> 4, jl = lane & 15;
-      const T* p = lds + (ks * 16 + 8 * (g >> 1) + (jl >> 2)) * L::kPitch + x_base + 16 * (g & 1) +
-                   4 * (jl & 3);
+      const int row = ks * 16 + 8 * (g >> 1) + (jl >> 2), col = x_base + 16 * (g & 1) + 4 * (jl & 3);
+      // (row + 4 has the same swizzle as row, so the second read is one pitch-multiple further)
+      const T* p = kDirect ? lds + row * L::kPitch + ((((col >> 5) ^ (row & 3)) << 5) | (col & 31))
+                           : lds + row * L::kPitch + col;
       typedef s16x4_t __attribute__((address_space(3))) * lds_s16x4_ptr;
       const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(p));
       const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(p + 4 * L::kPitch));
@@ -379,6 +396,65 @@ struct GemmKernel {
         colsum_turn = (colsum_turn + 1 == p.tiles_i) ? 0 : colsum_turn + 1;
       }
     };
+    // Direct staging: where a lane's q-th load instruction of a tile fetches from.  The
+    // instruction with index n = wave * kPieces + q fills LDS bytes [1024 n, 1024 n + 1024) of
+    // the stage, lane i the 16 bytes at 16 i; (row, col) is the source piece that the swizzled
+    // layout keeps there.
+    auto direct_src = [&](auto L, int layout, int q, int& row, int& col) {
+      typedef decltype(L) LL;
+      const int n = wave * LL::kPieces + q;
+      if (layout == kRContig) {
+        row = n * 8 + (lane >> 3);
+        col = ((lane & 7) ^ ((row >> 1) & 7)) * 8;
+      } else {
+        constexpr int kSlots = LL::kPitch / 8;          // 16-byte slots per row
+        row = n * (64 / kSlots) + lane / kSlots;
+        const int slot = lane % kSlots;
+        col = (((slot >> 2) ^ (row & 3)) << 5) | ((slot & 3) << 3);
+      }
+    };
+    auto direct_load = [&](const T* src, const T* stage, int q, int pieces) {
+      // the LDS address goes through M0 and must be the same for the whole wavefront
+      typedef const T __attribute__((address_space(3)))* lds_ptr;
+      const uint32_t dst = __builtin_amdgcn_readfirstlane(
+          (uint32_t)(uintptr_t)(lds_ptr)(stage) + (uint32_t)((wave * pieces + q) * 1024));
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(dst), "v"(src)
+                   : "memory", "m0");
+    };
+    // all tiles of R step `step` -> LDS stage `st`
+    auto direct_issue = [&](int step, int st) {
+      const int r0 = r_begin + step * TR;
+#pragma unroll
+      for (int q = 0; q < LA::kPieces; q++) {
+        int row, col;
+        direct_src(LA{}, A_LAYOUT, q, row, col);
+        const T* src = (A_LAYOUT == kRContig) ? gA + (int64_t)(i0 + row) * p.lda + r0 + col
+                                              : gA + (int64_t)(r0 + row) * p.lda + i0 + col;
+        direct_load(src, sm.a[st], q, LA::kPieces);
+      }
+      if constexpr (OP == kWeightGrad) {
+#pragma unroll
+        for (int q = 0; q < LB::kPieces; q++) {
+          int row, col;
+          direct_src(LB{}, B_LAYOUT, q, row, col);
+          direct_load(gB + (int64_t)(r0 + row) * p.ldb + j0 + col, sm.b[st], q, LB::kPieces);
+        }
+      } else {
+        const OffWindow w = window(step);
+        const int* tab = sm.off + (step & (kOffSlots - 1)) * kOffWindow;
+        int idx[LB::kPieces];
+#pragma unroll
+        for (int q = 0; q < LB::kPieces; q++) {   // all table lookups first, then the loads
+          int row, col;
+          direct_src(LB{}, B_LAYOUT, q, row, col);
+          const int k = (OP == kForward) ? r0 + row : j0 + row;
+          const int n = (OP == kForward) ? j0 + col : r0 + col;
+          idx[q] = hashed_index(p.h, tab, w, k, n);
+        }
+#pragma unroll
+        for (int q = 0; q < LB::kPieces; q++) direct_load(gHW + idx[q], sm.b[st], q, LB::kPieces);
+      }
+    };
     // MFMAs of one R step out of LDS stage `st`; fragments are read one sub-step ahead
     auto compute = [&](int st) {
       constexpr int NKS = TR / KS;
@@ -428,7 +504,7 @@ struct GemmKernel {
       hash_step(1);
       hash_step(2);
       if constexpr (OP != kWeightGrad) __syncthreads();
-      fetch(0);
+      if constexpr (!kDirect) fetch(0);
     }
     if constexpr (NSTAGE == 1) {
       // one LDS stage: write it, read it, two barriers per step; relies on several
@@ -451,6 +527,10 @@ struct GemmKernel {
       // waited for) its last reads of stage s&1 and has written stage (s+1)&1, so the last
       // sub-step can already read the first fragments of step s+1, and the next step's writes
       // into stage s&1 are safe.
+      // With direct staging the side jobs shrink to one: right after the barrier of step s,
+      // when stage s&1 has been read for the last time, the direct-to-LDS loads of step s+2
+      // are issued into it; they have a whole step to land and are waited for just before the
+      // barrier of step s+1.
       constexpr int NKS = TR / KS;
       static_assert(NKS >= 3, "pipeline needs at least three sub-steps per R step");
       Frag fa[2][MI], fb[2][MJ];
@@ -483,14 +563,24 @@ struct GemmKernel {
           if (ks + 1 < NKS) {
             frags(st, ks + 1, (ks + 1) & 1);
           } else {
+            if constexpr (kDirect) {
+              // the loads of step s+1 (the only ones in flight) must have landed
+              if constexpr (decltype(has_next)::value) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            }
             __syncthreads();
+            if constexpr (kDirect) {
+              // stage st has been read for the last time: refill it for step s+2
+              if constexpr (decltype(do_fetch)::value) direct_issue(s + 2, st);
+            }
             if constexpr (decltype(has_next)::value) frags(st ^ 1, 0, (ks + 1) & 1);
           }
-          if (ks == kCommitAt) {
-            if constexpr (decltype(do_commit)::value) commit(st ^ 1);
-          }
-          if (ks == kFetchAt) {
-            if constexpr (decltype(do_fetch)::value) fetch(s + 2);
+          if constexpr (!kDirect) {
+            if (ks == kCommitAt) {
+              if constexpr (decltype(do_commit)::value) commit(st ^ 1);
+            }
+            if (ks == kFetchAt) {
+              if constexpr (decltype(do_fetch)::value) fetch(s + 2);
+            }
           }
           mfmas(ks & 1);
         }
@@ -505,9 +595,21 @@ struct GemmKernel {
         step(s, late, std::false_type{}, std::false_type{}, std::false_type{});
       };
       if (steps > 0) {
-        commit(0);
-        if (steps > 1) fetch(1);
-        hash_step(3);
+        if constexpr (kDirect) {
+          direct_issue(0, 0);
+          if (steps > 1) {
+            direct_issue(1, 1);
+            hash_step(3);
+            // loads complete in order: all but the last step's worth have landed
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LA::kPieces + LB::kPieces) : "memory");
+          } else {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+          }
+        } else {
+          commit(0);
+          if (steps > 1) fetch(1);
+          hash_step(3);
+        }
         __syncthreads();
         frags(0, 0, 0);
         // wavefronts w and w + 4 of a workgroup share a SIMD
