@@ -245,6 +245,12 @@ struct GemmKernel {
     const int lane = tid & 63;
     const int wave = tid >> 6;
     const int wave_i = wave / WJ, wave_j = wave % WJ;
+    // Offset in the C tile of a wavefront's 32x32 block (a, b).  Forward and input-grad give a
+    // wavefront one contiguous WTI x WTJ sub-tile (whole cache lines per store).  Weight-grad
+    // deals the blocks round-robin instead, so that the blocks of one hashed tile belong to
+    // different wavefronts and its scatter round is shared between them.
+    auto blk_i = [&](int a) -> int { return (OP == kWeightGrad) ? (a * WI + wave_i) * 32 : wave_i * WTI + a * 32; };
+    auto blk_j = [&](int b) -> int { return (OP == kWeightGrad) ? (b * WJ + wave_j) * 32 : wave_j * WTJ + b * 32; };
 
     // Workgroup ids are dealt round-robin to the 8 XCDs; renumber so that each XCD (one L2)
     // gets a contiguous run of tiles, then walk tiles with J fastest (forward/input-grad
@@ -462,10 +468,10 @@ struct GemmKernel {
       auto frags = [&](int ks, int buf) {
 #pragma unroll
         for (int a = 0; a < MI; a++)
-          fa[buf][a] = lds_frag<A_LAYOUT, LA>(sm.a[st], wave_i * WTI + a * 32, ks, lane);
+          fa[buf][a] = lds_frag<A_LAYOUT, LA>(sm.a[st], blk_i(a), ks, lane);
 #pragma unroll
         for (int b = 0; b < MJ; b++)
-          fb[buf][b] = lds_frag<B_LAYOUT, LB>(sm.b[st], wave_j * WTJ + b * 32, ks, lane);
+          fb[buf][b] = lds_frag<B_LAYOUT, LB>(sm.b[st], blk_j(b), ks, lane);
       };
       frags(0, 0);
 #pragma unroll
@@ -537,10 +543,10 @@ struct GemmKernel {
       auto frags = [&](int st, int ks, int buf) {
 #pragma unroll
         for (int a = 0; a < MI; a++)
-          fa[buf][a] = lds_frag<A_LAYOUT, LA>(sm.a[st], wave_i * WTI + a * 32, ks, lane);
+          fa[buf][a] = lds_frag<A_LAYOUT, LA>(sm.a[st], blk_i(a), ks, lane);
 #pragma unroll
         for (int b = 0; b < MJ; b++)
-          fb[buf][b] = lds_frag<B_LAYOUT, LB>(sm.b[st], wave_j * WTJ + b * 32, ks, lane);
+          fb[buf][b] = lds_frag<B_LAYOUT, LB>(sm.b[st], blk_j(b), ks, lane);
       };
       auto mfmas = [&](int buf) {
 #pragma unroll
@@ -659,19 +665,19 @@ struct GemmKernel {
         for (int a = 0; a < MI; a++)
 #pragma unroll
           for (int b = 0; b < MJ; b++) {
-            const int n = j0 + wave_j * WTJ + b * 32 + (lane & 31);
+            const int n = j0 + blk_j(b) + (lane & 31);
             int base[4];
             bool ok[4];
 #pragma unroll
             for (int g = 0; g < 4; g++) {
-              const int k = i0 + wave_i * WTI + a * 32 + g * 8 + (lane >> 5) * 4;
+              const int k = i0 + blk_i(a) + g * 8 + (lane >> 5) * 4;
               ok[g] = FULL || (k < p.I && n < p.J);
               base[g] = etab[((k >> p.h.bk_shift) - w.tk0) * w.ntn + ((n >> p.h.bn_shift) - w.tn0)] +
                         (k & (p.h.BK - 1)) * p.h.BN + (n & (p.h.BN - 1));
             }
 #pragma unroll
             for (int e = 0; e < 16; e++) {
-              const int k = i0 + wave_i * WTI + a * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
+              const int k = i0 + blk_i(a) + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
               if (FULL || (ok[e >> 2] && k < p.I))
                 unsafeAtomicAdd(target + base[e >> 2] + (e & 3) * p.h.BN, acc[a][b][e] * p.scale);
             }
@@ -690,7 +696,7 @@ struct GemmKernel {
           for (int a = 0; a < MI; a++)
 #pragma unroll
             for (int b = 0; b < MJ; b++) {
-              const int k0 = i0 + wave_i * WTI + a * 32, n0 = j0 + wave_j * WTJ + b * 32;
+              const int k0 = i0 + blk_i(a), n0 = j0 + blk_j(b);
               const int t = __builtin_amdgcn_readfirstlane(((k0 >> p.h.bk_shift) - w.tk0) * w.ntn +
                                                            ((n0 >> p.h.bn_shift) - w.tn0));
               blk_tile[a][b] = t;
@@ -704,8 +710,8 @@ struct GemmKernel {
 #pragma unroll
                 for (int b = 0; b < MJ; b++) {
                   if (blk_tile[a][b] == t) {
-                    const int k0 = i0 + wave_i * WTI + a * 32 + (lane >> 5) * 4;
-                    const bool col_ok = FULL || (j0 + wave_j * WTJ + b * 32 + (lane & 31) < p.J);
+                    const int k0 = i0 + blk_i(a) + (lane >> 5) * 4;
+                    const bool col_ok = FULL || (j0 + blk_j(b) + (lane & 31) < p.J);
                     float cur[16];
 #pragma unroll
                     for (int e = 0; e < 16; e++)
@@ -739,10 +745,10 @@ struct GemmKernel {
         for (int a = 0; a < MI; a++) {
 #pragma unroll
           for (int e = 0; e < 16; e++) {
-            const int row = i0 + wave_i * WTI + a * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
+            const int row = i0 + blk_i(a) + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
 #pragma unroll
             for (int b = 0; b < MJ; b++) {
-              const int col = j0 + wave_j * WTJ + b * 32 + (lane & 31);
+              const int col = j0 + blk_j(b) + (lane & 31);
               if (FULL || (row < p.I && col < p.J)) gP[(size_t)row * p.J + col] = acc[a][b][e] * p.scale;
             }
           }
@@ -755,7 +761,7 @@ struct GemmKernel {
       float bias[MJ];
 #pragma unroll
       for (int b = 0; b < MJ; b++) {
-        const int col = j0 + wave_j * WTJ + b * 32 + (lane & 31);
+        const int col = j0 + blk_j(b) + (lane & 31);
         bias[b] = 0.f;
         if (gBias != nullptr && (FULL || col < p.J)) bias[b] = Tr::to_float(gBias[col]);
       }
@@ -765,10 +771,10 @@ struct GemmKernel {
       for (int a = 0; a < MI; a++) {
 #pragma unroll
         for (int e = 0; e < 16; e++) {
-          const int row = i0 + wave_i * WTI + a * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
+          const int row = i0 + blk_i(a) + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
 #pragma unroll
           for (int b = 0; b < MJ; b++) {
-            const int col = j0 + wave_j * WTJ + b * 32 + (lane & 31);
+            const int col = j0 + blk_j(b) + (lane & 31);
             if (FULL || (row < p.I && col < p.J))
               gC[(int64_t)row * p.ldc + col] = Tr::from_float(acc[a][b][e] * p.scale + bias[b]);
           }
