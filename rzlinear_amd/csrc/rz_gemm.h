@@ -127,7 +127,7 @@ struct GemmKernel {
   static_assert(WTI % 32 == 0 && WTJ % 32 == 0, "wavefront tile must be a multiple of 32");
 
   // direct-to-LDS staging (see the head of this file)
-  static constexpr bool kDirect = k16 && FULL && NSTAGE == 2 && !COLSUM && TI >= 128 && TJ >= 128;
+  static constexpr bool kDirect = k16 && FULL && NSTAGE == 2 && TI >= 128 && TJ >= 128;
 
   template <int LAYOUT, int TX> struct Lds {
     static constexpr int kPitch = kDirect ? (LAYOUT == kRContig ? TR : TX)
@@ -293,8 +293,9 @@ struct GemmKernel {
 
     // Bias gradient (COLSUM): the tiles_i workgroups of one tile column and slice stage the same
     // rows of dY, so they take turns: the workgroup whose turn it is adds the rows of that R
-    // step, from the registers on their way into LDS, into per-thread column sums.  A thread's
-    // pieces sit in one 16-byte column position, so VEC sums per thread suffice.
+    // step, from the registers on their way into LDS (direct staging: from the LDS stage), into
+    // per-thread column sums.  A thread's pieces sit in one 16-byte column position, so VEC
+    // sums per thread suffice.
     static_assert(!COLSUM || kThreads % LB::kCpr == 0, "a thread's pieces must share their columns");
     float colsum[VEC];
 #pragma unroll
@@ -401,6 +402,25 @@ struct GemmKernel {
         }
         colsum_turn = (colsum_turn + 1 == p.tiles_i) ? 0 : colsum_turn + 1;
       }
+    };
+    // Direct staging: the same sums out of the dY tile in LDS stage `st`.  Thread (g, c) =
+    // (tid / kCpr, tid % kCpr) adds rows g, g + groups, ... of the 16-byte column position c;
+    // the rows are a multiple of four apart, so they share one swizzle.
+    auto colsum_from_stage = [&](int st) {
+      constexpr int kGroups = kThreads / LB::kCpr;
+      static_assert(!(COLSUM && kDirect) || (kGroups % 4 == 0 && TR % kGroups == 0), "rows must share a swizzle");
+      if (colsum_turn == ti) {
+        const int g = tid / LB::kCpr, c = tid % LB::kCpr;
+        const int slot = (((c >> 2) ^ (g & 3)) << 2) | (c & 3);
+#pragma unroll
+        for (int i = 0; i < TR / kGroups; i++) {
+          T elems[VEC];
+          __builtin_memcpy(elems, sm.b[st] + (g + i * kGroups) * LB::kPitch + slot * VEC, 16);
+#pragma unroll
+          for (int e = 0; e < VEC; e++) colsum[e] += Tr::to_float(elems[e]);
+        }
+      }
+      colsum_turn = (colsum_turn + 1 == p.tiles_i) ? 0 : colsum_turn + 1;
     };
     // Direct staging: where a lane's q-th load instruction of a tile fetches from.  The
     // instruction with index n = wave * kPieces + q fills LDS bytes [1024 n, 1024 n + 1024) of
@@ -579,6 +599,9 @@ struct GemmKernel {
               if constexpr (decltype(do_fetch)::value) direct_issue(s + 2, st);
             }
             if constexpr (decltype(has_next)::value) frags(st ^ 1, 0, (ks + 1) & 1);
+          }
+          if constexpr (kDirect && COLSUM) {
+            if (ks == 1) colsum_from_stage(st);   // once per R step, in step order
           }
           if constexpr (!kDirect) {
             if (ks == kCommitAt) {
