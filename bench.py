@@ -59,8 +59,8 @@ TRAFFIC_BYTES = {
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--workload", default="square4096", choices=sorted(WORKLOADS))
     ap.add_argument("--dtype", default=None, choices=["bf16", "fp16", "fp32"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -174,8 +174,8 @@ def main():
         wt = w.t().contiguous()
         xt = x.t().contiguous()
 
-        def timeit(fn, n=20):
-            for _ in range(3):
+        def timeit(fn, n=100):
+            for _ in range(20):
                 fn()
             torch.cuda.synchronize()
             a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)

@@ -104,6 +104,13 @@ static inline WeightGradPlan plan_weight_grad(int M, int K, int N, int H, int el
     pl.tile = 64;
     if (tile_cover(K, N, 128) * 10 <= tile_cover(K, N, 64) * 13) pl.tile = 128;
     if (tile_cover(K, N, 256) * 10 <= tile_cover(K, N, pl.tile) * 13) pl.tile = 256;
+    // a short M cut over many slices leaves a 256 workgroup a step or two between its prologue
+    // and its scatter: the 128 tile then has less to set up and to scatter per workgroup
+    const long long tiles256 = tile_count(K, N, 256);
+    if (pl.tile == 256 && tiles256 < kComputeUnits &&
+        (long long)((M + TR - 1) / TR) * tiles256 < 4LL * kComputeUnits &&
+        tile_cover(K, N, 128) * 10 <= tile_cover(K, N, 256) * 13)
+      pl.tile = 128;
   } else {
     pl.tile = pick_tile(K, N);
   }
