@@ -49,9 +49,9 @@ PEAK = {"bf16": 2500.0, "fp16": 2500.0, "fp32": 157.3}
 # WRITE_SIZE x1.0); the rocprof summary with the raw readings is committed with the profiles.
 TRAFFIC_BYTES = {
     ("square4096", "bf16"): {
-        "forward": int((16659.0 * 2.0 + 32768.0) * 1024),       # algorithmic: 64.03 MiB
-        "input_grad": int((16659.0 * 2.0 + 32768.0) * 1024),
-        "weight_grad": int((98457.2 * 2.0 + 16784.1) * 1024),   # X, dY re-read by 3 XCD groups; + partial images
+        "forward": int((16672.7 * 2.0 + 32768.0) * 1024),       # algorithmic: 64.03 MiB
+        "input_grad": int((16672.7 * 2.0 + 32768.0) * 1024),
+        "weight_grad": int((98457.7 * 2.0 + 16785.8) * 1024),   # X, dY re-read by 3 XCD groups; + partial images
     },
 }
 
