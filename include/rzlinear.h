@@ -54,6 +54,15 @@ typedef enum rz_dtype {
   RZ_F16 = 2
 } rz_dtype;
 
+/* Which tile hash an entry point with a `hash_levels` argument evaluates. */
+typedef enum rz_hash {
+  RZ_HASH_ONE_LEVEL = 1,  /* ((tk*R3 + tn*R2 + R1) % R0) % (H - BK*BN)          impl/RzLinearIdx.py:70-71 */
+  RZ_HASH_TWO_LEVEL = 2,  /* the hash of the three kernels                       impl/RzLinearForward.py:316 */
+  RZ_HASH_LEGACY = 3      /* ((tk*R3 + tn*R2 + R1) % R0) % (H - BK*BN + 1) in 64-bit integers: the tiled
+                             location of the legacy generation (16 x 16 tiles, prime 2038074743),
+                             /rz_linear_kernel.cu:34-36,:56-64; R4..R7 unused; H >= BK*BN suffices */
+} rz_hash;
+
 /* Library / ABI version (major*10000 + minor*100 + patch). */
 int rz_version(void);
 
@@ -68,6 +77,8 @@ const char* rz_status_string(int status);
  *       rz_linear_backward_input_grad_core                            impl/RzLinearBackward.py:686,:716
  *   hash_levels = 1:  off = ((tk*R3 + tn*R2 + R1) % R0) % (H - BK*BN)
  *       replaces the hash of rz_linear_idx_kernel                     impl/RzLinearIdx.py:70-71
+ *   hash_levels = 3:  the legacy generation's tiled location (see rz_hash)
+ *       replaces location_tiled                                       /rz_linear_kernel.cu:56-64
  * out has ceil(K/BK)*ceil(N/BN) entries, index tk*ceil(N/BN) + tn.
  */
 int rz_tile_offsets(int32_t* out, int K, int N, int H, int BK, int BN, const int32_t R[8],
@@ -172,6 +183,26 @@ int rz_weight_grad_ex(const void* X, const void* dY, void* dHW, void* dbias, voi
                       size_t workspace_bytes, int M, int K, int N, int H, int BK, int BN,
                       const int32_t R[8], float init_factor, int64_t ldx, int64_t lddy, int dtype,
                       unsigned flags, void* stream);
+
+/*
+ * The three contractions with an explicit tile hash (rz_hash).  hash_levels = RZ_HASH_TWO_LEVEL
+ * gives rz_forward_ws / rz_input_grad_ws / rz_weight_grad_ex (same workspace sizes, same
+ * flags).  RZ_HASH_LEGACY runs a hashed_weight laid out by the legacy generation — its
+ * forward /rz_linear_kernel.cu:245-338 and backward :516-592 in tiled mode — with BK = BN = 16
+ * and the constants of /RzLinear.py:70-75 (larger tiles follow the same formula).
+ */
+int rz_forward_hashed(const void* X, const void* HW, const void* bias, void* Y, void* workspace,
+                      size_t workspace_bytes, int M, int K, int N, int H, int BK, int BN,
+                      const int32_t R[8], int hash_levels, float init_factor, int64_t ldx, int64_t ldy,
+                      int dtype, void* stream);
+int rz_input_grad_hashed(const void* dY, const void* HW, void* dX, void* workspace,
+                         size_t workspace_bytes, int M, int K, int N, int H, int BK, int BN,
+                         const int32_t R[8], int hash_levels, float init_factor, int64_t lddy,
+                         int64_t lddx, int dtype, void* stream);
+int rz_weight_grad_hashed(const void* X, const void* dY, void* dHW, void* dbias, void* workspace,
+                          size_t workspace_bytes, int M, int K, int N, int H, int BK, int BN,
+                          const int32_t R[8], int hash_levels, float init_factor, int64_t ldx,
+                          int64_t lddy, int dtype, unsigned flags, void* stream);
 
 /*
  * Materialise W[K,N] (row pitch ldw) from hashed_weight; edge tiles are clipped.

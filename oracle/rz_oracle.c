@@ -43,6 +43,8 @@ RZ_EXPORT int64_t rz_oracle_tile_offset(int64_t tk, int64_t tn, int64_t H, int64
   const int64_t R0 = R[0];
   const int64_t range = H - BK * BN; /* precondition H > BK*BN, RzLinearForward.py:28 */
   const int64_t hi = (tk * R[3] + tn * R[2] + R[1]) % R0;
+  /* legacy generation: one level, 64-bit, range + 1 (/rz_linear_kernel.cu:34-36,:56-64) */
+  if (hash_levels == 3) return hi % (range + 1);
   if (hash_levels == 1) return hi % range; /* RzLinearIdx.py:70-71 */
   const int64_t lo = (tk * R[7] + tn * R[5] + R[4]) % R0;
   return (hi * R0 + lo) % range;
@@ -53,13 +55,15 @@ RZ_EXPORT int64_t rz_oracle_tile_offset(int64_t tk, int64_t tn, int64_t H, int64
  * (the reference evaluates the hash in 32-bit integers). */
 RZ_EXPORT int rz_oracle_tile_offsets(int64_t *out, int64_t K, int64_t N, int64_t H, int64_t BK,
                                      int64_t BN, const int32_t *R, int hash_levels) {
-  if (H <= BK * BN) return -1;
+  if (hash_levels == 3 ? H < BK * BN : H <= BK * BN) return -1;
   const int64_t TK = (K + BK - 1) / BK, TN = (N + BN - 1) / BN;
   const int64_t lim = 2147483647LL;
   const int64_t R0 = R[0];
-  if ((TK * (int64_t)R[3] + TN * (int64_t)R[2] + R[1]) > lim) return -2;
-  if ((TK * (int64_t)R[7] + TN * (int64_t)R[5] + R[4]) > lim) return -2;
-  if (hash_levels != 1 && (R0 - 1) * R0 + (R0 - 1) > lim) return -2;
+  if (hash_levels != 3) { /* the legacy hash is evaluated in 64-bit integers */
+    if ((TK * (int64_t)R[3] + TN * (int64_t)R[2] + R[1]) > lim) return -2;
+    if ((TK * (int64_t)R[7] + TN * (int64_t)R[5] + R[4]) > lim) return -2;
+    if (hash_levels != 1 && (R0 - 1) * R0 + (R0 - 1) > lim) return -2;
+  }
   for (int64_t tk = 0; tk < TK; tk++)
     for (int64_t tn = 0; tn < TN; tn++)
       out[tk * TN + tn] = rz_oracle_tile_offset(tk, tn, H, BK, BN, R, hash_levels);

@@ -38,10 +38,28 @@ HASH_CONSTANTS = {
 
 
 # ------------------------------------------------------------------ numpy restatement
+LEGACY_PRIME = 2038074743
+HASH_LEGACY = 3
+
+
+def legacy_constants(seed):
+    """[R0..R7] of the legacy generation for `seed` (/RzLinear.py:70-75): the prime, then odd
+    numbers from numpy's RandomState(seed).randint(0, prime, 50) (an even draw is bumped by 1).
+    Only R0..R3 enter its tile hash."""
+    x = np.random.RandomState(seed).randint(0, LEGACY_PRIME, (50,))
+    x = x + 1 * (x % 2 == 0)
+    return [LEGACY_PRIME] + [int(v) for v in x[:7]]
+
+
 def tile_offset(tk, tn, H, BK, BN, R, hash_levels=2):
     """Offset of tile (tk, tn) in hashed_weight, Python integers (no overflow possible).
-    Two-level: RzLinearForward.py:316; one-level: RzLinearIdx.py:70-71."""
+    Two-level: RzLinearForward.py:316; one-level: RzLinearIdx.py:70-71; 3 = the legacy
+    generation's tile hash, one level with range H - BK*BN + 1 (/rz_linear_kernel.cu:34-36,:56-64,
+    where the tile is 16 x 16)."""
     R = [int(v) for v in R]
+    if hash_levels == HASH_LEGACY:
+        assert H >= BK * BN
+        return ((tk * R[3] + tn * R[2] + R[1]) % R[0]) % (H - BK * BN + 1)
     rng = H - BK * BN
     assert rng > 0, "need H > BK*BN (RzLinearForward.py:28)"
     hi = (tk * R[3] + tn * R[2] + R[1]) % R[0]
@@ -73,24 +91,24 @@ def materialize(hw, K, N, BK, BN, R, hash_levels=2):
     return hw[index_map(K, N, hw.shape[0], BK, BN, R, hash_levels)]
 
 
-def forward(X, hw, N, BK, BN, R, init_factor=1.0):
+def forward(X, hw, N, BK, BN, R, init_factor=1.0, hash_levels=2):
     X = np.asarray(X, dtype=np.float64)
-    W = materialize(hw, X.shape[1], N, BK, BN, R)
+    W = materialize(hw, X.shape[1], N, BK, BN, R, hash_levels)
     return (X @ W) * init_factor
 
 
-def input_grad(dY, hw, K, BK, BN, R, init_factor=1.0):
+def input_grad(dY, hw, K, BK, BN, R, init_factor=1.0, hash_levels=2):
     dY = np.asarray(dY, dtype=np.float64)
-    W = materialize(hw, K, dY.shape[1], BK, BN, R)
+    W = materialize(hw, K, dY.shape[1], BK, BN, R, hash_levels)
     return (dY @ W.T) * init_factor
 
 
-def weight_grad(X, dY, H, BK, BN, R, init_factor=1.0):
+def weight_grad(X, dY, H, BK, BN, R, init_factor=1.0, hash_levels=2):
     X = np.asarray(X, dtype=np.float64)
     dY = np.asarray(dY, dtype=np.float64)
     K, N = X.shape[1], dY.shape[1]
     dW = X.T @ dY
-    idx = index_map(K, N, H, BK, BN, R)
+    idx = index_map(K, N, H, BK, BN, R, hash_levels)
     return np.bincount(idx.ravel(), weights=dW.ravel(), minlength=H) * init_factor
 
 

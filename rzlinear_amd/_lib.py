@@ -21,7 +21,7 @@ EXPORTS = (
     "rz_version", "rz_status_string", "rz_tile_offsets", "rz_tile_offsets_device", "rz_forward",
     "rz_forward_bias", "rz_forward_workspace_bytes", "rz_forward_ws", "rz_input_grad",
     "rz_input_grad_workspace_bytes", "rz_input_grad_ws", "rz_weight_grad_workspace_bytes", "rz_weight_grad", "rz_weight_grad_ex_workspace_bytes",
-    "rz_weight_grad_ex", "rz_materialize",
+    "rz_weight_grad_ex", "rz_forward_hashed", "rz_input_grad_hashed", "rz_weight_grad_hashed", "rz_materialize",
 )
 
 _lib = None
@@ -83,6 +83,15 @@ def load():
     lib.rz_weight_grad_ex.restype = c_int
     lib.rz_weight_grad_ex.argtypes = [c_vp, c_vp, c_vp, c_vp, c_vp, c_sz, c_int, c_int, c_int, c_int, c_int, c_int,
                                       i32p, c_f, c_i64, c_i64, c_int, ctypes.c_uint, c_vp]
+    lib.rz_forward_hashed.restype = c_int
+    lib.rz_forward_hashed.argtypes = [c_vp, c_vp, c_vp, c_vp, c_vp, c_sz, c_int, c_int, c_int, c_int, c_int, c_int,
+                                      i32p, c_int, c_f, c_i64, c_i64, c_int, c_vp]
+    lib.rz_input_grad_hashed.restype = c_int
+    lib.rz_input_grad_hashed.argtypes = [c_vp, c_vp, c_vp, c_vp, c_sz, c_int, c_int, c_int, c_int, c_int, c_int,
+                                         i32p, c_int, c_f, c_i64, c_i64, c_int, c_vp]
+    lib.rz_weight_grad_hashed.restype = c_int
+    lib.rz_weight_grad_hashed.argtypes = [c_vp, c_vp, c_vp, c_vp, c_vp, c_sz, c_int, c_int, c_int, c_int, c_int,
+                                          c_int, i32p, c_int, c_f, c_i64, c_i64, c_int, ctypes.c_uint, c_vp]
     lib.rz_materialize.restype = c_int
     lib.rz_materialize.argtypes = [c_vp, c_vp, c_int, c_int, c_int, c_int, c_int, i32p, c_int, c_i64,
                                    c_int, c_vp]
@@ -92,6 +101,8 @@ def load():
 
 # options of rz_weight_grad_ex
 WG_ACCUMULATE, WG_DHW_F32, WG_DBIAS_F32 = 1, 2, 4
+# tile hashes (rz_hash)
+HASH_ONE_LEVEL, HASH_TWO_LEVEL, HASH_LEGACY = 1, 2, 3
 
 
 def check(status):

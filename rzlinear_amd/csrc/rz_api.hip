@@ -29,16 +29,21 @@ static int make_hash(HashParams* h, int K, int N, int H, int BK, int BN, const i
   if (K < 1 || N < 1 || H < 1) return RZ_ERR_BAD_SHAPE;
   int st = check_tile(BK, BN);
   if (st != RZ_OK) return st;
-  if ((long long)H <= (long long)BK * BN) return RZ_ERR_HASH_RANGE;
-  if (levels != 1 && levels != 2) return RZ_ERR_BAD_ARGUMENT;
+  if (levels != RZ_HASH_ONE_LEVEL && levels != RZ_HASH_TWO_LEVEL && levels != RZ_HASH_LEGACY)
+    return RZ_ERR_BAD_ARGUMENT;
+  const bool legacy = levels == RZ_HASH_LEGACY;
+  if (legacy ? (long long)H < (long long)BK * BN : (long long)H <= (long long)BK * BN)
+    return RZ_ERR_HASH_RANGE;
   for (int i = 0; i < 8; i++)
     if (R[i] < 0) return RZ_ERR_BAD_ARGUMENT;
   if (R[0] < 1) return RZ_ERR_BAD_ARGUMENT;
   const long long lim = 2147483647LL;
   const long long TK = ((long long)K + BK - 1) / BK, TN = ((long long)N + BN - 1) / BN;
-  if (TK * R[3] + TN * R[2] + R[1] > lim) return RZ_ERR_HASH_OVERFLOW;
-  if (TK * R[7] + TN * R[5] + R[4] > lim) return RZ_ERR_HASH_OVERFLOW;
-  if (levels == 2 && ((long long)R[0] - 1) * R[0] + (R[0] - 1) > lim) return RZ_ERR_HASH_OVERFLOW;
+  if (!legacy) {   // the legacy hash is evaluated in 64-bit integers and cannot overflow them
+    if (TK * R[3] + TN * R[2] + R[1] > lim) return RZ_ERR_HASH_OVERFLOW;
+    if (TK * R[7] + TN * R[5] + R[4] > lim) return RZ_ERR_HASH_OVERFLOW;
+    if (levels == 2 && ((long long)R[0] - 1) * R[0] + (R[0] - 1) > lim) return RZ_ERR_HASH_OVERFLOW;
+  }
   h->R0 = (uint32_t)R[0];
   h->R1 = (uint32_t)R[1];
   h->R2 = (uint32_t)R[2];
@@ -46,7 +51,7 @@ static int make_hash(HashParams* h, int K, int N, int H, int BK, int BN, const i
   h->R4 = (uint32_t)R[4];
   h->R5 = (uint32_t)R[5];
   h->R7 = (uint32_t)R[7];
-  h->range = (uint32_t)(H - BK * BN);
+  h->range = (uint32_t)(H - BK * BN + (legacy ? 1 : 0));
   h->BK = BK;
   h->BN = BN;
   h->bk_shift = ilog2_exact(BK);
@@ -280,13 +285,13 @@ static WeightGradWorkspace weight_grad_workspace(const WeightGradPlan& plan, int
 static int weight_grad_impl(const void* X, const void* dY, void* dHW, void* dbias, void* workspace,
                             size_t workspace_bytes, int M, int K, int N, int H, int BK, int BN,
                             const int32_t R[8], float init_factor, int64_t ldx, int64_t lddy, int dtype,
-                            unsigned flags, void* stream) {
+                            unsigned flags, void* stream, int hash_levels = RZ_HASH_TWO_LEVEL) {
   if (X == nullptr || dY == nullptr || dHW == nullptr) return RZ_ERR_NULL_POINTER;
   if (dtype_bytes(dtype) == 0) return RZ_ERR_BAD_DTYPE;
   if (M < 1 || ldx < K || lddy < N) return RZ_ERR_BAD_SHAPE;
   if (flags & ~(unsigned)(RZ_WG_ACCUMULATE | RZ_WG_DHW_F32 | RZ_WG_DBIAS_F32)) return RZ_ERR_BAD_ARGUMENT;
   GemmParams p = {};
-  int st = make_hash(&p.h, K, N, H, BK, BN, R, 2);
+  int st = make_hash(&p.h, K, N, H, BK, BN, R, hash_levels);
   if (st != RZ_OK) return st;
   const bool accumulate = (flags & RZ_WG_ACCUMULATE) != 0;
   const int dhw_dtype = (flags & RZ_WG_DHW_F32) ? RZ_F32 : dtype;
@@ -388,12 +393,12 @@ RZ_API int rz_tile_offsets_device(int32_t* d_out, int K, int N, int H, int BK, i
 static int forward_impl(const void* X, const void* HW, const void* bias, void* Y, void* workspace,
                         size_t workspace_bytes, bool may_split, int M, int K, int N, int H, int BK, int BN,
                         const int32_t R[8], float init_factor, int64_t ldx, int64_t ldy, int dtype,
-                        void* stream) {
+                        void* stream, int hash_levels = RZ_HASH_TWO_LEVEL) {
   if (X == nullptr || HW == nullptr || Y == nullptr) return RZ_ERR_NULL_POINTER;
   if (dtype_bytes(dtype) == 0) return RZ_ERR_BAD_DTYPE;
   if (M < 1 || ldx < K || ldy < N) return RZ_ERR_BAD_SHAPE;
   GemmParams p = {};
-  int st = make_hash(&p.h, K, N, H, BK, BN, R, 2);
+  int st = make_hash(&p.h, K, N, H, BK, BN, R, hash_levels);
   if (st != RZ_OK) return st;
   p.A = X;
   p.HW = HW;
@@ -409,12 +414,13 @@ static int forward_impl(const void* X, const void* HW, const void* bias, void* Y
 
 static int input_grad_impl(const void* dY, const void* HW, void* dX, void* workspace, size_t workspace_bytes,
                            bool may_split, int M, int K, int N, int H, int BK, int BN, const int32_t R[8],
-                           float init_factor, int64_t lddy, int64_t lddx, int dtype, void* stream) {
+                           float init_factor, int64_t lddy, int64_t lddx, int dtype, void* stream,
+                           int hash_levels = RZ_HASH_TWO_LEVEL) {
   if (dY == nullptr || HW == nullptr || dX == nullptr) return RZ_ERR_NULL_POINTER;
   if (dtype_bytes(dtype) == 0) return RZ_ERR_BAD_DTYPE;
   if (M < 1 || lddy < N || lddx < K) return RZ_ERR_BAD_SHAPE;
   GemmParams p = {};
-  int st = make_hash(&p.h, K, N, H, BK, BN, R, 2);
+  int st = make_hash(&p.h, K, N, H, BK, BN, R, hash_levels);
   if (st != RZ_OK) return st;
   p.A = dY;
   p.HW = HW;
@@ -508,6 +514,30 @@ RZ_API int rz_weight_grad_ex(const void* X, const void* dY, void* dHW, void* dbi
                              int dtype, unsigned flags, void* stream) {
   return weight_grad_impl(X, dY, dHW, dbias, workspace, workspace_bytes, M, K, N, H, BK, BN, R,
                           init_factor, ldx, lddy, dtype, flags, stream);
+}
+
+RZ_API int rz_forward_hashed(const void* X, const void* HW, const void* bias, void* Y, void* workspace,
+                             size_t workspace_bytes, int M, int K, int N, int H, int BK, int BN,
+                             const int32_t R[8], int hash_levels, float init_factor, int64_t ldx,
+                             int64_t ldy, int dtype, void* stream) {
+  return forward_impl(X, HW, bias, Y, workspace, workspace_bytes, true, M, K, N, H, BK, BN, R, init_factor,
+                      ldx, ldy, dtype, stream, hash_levels);
+}
+
+RZ_API int rz_input_grad_hashed(const void* dY, const void* HW, void* dX, void* workspace,
+                                size_t workspace_bytes, int M, int K, int N, int H, int BK, int BN,
+                                const int32_t R[8], int hash_levels, float init_factor, int64_t lddy,
+                                int64_t lddx, int dtype, void* stream) {
+  return input_grad_impl(dY, HW, dX, workspace, workspace_bytes, true, M, K, N, H, BK, BN, R, init_factor,
+                         lddy, lddx, dtype, stream, hash_levels);
+}
+
+RZ_API int rz_weight_grad_hashed(const void* X, const void* dY, void* dHW, void* dbias, void* workspace,
+                                 size_t workspace_bytes, int M, int K, int N, int H, int BK, int BN,
+                                 const int32_t R[8], int hash_levels, float init_factor, int64_t ldx,
+                                 int64_t lddy, int dtype, unsigned flags, void* stream) {
+  return weight_grad_impl(X, dY, dHW, dbias, workspace, workspace_bytes, M, K, N, H, BK, BN, R,
+                          init_factor, ldx, lddy, dtype, flags, stream, hash_levels);
 }
 
 RZ_API int rz_materialize(const void* HW, void* W, int K, int N, int H, int BK, int BN,

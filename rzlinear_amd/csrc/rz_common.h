@@ -66,9 +66,11 @@ template <> struct ElemTraits<f16_t> {
 // off(tk,tn) = (((tk*R3 + tn*R2 + R1) % R0) * R0 + ((tk*R7 + tn*R5 + R4) % R0)) % (H - BK*BN)
 // (levels == 1 keeps only the first term).  The host checks that every intermediate stays
 // below 2^31, so unsigned 32-bit arithmetic equals the reference's signed 32-bit arithmetic.
+// levels == 3 is the legacy generation's tile hash: the first term alone, evaluated in 64-bit
+// integers (its prime is close to 2^31), modulo H - BK*BN + 1; `range` then holds that value.
 struct HashParams {
   uint32_t R0, R1, R2, R3, R4, R5, R7;
-  uint32_t range;      // H - BK*BN
+  uint32_t range;      // H - BK*BN  (legacy hash: H - BK*BN + 1)
   int bk_shift, bn_shift;
   int BK, BN;
   int levels;
@@ -76,6 +78,8 @@ struct HashParams {
 
 __host__ __device__ __forceinline__ uint32_t tile_offset(const HashParams& h, uint32_t tk,
                                                          uint32_t tn) {
+  if (h.levels == 3)
+    return (uint32_t)((((uint64_t)tk * h.R3 + (uint64_t)tn * h.R2 + h.R1) % h.R0) % h.range);
   const uint32_t hi = (tk * h.R3 + tn * h.R2 + h.R1) % h.R0;
   if (h.levels == 1) return hi % h.range;
   const uint32_t lo = (tk * h.R7 + tn * h.R5 + h.R4) % h.R0;

@@ -27,9 +27,9 @@ def rz_linear_backward_tl(input: torch.Tensor, hashed_weight: torch.Tensor, outp
     return input_grad, weight_grad
 
 
-def _weight_grad(input, output_grad, init_factor, M, K, N, H, R, BLOCK_SIZE_K, BLOCK_SIZE_N,
-                 out=None, accumulate=False, with_bias_grad=False):
-    """One rz_weight_grad_ex call; returns (hashed_weight_grad, bias_grad or None)."""
+def weight_grad_hashed(input, output_grad, init_factor, M, K, N, H, R, BLOCK_SIZE_K, BLOCK_SIZE_N,
+                       out=None, accumulate=False, with_bias_grad=False, hash_levels=_lib.HASH_TWO_LEVEL):
+    """One rz_weight_grad_hashed call; returns (hashed_weight_grad, bias_grad or None)."""
     stream = _lib.require_gpu(input, output_grad)
     if input.dtype != output_grad.dtype:
         raise TypeError("input is %s but output_grad is %s" % (input.dtype, output_grad.dtype))
@@ -56,9 +56,9 @@ def _weight_grad(input, output_grad, init_factor, M, K, N, H, R, BLOCK_SIZE_K, B
     need = lib.rz_weight_grad_ex_workspace_bytes(M, K, N, H, BLOCK_SIZE_K, BLOCK_SIZE_N, code, flags,
                                                  int(with_bias_grad))
     ws = _lib.workspace(need, output_grad.device)
-    _lib.check(lib.rz_weight_grad_ex(
+    _lib.check(lib.rz_weight_grad_hashed(
         x.data_ptr(), dy.data_ptr(), out.data_ptr(), bias_grad.data_ptr() if with_bias_grad else None,
-        ws.data_ptr() if need else None, need, M, K, N, H, BLOCK_SIZE_K, BLOCK_SIZE_N, R,
+        ws.data_ptr() if need else None, need, M, K, N, H, BLOCK_SIZE_K, BLOCK_SIZE_N, R, hash_levels,
         float(init_factor), ldx, lddy, code, flags, stream))
     return out, bias_grad
 
@@ -82,7 +82,7 @@ def rz_linear_backward_weight_grad_tl(input: torch.Tensor, output_grad: torch.Te
     ``out`` holds — for layers that share one hashed_weight and for fp32 master gradients.
     """
     R = _lib.hash_constants(R7, R6, R5, R4, R3, R2, R1, R0)
-    return _weight_grad(input, output_grad, init_factor, M, K, N, H, R, BLOCK_SIZE_K, BLOCK_SIZE_N,
+    return weight_grad_hashed(input, output_grad, init_factor, M, K, N, H, R, BLOCK_SIZE_K, BLOCK_SIZE_N,
                         out=out, accumulate=accumulate)[0]
 
 
@@ -102,7 +102,7 @@ def rz_linear_backward_weight_bias_grad_tl(input: torch.Tensor, output_grad: tor
     the reference; arguments as rz_linear_backward_weight_grad_tl.
     """
     R = _lib.hash_constants(R7, R6, R5, R4, R3, R2, R1, R0)
-    return _weight_grad(input, output_grad, init_factor, M, K, N, H, R, BLOCK_SIZE_K, BLOCK_SIZE_N,
+    return weight_grad_hashed(input, output_grad, init_factor, M, K, N, H, R, BLOCK_SIZE_K, BLOCK_SIZE_N,
                         out=out, accumulate=accumulate, with_bias_grad=True)
 
 
@@ -118,6 +118,13 @@ def rz_linear_backward_input_grad_tl(output_grad: torch.Tensor, hashed_weight: t
     Same signature as the reference launcher (python/rz_linear/impl/RzLinearBackward.py:374-449).
     """
     assert (H > (BLOCK_SIZE_K * BLOCK_SIZE_N))
+    return input_grad_hashed(output_grad, hashed_weight, init_factor, M, K, N, H,
+                             _lib.hash_constants(R7, R6, R5, R4, R3, R2, R1, R0), BLOCK_SIZE_K, BLOCK_SIZE_N,
+                             _lib.HASH_TWO_LEVEL)
+
+
+def input_grad_hashed(output_grad, hashed_weight, init_factor, M, K, N, H, R, BK, BN, hash_levels):
+    """One rz_input_grad_hashed call: R is the int32[8] constant array, hash_levels an rz_hash code."""
     stream = _lib.require_gpu(output_grad, hashed_weight)
     if hashed_weight.dtype != output_grad.dtype:
         raise TypeError("output_grad is %s but hashed_weight is %s" % (output_grad.dtype, hashed_weight.dtype))
@@ -126,10 +133,9 @@ def rz_linear_backward_input_grad_tl(output_grad: torch.Tensor, hashed_weight: t
     input_grad = torch.empty((M, K), device=output_grad.device, dtype=output_grad.dtype)
     lib = _lib.load()
     code = _lib.dtype_code(output_grad)
-    need = lib.rz_input_grad_workspace_bytes(M, K, N, H, BLOCK_SIZE_K, BLOCK_SIZE_N, code)
+    need = lib.rz_input_grad_workspace_bytes(M, K, N, H, BK, BN, code)
     ws = _lib.workspace(need, output_grad.device)
-    _lib.check(lib.rz_input_grad_ws(
+    _lib.check(lib.rz_input_grad_hashed(
         dy.data_ptr(), hw.data_ptr(), input_grad.data_ptr(), ws.data_ptr() if need else None, need,
-        M, K, N, H, BLOCK_SIZE_K, BLOCK_SIZE_N,
-        _lib.hash_constants(R7, R6, R5, R4, R3, R2, R1, R0), float(init_factor), lddy, K, code, stream))
+        M, K, N, H, BK, BN, R, hash_levels, float(init_factor), lddy, K, code, stream))
     return input_grad

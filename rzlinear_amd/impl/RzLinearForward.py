@@ -37,6 +37,13 @@ def rz_linear_forward_bias_tl(input: torch.Tensor, hashed_weight: torch.Tensor, 
     kernel's store, instead of by the separate ``x + self._bias`` of the reference module
     (python/rz_linear/RzLinear.py:93-94)."""
     assert (H > (BLOCK_SIZE_K * BLOCK_SIZE_N))
+    return forward_hashed(input, hashed_weight, bias, init_factor, M, K, N, H,
+                          _lib.hash_constants(R7, R6, R5, R4, R3, R2, R1, R0), BLOCK_SIZE_K, BLOCK_SIZE_N,
+                          _lib.HASH_TWO_LEVEL)
+
+
+def forward_hashed(input, hashed_weight, bias, init_factor, M, K, N, H, R, BK, BN, hash_levels):
+    """One rz_forward_hashed call: R is the int32[8] constant array, hash_levels an rz_hash code."""
     stream = _lib.require_gpu(input, hashed_weight, *([bias] if bias is not None else []))
     if hashed_weight.dtype != input.dtype:
         raise TypeError("input is %s but hashed_weight is %s" % (input.dtype, hashed_weight.dtype))
@@ -50,10 +57,10 @@ def rz_linear_forward_bias_tl(input: torch.Tensor, hashed_weight: torch.Tensor, 
     lib = _lib.load()
     code = _lib.dtype_code(input)
     # skinny problems split the contraction and need a scratch buffer for the partial results
-    need = lib.rz_forward_workspace_bytes(M, K, N, H, BLOCK_SIZE_K, BLOCK_SIZE_N, code)
+    need = lib.rz_forward_workspace_bytes(M, K, N, H, BK, BN, code)
     ws = _lib.workspace(need, input.device)
-    _lib.check(lib.rz_forward_ws(
+    _lib.check(lib.rz_forward_hashed(
         x.data_ptr(), hw.data_ptr(), bias.data_ptr() if bias is not None else None, output.data_ptr(),
-        ws.data_ptr() if need else None, need, M, K, N, H, BLOCK_SIZE_K, BLOCK_SIZE_N,
-        _lib.hash_constants(R7, R6, R5, R4, R3, R2, R1, R0), float(init_factor), ldx, N, code, stream))
+        ws.data_ptr() if need else None, need, M, K, N, H, BK, BN, R, hash_levels, float(init_factor),
+        ldx, N, code, stream))
     return output

@@ -56,6 +56,21 @@ def test_host_tile_offsets_bit_exact(lib, oracle, cfg, levels):
         assert np.array_equal(got, oracle.c_tile_offsets(K, N, H, BK, BN, R, levels))
 
 
+@pytest.mark.parametrize("cfg", [(128, 128, 1000, 16, 16), (99999, 99999, 66000, 256, 256), (99999, 16, 300, 16, 16),
+                                 (40000, 500, 1000000, 16, 16), (64, 64, 256, 16, 16)])
+def test_host_tile_offsets_legacy_hash(lib, oracle, cfg):
+    """hash_levels = 3: the legacy generation's 64-bit hash with its prime near 2^31."""
+    from rzlinear_amd import _lib
+    K, N, H, BK, BN = cfg
+    for seed in (1024, 7):
+        R = oracle.legacy_constants(seed)
+        got = _lib.tile_offsets(K, N, H, BK, BN, R, 3).numpy().astype(np.int64)
+        assert np.array_equal(got, oracle.c_tile_offsets(K, N, H, BK, BN, R, 3))
+    if cfg == (128, 128, 1000, 16, 16):   # tile bases behind the row the reference's notebook recorded
+        R = oracle.legacy_constants(1024)
+        assert _lib.tile_offsets(K, N, H, BK, BN, R, 3)[0].tolist() == [259, 417, 575, 581, 739, 152, 310, 468]
+
+
 def test_status_codes(lib):
     out = (ctypes.c_int32 * 64)()
     i32p = ctypes.POINTER(ctypes.c_int32)
@@ -69,7 +84,12 @@ def test_status_codes(lib):
     assert call(0, 128, 65536, 64, 64, R1024) == -2
     assert call(128, 128, 65536, 64, 64, [2**31 - 1] + R1024[1:]) == -6
     assert call(128, 128, 65536, 64, 64, [45007, -1] + R1024[2:]) == -9
-    assert call(128, 128, 65536, 64, 64, R1024, 3) == -9
+    assert call(128, 128, 65536, 64, 64, R1024, 4) == -9          # no such hash
+    assert call(128, 128, 65536, 64, 64, R1024, 0) == -9
+    # the legacy hash is 64-bit (no overflow status) and accepts H == BK*BN
+    assert call(128, 128, 65536, 64, 64, [2**31 - 1] + R1024[1:], 3) == 0
+    assert call(128, 128, 4096, 64, 64, R1024, 3) == 0
+    assert call(128, 128, 4095, 64, 64, R1024, 3) == -4
     assert lib.rz_tile_offsets(None, 128, 128, 65536, 64, 64, _R(R1024), 2) == -1
     # device entry points validate before they touch the GPU
     assert lib.rz_forward(None, None, None, 1, 1, 1, 65536, 64, 64, _R(R1024), 1.0, 1, 1, 0, None) == -1
@@ -90,6 +110,8 @@ def test_status_codes(lib):
                                 10240, 1024, 0, None) == -7
     assert lib.rz_weight_grad_workspace_bytes(8, 128, 128, 65536, 64, 64, 0) == 0
     assert lib.rz_weight_grad_workspace_bytes(8, 128, 128, 65536, 64, 64, 1) == 65536 * 4
+    assert lib.rz_forward_hashed(one, one, None, one, None, 0, 8, 128, 128, 65536, 64, 64, _R(R1024), 5, 1.0,
+                                 128, 128, 0, None) == -9
     for code in range(0, -10, -1):
         assert lib.rz_status_string(code) not in (None, b"", b"unknown status")
     assert lib.rz_status_string(-99) == b"unknown status"

@@ -269,3 +269,37 @@ def test_oracle_matches_vectors_produced_by_the_reference_kernels(oracle):
                 assert ref.shape == got.shape
                 # the reference accumulates in fp32: allow its rounding, nothing more
                 assert np.abs(ref - got).max() <= 2e-6 * np.abs(got).max()
+
+
+# ---------------------------------------------------------------- legacy generation hash
+# Row 1 of the output the reference's notebook recorded for hashed_weight = arange(1000),
+# input = eye(128), a 128 x 128 layer, seed 1024 (verify.ipynb, cell 3): with an identity
+# input the output is the index map itself.
+NOTEBOOK_ROW1 = sum((list(range(a, a + 16)) for a in (275, 433, 591, 597, 755, 168, 326, 484)), [])
+# the first numbers the legacy module printed for seed 1024 (same notebook)
+NOTEBOOK_NUMBERS = [2038074743, 634329019, 1825252241, 871205357]
+
+
+def test_legacy_hash_reproduces_the_notebook_row(oracle):
+    R = oracle.legacy_constants(1024)
+    assert R[:4] == NOTEBOOK_NUMBERS
+    assert all(v % 2 == 1 for v in R[1:])
+    W = oracle.materialize(np.arange(1000), 128, 128, 16, 16, R, hash_levels=3)
+    assert W[1].astype(np.int64).tolist() == NOTEBOOK_ROW1
+    Wc = oracle.c_materialize(np.arange(1000.0), 128, 128, 16, 16, R, hash_levels=3)
+    assert np.array_equal(W, Wc)
+    # identity input: forward output = W (the notebook's trick)
+    assert np.array_equal(oracle.forward(np.eye(128), np.arange(1000), 128, 16, 16, R, hash_levels=3), W)
+
+
+def test_legacy_hash_is_64_bit_and_uses_range_plus_one(oracle):
+    R = oracle.legacy_constants(7)
+    # products far beyond 2^31: Python integers vs the C restatement
+    offs = oracle.c_tile_offsets(16 * 3000, 16 * 5, 70001, 16, 16, R, 3)
+    for tk in (0, 1, 2999):
+        for tn in range(5):
+            want = ((tk * R[3] + tn * R[2] + R[1]) % R[0]) % (70001 - 256 + 1)
+            assert offs[tk, tn] == want == oracle.tile_offset(tk, tn, 70001, 16, 16, R, 3)
+    # H == BK*BN is legal there: every tile at offset 0
+    assert not oracle.c_tile_offsets(64, 64, 256, 16, 16, R, 3).any()
+    assert (oracle.c_tile_offsets(640, 640, 257, 16, 16, R, 3) <= 1).all()
