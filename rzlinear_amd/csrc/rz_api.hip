@@ -5,6 +5,7 @@
 
 #include "rz_common.h"
 #include "rz_launch.h"
+#include "rz_window.h"
 
 namespace rz {
 
@@ -273,9 +274,11 @@ static inline size_t round256(size_t b) { return (b + 255) & ~(size_t)255; }
 struct WeightGradWorkspace {
   size_t main_bytes, total_bytes;
 };
-static WeightGradWorkspace weight_grad_workspace(const WeightGradPlan& plan, int H, bool dhw_f32, bool with_dbias) {
+static WeightGradWorkspace weight_grad_workspace(const WeightGradPlan& plan, const WindowPlan& window, int H,
+                                                 bool dhw_f32, bool with_dbias) {
   WeightGradWorkspace w;
   if (plan.image_pitch > 0) w.main_bytes = plan.workspace_bytes;
+  else if (window.use && !with_dbias) w.main_bytes = round256((size_t)window.tiles * sizeof(int32_t));  // tile offsets
   else w.main_bytes = dhw_f32 ? 0 : round256((size_t)H * sizeof(float));
   w.total_bytes = w.main_bytes + (with_dbias ? plan.colsum_bytes : 0);
   return w;
@@ -297,7 +300,9 @@ static int weight_grad_impl(const void* X, const void* dY, void* dHW, void* dbia
   const int dhw_dtype = (flags & RZ_WG_DHW_F32) ? RZ_F32 : dtype;
   const int dbias_dtype = (flags & RZ_WG_DBIAS_F32) ? RZ_F32 : dtype;
   const WeightGradPlan plan = plan_weight_grad(M, K, N, H, dtype_bytes(dtype));
-  const WeightGradWorkspace ws = weight_grad_workspace(plan, H, dhw_dtype == RZ_F32, dbias != nullptr);
+  WindowPlan wp = {};
+  if (plan.image_pitch == 0) wp = plan_window(M, K, N, H, BK, BN, dtype_bytes(dtype));
+  const WeightGradWorkspace ws = weight_grad_workspace(plan, wp, H, dhw_dtype == RZ_F32, dbias != nullptr);
   if (ws.total_bytes > 0 && (workspace == nullptr || workspace_bytes < ws.total_bytes)) return RZ_ERR_WORKSPACE;
   hipStream_t s = (hipStream_t)stream;
   p.A = X;
@@ -309,6 +314,32 @@ static int weight_grad_impl(const void* X, const void* dY, void* dHW, void* dbia
   p.ldb = lddy;
   p.scale = init_factor;
   if (dbias != nullptr) p.colsum = reinterpret_cast<float*>(static_cast<char*>(workspace) + ws.main_bytes);
+  if (plan.image_pitch == 0 && dbias == nullptr && wp.use) {
+    // large hashed_weight, short contraction: windows of dHW instead of K*N atomics.  The
+    // tile offsets are hashed once into the workspace; every workgroup scans them.
+    {
+      const int TK = (K + BK - 1) / BK, TN = (N + BN - 1) / BN;
+      hipLaunchKernelGGL(tile_offsets_kernel, dim3((TK * TN + 255) / 256), dim3(256), 0, s, (int32_t*)workspace,
+                         TK, TN, p.h);
+      if (hipGetLastError() != hipSuccess) return RZ_ERR_LAUNCH;
+      WindowParams w = {};
+      w.offsets = (const int32_t*)workspace;
+      w.X = X; w.dY = dY; w.dHW = dHW;
+      w.M = M; w.K = K; w.N = N; w.H = H;
+      w.ldx = ldx; w.lddy = lddy;
+      w.scale = init_factor;
+      w.h = p.h;
+      w.window = wp.window;
+      w.tiles_k = (K + BK - 1) / BK;
+      w.tiles_n = (N + BN - 1) / BN;
+      w.accumulate = accumulate ? 1 : 0;
+      w.out_f32 = dhw_dtype == RZ_F32 ? 1 : 0;
+      hipError_t e = dtype == RZ_F32 ? launch_window_f32(w, wp.windows, s)
+                     : dtype == RZ_BF16 ? launch_window_bf16(w, wp.windows, s)
+                                        : launch_window_f16(w, wp.windows, s);
+      return e == hipSuccess ? RZ_OK : RZ_ERR_LAUNCH;
+    }
+  }
   if (plan.image_pitch > 0) {
     // every workgroup sums its tiles into an LDS image of dHW and stores it as a partial image;
     // the partial images are then added up (no global atomics, fixed summation order)
@@ -500,12 +531,13 @@ RZ_API int rz_weight_grad(const void* X, const void* dY, void* dHW, void* worksp
 
 RZ_API size_t rz_weight_grad_ex_workspace_bytes(int M, int K, int N, int H, int BK, int BN, int dtype,
                                                 unsigned flags, int with_dbias) {
-  (void)BK; (void)BN;
   const int eb = dtype_bytes(dtype);
   if (eb == 0 || M < 1 || K < 1 || N < 1 || H < 1) return 0;
   const WeightGradPlan plan = plan_weight_grad(M, K, N, H, eb);
   const bool dhw_f32 = (flags & RZ_WG_DHW_F32) != 0 || dtype == RZ_F32;
-  return weight_grad_workspace(plan, H, dhw_f32, with_dbias != 0).total_bytes;
+  WindowPlan wp = {};
+  if (plan.image_pitch == 0 && check_tile(BK, BN) == RZ_OK) wp = plan_window(M, K, N, H, BK, BN, eb);
+  return weight_grad_workspace(plan, wp, H, dhw_f32, with_dbias != 0).total_bytes;
 }
 
 RZ_API int rz_weight_grad_ex(const void* X, const void* dY, void* dHW, void* dbias, void* workspace,

@@ -6,4 +6,7 @@ hipError_t launch_gemm_bf16(int op, GemmParams p, const WeightGradPlan* plan, co
                            hipStream_t stream) {
   return launch_gemm_t<bf16_t>(op, p, plan, split, stream);
 }
+hipError_t launch_window_bf16(const WindowParams& p, int windows, hipStream_t stream) {
+  return launch_window_t<bf16_t>(p, windows, stream);
+}
 }  // namespace rz

@@ -6,4 +6,7 @@ hipError_t launch_gemm_f32(int op, GemmParams p, const WeightGradPlan* plan, con
                            hipStream_t stream) {
   return launch_gemm_t<float>(op, p, plan, split, stream);
 }
+hipError_t launch_window_f32(const WindowParams& p, int windows, hipStream_t stream) {
+  return launch_window_t<float>(p, windows, stream);
+}
 }  // namespace rz

@@ -3,6 +3,7 @@
 
 #include "rz_gemm.h"
 #include "rz_launch.h"
+#include "rz_window.h"
 
 namespace rz {
 
@@ -106,6 +107,30 @@ static hipError_t launch_gemm_t(int op, GemmParams p, const WeightGradPlan* plan
       return launch_op<T, 128, 2, 2, 2>(op, p, plan, split, stream);
     default: return hipErrorInvalidValue;
   }
+}
+
+template <typename T, int TBK, int TBN>
+static hipError_t launch_window_one(const WindowParams& p, int windows, hipStream_t stream) {
+  typedef WindowKernel<T, TBK, TBN> K;
+  static_assert(K::kFixedBytes + sizeof(float) * kWindowFloats <= 160 * 1024, "window does not fit the LDS");
+  if (p.window < 4 || p.window > kWindowFloats || (p.window & 3) || windows < 1) return hipErrorInvalidValue;
+  if ((long long)windows * p.window < p.H) return hipErrorInvalidValue;
+  auto kernel = rz_window_kernel<T, TBK, TBN>;
+  const size_t smem = K::kFixedBytes + sizeof(float) * (size_t)p.window;
+  if (smem > 64 * 1024) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    if (e != hipSuccess) return e;
+  }
+  hipLaunchKernelGGL(kernel, dim3((unsigned)windows), dim3(K::kThreads), smem, stream, p);
+  return hipGetLastError();
+}
+
+template <typename T>
+static hipError_t launch_window_t(const WindowParams& p, int windows, hipStream_t stream) {
+  if (p.h.BK == 64 && p.h.BN == 64) return launch_window_one<T, 64, 64>(p, windows, stream);
+  if (p.h.BK == 32 && p.h.BN == 64) return launch_window_one<T, 32, 64>(p, windows, stream);
+  return hipErrorInvalidValue;
 }
 
 }  // namespace rz

@@ -137,6 +137,47 @@ static inline WeightGradPlan plan_weight_grad(int M, int K, int N, int H, int el
   return pl;
 }
 
+// Weight-grad by windows of dHW (rz_window.h): used when hashed_weight is too large for one
+// LDS image and the contraction over M is short, so that the K*N global atomics of the scatter
+// kernel would dominate.
+struct WindowPlan {
+  bool use;
+  int window;    // elements of dHW per workgroup
+  int windows;   // workgroups
+  long long tiles;   // W tiles (entries of the offset table the kernel scans)
+};
+static constexpr int kWindowFloats = 25600;   // LDS floats a workgroup can hold next to its staging
+
+static inline bool window_tile_supported(int BK, int BN) { return BN == 64 && (BK == 64 || BK == 32); }
+
+static inline WindowPlan plan_window(int M, int K, int N, int H, int BK, int BN, int elem_bytes) {
+  WindowPlan pl = {false, 0, 0, 0};
+  const char* env = getenv("RZLINEAR_WINDOW");   // tuning aid: 0 = never, 1 = whenever possible
+  const int forced = env ? atoi(env) : -1;
+  if (forced == 0 || !window_tile_supported(BK, BN)) return pl;
+  const long long tiles = (long long)((K + BK - 1) / BK) * ((N + BN - 1) / BN);
+  if (tiles > (1 << 20)) return pl;              // every workgroup scans every tile's offset
+  pl.tiles = tiles;
+  // one workgroup per compute unit when the windows can be that large, else whole rounds
+  const long long rounds = ((long long)H + (long long)kWindowFloats * kComputeUnits - 1) /
+                           ((long long)kWindowFloats * kComputeUnits);
+  long long w = (((long long)H + rounds * kComputeUnits - 1) / (rounds * kComputeUnits) + 3) & ~3LL;
+  if (w < 1024) w = 1024;                        // tiny windows would each redo most tiles
+  pl.window = (int)w;
+  pl.windows = (int)(((long long)H + w - 1) / w);
+  // Rough times in microseconds, fitted to measurements at K = N = 10240, H = 6.5 M on MI355X.
+  // Scatter kernel: K*N atomics at about 184 G/s plus the product.  Window kernel: every
+  // workgroup works through tiles * (window + tile) / H tiles; a tile costs about 0.7 us plus
+  // 0.3 us (16-bit) or 1.2 us (fp32) per 32 rows of M.
+  const double chunks = (double)((M + 31) / 32);
+  const double per_wg = (double)tiles * ((double)w + (double)BK * BN) / (double)H;
+  const double wg_rounds = (double)((pl.windows + kComputeUnits - 1) / kComputeUnits);
+  const double t_window = wg_rounds * per_wg * (0.72 + (elem_bytes == 4 ? 1.2 : 0.32) * chunks) + 30.0;
+  const double t_scatter = 0.9 * (double)K * N / 184e3 + 2.0 * M * (double)K * N / 800e6;
+  pl.use = forced == 1 || t_window * 1.2 < t_scatter;
+  return pl;
+}
+
 // Forward / input-grad with few C tiles and a long contraction (skinny batches): R is cut into
 // slices over blockIdx.y, every slice writes an fp32 partial result, a second kernel adds them.
 struct SplitPlan {
@@ -176,5 +217,11 @@ hipError_t launch_gemm_bf16(int op, GemmParams p, const WeightGradPlan* plan, co
                             hipStream_t stream);
 hipError_t launch_gemm_f16(int op, GemmParams p, const WeightGradPlan* plan, const SplitPlan* split,
                            hipStream_t stream);
+
+struct WindowParams;
+// Enqueues the windowed weight-grad kernel; p.window and the tile grid must come from plan_window.
+hipError_t launch_window_f32(const WindowParams& p, int windows, hipStream_t stream);
+hipError_t launch_window_bf16(const WindowParams& p, int windows, hipStream_t stream);
+hipError_t launch_window_f16(const WindowParams& p, int windows, hipStream_t stream);
 
 }  // namespace rz

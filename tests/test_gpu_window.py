@@ -1,0 +1,94 @@
+"""GPU parity of the windowed weight-grad (large hashed_weight, short contraction): every
+workgroup owns a range of dHW and pulls in the tiles that touch it.  RZLINEAR_WINDOW=1 forces
+that path wherever it is possible; the last test lets the library choose it by itself."""
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import SEED_CONSTANTS, TOL, make_inputs, rargs, rel_err
+
+pytestmark = pytest.mark.gpu
+
+R1024 = SEED_CONSTANTS[1024]
+
+# (M, K, N, H, BK, BN): H too large for one LDS image in every case
+CASES = [
+    (256, 256, 512, 70000, 64, 64),
+    (32, 1024, 1024, 65536, 64, 64),
+    (50, 300, 330, 70000, 32, 64),        # ragged in M, K and N; the reference's default tile
+    (200, 512, 512, 300000, 64, 64),      # 256 windows of about 1.2 K elements
+    (31, 640, 640, 2000001, 64, 64),      # most of dHW untouched, odd H
+    (130, 192, 128, 7000000, 64, 64),     # two rounds of windows; M spans several chunks
+]
+_dt_id = lambda d: str(d).split(".")[-1]
+_shape_id = lambda s: "x".join(map(str, s))
+
+
+def _say(*a):
+    print(*a, flush=True)
+    sys.stdout.flush()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16], ids=_dt_id)
+@pytest.mark.parametrize("shape", CASES, ids=_shape_id)
+def test_windowed_weight_grad(oracle, monkeypatch, shape, dtype):
+    from rzlinear_amd.impl.RzLinearBackward import rz_linear_backward_weight_grad_tl
+    monkeypatch.setenv("RZLINEAR_WINDOW", "1")
+    M, K, N, H, BK, BN = shape
+    _say("windowed weight grad", shape, dtype)
+    (x, _, dy), (x64, _, dy64) = make_inputs(M, K, N, H, dtype, seed=31)
+    dhw = rz_linear_backward_weight_grad_tl(x, dy, 0.5, M, K, N, H, *rargs(R1024), BLOCK_SIZE_K=BK,
+                                            BLOCK_SIZE_N=BN)
+    torch.cuda.synchronize()
+    ref = oracle.weight_grad(x64, dy64, H, BK, BN, R1024, 0.5)
+    got = dhw.float().cpu().numpy()
+    assert rel_err(got, ref) <= TOL[dtype]
+    assert (got[ref == 0] == 0).all()          # slots that no tile covers stay exactly zero
+    # the summation order is fixed: a second call gives the same bits
+    again = rz_linear_backward_weight_grad_tl(x, dy, 0.5, M, K, N, H, *rargs(R1024), BLOCK_SIZE_K=BK,
+                                              BLOCK_SIZE_N=BN)
+    assert torch.equal(dhw, again)
+    # and the scatter kernel agrees
+    monkeypatch.setenv("RZLINEAR_WINDOW", "0")
+    scatter = rz_linear_backward_weight_grad_tl(x, dy, 0.5, M, K, N, H, *rargs(R1024), BLOCK_SIZE_K=BK,
+                                                BLOCK_SIZE_N=BN)
+    torch.cuda.synchronize()
+    assert rel_err(scatter.float().cpu().numpy(), ref) <= TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=_dt_id)
+def test_windowed_accumulate_and_fp32_buffer(oracle, monkeypatch, dtype):
+    from rzlinear_amd.impl.RzLinearBackward import rz_linear_backward_weight_grad_tl
+    monkeypatch.setenv("RZLINEAR_WINDOW", "1")
+    M, K, N, H, BK, BN = 64, 512, 256, 90000, 64, 64
+    _say("windowed accumulate", dtype)
+    (x, _, dy), (x64, _, dy64) = make_inputs(M, K, N, H, dtype, seed=32)
+    ref = oracle.weight_grad(x64, dy64, H, BK, BN, R1024, 1.0)
+    for odt in (dtype, torch.float32):
+        start = (torch.randn((H,), generator=torch.Generator().manual_seed(6)) * float(np.abs(ref).max())).to(odt)
+        buf = start.clone().cuda()
+        rz_linear_backward_weight_grad_tl(x, dy, 1.0, M, K, N, H, *rargs(R1024), BLOCK_SIZE_K=BK, BLOCK_SIZE_N=BN,
+                                          out=buf, accumulate=True)
+        torch.cuda.synchronize()
+        tol = TOL[odt if odt != torch.float32 else dtype]
+        assert rel_err(buf.float().cpu().numpy(), start.double().numpy() + ref) <= tol
+        buf = start.clone().cuda()
+        rz_linear_backward_weight_grad_tl(x, dy, 1.0, M, K, N, H, *rargs(R1024), BLOCK_SIZE_K=BK, BLOCK_SIZE_N=BN,
+                                          out=buf)
+        torch.cuda.synchronize()
+        assert rel_err(buf.float().cpu().numpy(), ref) <= TOL[dtype]
+
+
+def test_library_picks_the_window_path_for_skinny_batches(oracle):
+    """M = 32 against K = N = 4096 with a 2^20-element hashed_weight: no environment switch."""
+    from rzlinear_amd.impl.RzLinearBackward import rz_linear_backward_weight_grad_tl
+    M, K, N, H, BK, BN = 32, 4096, 4096, 1 << 20, 64, 64
+    _say("window path chosen by the plan")
+    (x, _, dy), (x64, _, dy64) = make_inputs(M, K, N, H, torch.bfloat16, seed=33)
+    a = rz_linear_backward_weight_grad_tl(x, dy, 1.0, M, K, N, H, *rargs(R1024), BLOCK_SIZE_K=BK, BLOCK_SIZE_N=BN)
+    b = rz_linear_backward_weight_grad_tl(x, dy, 1.0, M, K, N, H, *rargs(R1024), BLOCK_SIZE_K=BK, BLOCK_SIZE_N=BN)
+    torch.cuda.synchronize()
+    assert rel_err(a.float().cpu().numpy(), oracle.weight_grad(x64, dy64, H, BK, BN, R1024, 1.0)) <= TOL[torch.bfloat16]
+    assert torch.equal(a, b)   # deterministic, unlike the atomic scatter
