@@ -90,7 +90,7 @@ template <typename T>
 static hipError_t launch_gemm_t(int op, GemmParams p, const WeightGradPlan* plan, const SplitPlan* split,
                                 hipStream_t stream) {
   const int tile = (op == kWeightGrad && plan != nullptr) ? plan->tile
-                   : (split != nullptr ? split->tile : pick_tile(p.I, p.J));
+                   : (split != nullptr ? split->tile : pick_tile(p.I, p.J, (int)sizeof(T)));
   const char* stages_env = getenv("RZLINEAR_STAGES");
   const bool one_stage = stages_env != nullptr && atoi(stages_env) == 1;
   switch (tile) {

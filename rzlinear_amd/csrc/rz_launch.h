@@ -23,23 +23,19 @@ static inline long long tile_count(int I, int J, int t) {
   return (long long)((I + t - 1) / t) * ((J + t - 1) / t);
 }
 
-// Relative throughput of a tile shape at a given number of workgroups, from bf16 measurements
-// on MI355X (256 tile at one workgroup per compute unit = 1): the 128 tile reaches 0.51 with one
-// workgroup per compute unit and 0.75 with two or more, the 64 tile 0.16 and 0.33 (four or
-// more); below one workgroup per compute unit the rate falls with the idle compute units, and
-// a last, partly filled round of workgroups costs a full one.
-static inline double tile_score_full(int I, int J, int t);
-// ... times the share of a tile grid's MFMA work that is not padding
-static inline double tile_score(int I, int J, int t) {
-  const double wgs = (double)tile_count(I, J, t);
-  return tile_score_full(I, J, t) * ((double)I * (double)J) / (wgs * t * t);
-}
-static inline double tile_score_full(int I, int J, int t) {
+// Relative throughput of a tile shape at a given number of workgroups, from measurements on
+// MI355X (256 tile at one workgroup per compute unit = 1).  16-bit types: the 128 tile reaches
+// 0.51 with one workgroup per compute unit and 0.75 with two or more, the 64 tile 0.16 and 0.33
+// (four or more).  fp32 is bound by the slower fp32 MFMA rate, so the small tiles lose far less:
+// 0.86 / 0.90 and 0.45 / 0.80.  Below one workgroup per compute unit the rate falls with the
+// idle compute units, and a last, partly filled round of workgroups costs a full one.
+static inline double tile_score_full(int I, int J, int t, int elem_bytes) {
   const double wgs = (double)tile_count(I, J, t);
   const double per_cu = wgs / kComputeUnits;
+  const bool f32 = elem_bytes == 4;
   const int slots = (t == 256) ? 1 : (t == 128 ? 2 : 4);          // resident workgroups per CU
-  const double lo = (t == 256) ? 1.0 : (t == 128 ? 0.51 : 0.16);  // at one workgroup per CU
-  const double hi = (t == 256) ? 1.0 : (t == 128 ? 0.75 : 0.33);  // at `slots` per CU
+  const double lo = (t == 256) ? 1.0 : (t == 128 ? (f32 ? 0.86 : 0.51) : (f32 ? 0.45 : 0.16));  // one workgroup per CU
+  const double hi = (t == 256) ? 1.0 : (t == 128 ? (f32 ? 0.90 : 0.75) : (f32 ? 0.80 : 0.33));  // `slots` per CU
   if (per_cu <= 1.0) return lo * per_cu;
   const double cap = (double)kComputeUnits * slots;
   const double rounds = (double)((long long)((wgs + cap - 1) / cap));
@@ -49,14 +45,19 @@ static inline double tile_score_full(int I, int J, int t) {
   // between one and `slots` workgroups per CU every CU is busy: no tail penalty yet
   return per_cu >= slots ? e * util : e;
 }
+// ... times the share of a tile grid's MFMA work that is not padding
+static inline double tile_score(int I, int J, int t, int elem_bytes) {
+  const double wgs = (double)tile_count(I, J, t);
+  return tile_score_full(I, J, t, elem_bytes) * ((double)I * (double)J) / (wgs * t * t);
+}
 
-static inline int pick_tile(int I, int J) {
+static inline int pick_tile(int I, int J, int elem_bytes) {
   if (forced_tile()) return forced_tile();
   int best = 256;
-  double best_score = tile_score(I, J, 256);
+  double best_score = tile_score(I, J, 256, elem_bytes);
   const int others[2] = {128, 64};
   for (int t : others) {
-    const double sc = tile_score(I, J, t);
+    const double sc = tile_score(I, J, t, elem_bytes);
     if (sc > best_score * 1.02) {   // prefer the larger tile on a near tie
       best = t;
       best_score = sc;
@@ -112,7 +113,7 @@ static inline WeightGradPlan plan_weight_grad(int M, int K, int N, int H, int el
         tile_cover(K, N, 128) * 10 <= tile_cover(K, N, 256) * 13)
       pl.tile = 128;
   } else {
-    pl.tile = pick_tile(K, N);
+    pl.tile = pick_tile(K, N, elem_bytes);
   }
   const long long tiles = (long long)((K + pl.tile - 1) / pl.tile) * ((N + pl.tile - 1) / pl.tile);
   const int r_steps = (M + TR - 1) / TR;
@@ -190,7 +191,7 @@ struct SplitPlan {
 static inline SplitPlan plan_split(int I, int J, int R, int elem_bytes) {
   SplitPlan pl;
   const int TR = 128 / elem_bytes;
-  pl.tile = pick_tile(I, J);
+  pl.tile = pick_tile(I, J, elem_bytes);
   const long long tiles = tile_count(I, J, pl.tile);
   const int r_steps = (R + TR - 1) / TR;
   const int slots = (pl.tile == 256) ? 1 : (pl.tile == 128 ? 2 : 4);
