@@ -1,0 +1,95 @@
+"""The baseline configurations at their full sizes, on the GPU.
+
+The CPU oracle would take minutes there, so the check is assembled from pieces that are pinned
+elsewhere: the index map comes from the materialiser (bit-exact against the oracle in
+test_gpu_parity.py, and checked against the oracle again here at full size), the dense products
+are float64 torch.matmul on the GPU, and the reduction into hashed_weight is torch's index_add_
+— the reference tests' own design (python/tests/test_rz_linear.py:21-33,:77-90)."""
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import SEED_CONSTANTS, TOL, rargs
+
+pytestmark = pytest.mark.gpu
+
+R1024 = SEED_CONSTANTS[1024]
+
+# name -> (M, K, N, H, dtype); 64 x 64 tiles, as benchmarked
+CONFIGS = {
+    "square4096_bf16": (4096, 4096, 4096, 16778, torch.bfloat16),
+    "square4096_fp32": (4096, 4096, 4096, 16778, torch.float32),
+    "rec_mlp_bf16": (16384, 512, 1024, 5243, torch.bfloat16),
+    "ffn_bf16": (8192, 4096, 16384, 67109, torch.bfloat16),
+    "collision_fp32": (32768, 2048, 2048, 32768, torch.float32),
+}
+
+
+def _say(*a):
+    print(*a, flush=True)
+    sys.stdout.flush()
+
+
+def _rel(out, ref):
+    ref = ref.double()
+    return float((out.double() - ref).abs().max() / ref.abs().max())
+
+
+@pytest.mark.parametrize("name", sorted(CONFIGS))
+def test_baseline_configuration_at_full_size(oracle, name):
+    from rzlinear_amd.impl.RzLinearBackward import rz_linear_backward_tl
+    from rzlinear_amd.impl.RzLinearForward import rz_linear_forward_tl
+    from rzlinear_amd.impl.RzLinearIdx import rz_linear_weight_tl
+    M, K, N, H, dtype = CONFIGS[name]
+    BK = BN = 64
+    _say("full size", name)
+    g = torch.Generator().manual_seed(77)
+    x = torch.randn((M, K), generator=g).to(dtype).cuda()
+    hw = ((torch.rand((H,), generator=g) * 2 - 1) / K ** 0.5).to(dtype).cuda()
+    dy = torch.randn((M, N), generator=g).to(dtype).cuda()
+    kw = dict(BLOCK_SIZE_K=BK, BLOCK_SIZE_N=BN)
+
+    # index map: materialise arange(H) in fp32 (exact), compare with the oracle's map
+    idx = rz_linear_weight_tl(torch.arange(H, dtype=torch.float32, device="cuda"), K, N, H, *rargs(R1024), **kw).long()
+    assert np.array_equal(idx.cpu().numpy(), oracle.index_map(K, N, H, BK, BN, R1024))
+    W = hw.double()[idx]
+
+    y = rz_linear_forward_tl(x, hw, 1.0, M, K, N, H, *rargs(R1024), **kw)
+    dx, dhw = rz_linear_backward_tl(x, hw, dy, 1.0, M, K, N, H, *rargs(R1024), **kw)
+    torch.cuda.synchronize()
+    assert _rel(y, x.double() @ W) <= TOL[dtype]
+    assert _rel(dx, dy.double() @ W.t()) <= TOL[dtype]
+    dW = x.double().t() @ dy.double()
+    ref = torch.zeros((H,), dtype=torch.float64, device="cuda").index_add_(0, idx.reshape(-1), dW.reshape(-1))
+    assert _rel(dhw, ref) <= TOL[dtype]
+    # mass conservation, a check that does not go through the index map: every element of
+    # X^T.dY lands in exactly one slot
+    assert abs(float(dhw.double().sum() - dW.sum())) <= TOL[dtype] * float(dW.abs().sum()) / 10
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32], ids=lambda d: str(d).split(".")[-1])
+def test_row_pitches_that_break_16_byte_alignment(oracle, dtype):
+    """Complete tiles (the kernels without bounds checks, direct-to-LDS staging for bf16) on
+    operands whose rows start at odd element offsets."""
+    from rzlinear_amd.impl.RzLinearBackward import rz_linear_backward_tl
+    from rzlinear_amd.impl.RzLinearForward import rz_linear_forward_tl
+    M, K, N, H, BK, BN = 512, 512, 768, 9000, 64, 64
+    _say("odd row pitch", dtype)
+    g = torch.Generator().manual_seed(78)
+    xbig = torch.randn((M, K + 3), generator=g).to(dtype).cuda()
+    dybig = torch.randn((M, N + 5), generator=g).to(dtype).cuda()
+    x, dy = xbig[:, 1:K + 1], dybig[:, 3:N + 3]
+    assert x.stride(0) == K + 3 and x.data_ptr() % 16 != 0
+    hw = ((torch.rand((H + 1,), generator=g) * 2 - 1) / K ** 0.5).to(dtype).cuda()[1:]   # odd start as well
+    kw = dict(BLOCK_SIZE_K=BK, BLOCK_SIZE_N=BN)
+    y = rz_linear_forward_tl(x, hw, 1.0, M, K, N, H, *rargs(R1024), **kw)
+    dx, dhw = rz_linear_backward_tl(x, hw, dy, 1.0, M, K, N, H, *rargs(R1024), **kw)
+    torch.cuda.synchronize()
+    x64, hw64, dy64 = (t.double().cpu().numpy() for t in (x, hw, dy))
+    f = lambda t: t.float().cpu().numpy()
+    from helpers import rel_err
+    assert rel_err(f(y), oracle.forward(x64, hw64, N, BK, BN, R1024)) <= TOL[dtype]
+    assert rel_err(f(dx), oracle.input_grad(dy64, hw64, K, BK, BN, R1024)) <= TOL[dtype]
+    assert rel_err(f(dhw), oracle.weight_grad(x64, dy64, H, BK, BN, R1024)) <= TOL[dtype]
