@@ -110,8 +110,15 @@ __device__ __forceinline__ u32x4_t mask_tail(u32x4_t v, int col, int col_lim) {
 }
 
 // COLSUM (weight-grad only): also sum the columns of B (dY) for the bias gradient.
-template <typename T, int OP, int TI, int TJ, int WI, int WJ, int NSTAGE, bool FULL, bool COLSUM = false>
+// CLAMP (with FULL = false): the contracted dimension is complete (R a multiple of the R step;
+// weight-grad: any R, its last step is cleared in LDS) but the C tile grid has ragged edges.  Tiles are then still staged directly: a piece that
+// would start outside the operand is fetched from the nearest row / piece inside it (hashed
+// pieces need nothing: every tile index hashes to a valid slice).  What such a piece holds
+// only reaches rows or columns of C that the bounds-checked epilogue never stores.
+template <typename T, int OP, int TI, int TJ, int WI, int WJ, int NSTAGE, bool FULL, bool COLSUM = false,
+          bool CLAMP = false>
 struct GemmKernel {
+  static_assert(!(FULL && CLAMP), "complete tiles need no clamping");
   static_assert(!COLSUM || OP == kWeightGrad, "column sums belong to the weight-grad contraction");
   typedef ElemTraits<T> Tr;
   typedef typename Mfma<T>::Frag Frag;
@@ -127,7 +134,7 @@ struct GemmKernel {
   static_assert(WTI % 32 == 0 && WTJ % 32 == 0, "wavefront tile must be a multiple of 32");
 
   // direct-to-LDS staging (see the head of this file)
-  static constexpr bool kDirect = k16 && FULL && NSTAGE == 2 && TI >= 128 && TJ >= 128;
+  static constexpr bool kDirect = k16 && (FULL || CLAMP) && NSTAGE == 2 && TI >= 128 && TJ >= 128;
 
   template <int LAYOUT, int TX> struct Lds {
     static constexpr int kPitch = kDirect ? (LAYOUT == kRContig ? TR : TX)
@@ -454,8 +461,15 @@ struct GemmKernel {
       for (int q = 0; q < LA::kPieces; q++) {
         int row, col;
         direct_src(LA{}, A_LAYOUT, q, row, col);
-        const T* src = (A_LAYOUT == kRContig) ? gA + (int64_t)(i0 + row) * p.lda + r0 + col
-                                              : gA + (int64_t)(r0 + row) * p.lda + i0 + col;
+        // (CLAMP: rows / 16-byte columns beyond I come from the last one inside)
+        const int gi = (A_LAYOUT == kRContig) ? i0 + row : i0 + col;
+        const int ci = !CLAMP ? gi : (A_LAYOUT == kRContig) ? (gi < p.I ? gi : p.I - 1) : (gi < p.I ? gi : p.I - VEC);
+        // (CLAMP weight-grad: rows of the last, partial R step beyond R come from row R - 1 and
+        //  are cleared in LDS before they are used, see clear_tail_rows)
+        const int gr = r0 + row;
+        const int cr = (CLAMP && OP == kWeightGrad && gr >= p.R) ? p.R - 1 : gr;
+        const T* src = (A_LAYOUT == kRContig) ? gA + (int64_t)ci * p.lda + r0 + col
+                                              : gA + (int64_t)cr * p.lda + ci;
         direct_load(src, sm.a[st], q, LA::kPieces);
       }
       if constexpr (OP == kWeightGrad) {
@@ -463,7 +477,11 @@ struct GemmKernel {
         for (int q = 0; q < LB::kPieces; q++) {
           int row, col;
           direct_src(LB{}, B_LAYOUT, q, row, col);
-          direct_load(gB + (int64_t)(r0 + row) * p.ldb + j0 + col, sm.b[st], q, LB::kPieces);
+          const int gj = j0 + col;
+          const int cj = (!CLAMP || gj < p.J) ? gj : p.J - VEC;
+          const int gr = r0 + row;
+          const int cr = (CLAMP && gr >= p.R) ? p.R - 1 : gr;
+          direct_load(gB + (int64_t)cr * p.ldb + cj, sm.b[st], q, LB::kPieces);
         }
       } else {
         const OffWindow w = window(step);
@@ -479,6 +497,24 @@ struct GemmKernel {
         }
 #pragma unroll
         for (int q = 0; q < LB::kPieces; q++) direct_load(gHW + idx[q], sm.b[st], q, LB::kPieces);
+      }
+    };
+    // CLAMP weight-grad, last R step with fewer than TR rows: once every wavefront's loads of
+    // that step have landed (the caller has just passed a barrier), the rows beyond R — whole
+    // LDS rows of both operands, fetched from row R - 1 — are set to zero; a second barrier
+    // makes that visible.  Happens at most once per workgroup.
+    const int tail_rows = (CLAMP && OP == kWeightGrad) ? steps * TR - (r_end - r_begin) : 0;
+    auto clear_tail_rows = [&](int st) {
+      if constexpr (CLAMP && OP == kWeightGrad) {
+        if (tail_rows > 0) {
+          const u32x4_t z = {0u, 0u, 0u, 0u};
+          const int first = TR - tail_rows;
+          for (int i = tid; i < tail_rows * (LA::kPitch / VEC); i += kThreads)
+            *reinterpret_cast<u32x4_t*>(sm.a[st] + first * LA::kPitch + i * VEC) = z;
+          for (int i = tid; i < tail_rows * (LB::kPitch / VEC); i += kThreads)
+            *reinterpret_cast<u32x4_t*>(sm.b[st] + first * LB::kPitch + i * VEC) = z;
+          __syncthreads();
+        }
       }
     };
     // MFMAs of one R step out of LDS stage `st`; fragments are read one sub-step ahead
@@ -597,6 +633,8 @@ struct GemmKernel {
             if constexpr (kDirect) {
               // stage st has been read for the last time: refill it for step s+2
               if constexpr (decltype(do_fetch)::value) direct_issue(s + 2, st);
+              // (no refill left = the next step is the last one: it may be a partial step)
+              if constexpr (decltype(has_next)::value && !decltype(do_fetch)::value) clear_tail_rows(st ^ 1);
             }
             if constexpr (decltype(has_next)::value) frags(st ^ 1, 0, (ks + 1) & 1);
           }
@@ -640,6 +678,9 @@ struct GemmKernel {
           hash_step(3);
         }
         __syncthreads();
+        if constexpr (kDirect) {
+          if (steps == 1) clear_tail_rows(0);
+        }
         frags(0, 0, 0);
         // wavefronts w and w + 4 of a workgroup share a SIMD
         if (kThreads == 512 && wave >= 4) loop(std::true_type{});
@@ -807,9 +848,9 @@ struct GemmKernel {
   }
 };
 
-template <typename T, int OP, int TI, int TJ, int WI, int WJ, int NSTAGE, bool FULL, bool COLSUM>
+template <typename T, int OP, int TI, int TJ, int WI, int WJ, int NSTAGE, bool FULL, bool COLSUM, bool CLAMP>
 __global__ __launch_bounds__(64 * WI * WJ) void rz_gemm_kernel(GemmParams p) {
-  typedef GemmKernel<T, OP, TI, TJ, WI, WJ, NSTAGE, FULL, COLSUM> K;
+  typedef GemmKernel<T, OP, TI, TJ, WI, WJ, NSTAGE, FULL, COLSUM, CLAMP> K;
   extern __shared__ __attribute__((aligned(16))) unsigned char rz_smem_raw[];
   K::run(p, *reinterpret_cast<typename K::Smem*>(rz_smem_raw));
 }

@@ -7,10 +7,10 @@
 
 namespace rz {
 
-template <typename T, int OP, int TI, int TJ, int WI, int WJ, int NSTAGE, bool FULL, bool COLSUM>
+template <typename T, int OP, int TI, int TJ, int WI, int WJ, int NSTAGE, bool FULL, bool COLSUM, bool CLAMP = false>
 static hipError_t launch_one(GemmParams p, const WeightGradPlan* plan, const SplitPlan* split,
                              hipStream_t stream) {
-  typedef GemmKernel<T, OP, TI, TJ, WI, WJ, NSTAGE, FULL, COLSUM> K;
+  typedef GemmKernel<T, OP, TI, TJ, WI, WJ, NSTAGE, FULL, COLSUM, CLAMP> K;
   p.tiles_i = (p.I + TI - 1) / TI;
   p.tiles_j = (p.J + TJ - 1) / TJ;
   const long long tiles = (long long)p.tiles_i * p.tiles_j;
@@ -37,7 +37,7 @@ static hipError_t launch_one(GemmParams p, const WeightGradPlan* plan, const Spl
     p.r_chunk = r_steps * K::TR;
     p.partial = nullptr;
   }
-  auto kernel = rz_gemm_kernel<T, OP, TI, TJ, WI, WJ, NSTAGE, FULL, COLSUM>;
+  auto kernel = rz_gemm_kernel<T, OP, TI, TJ, WI, WJ, NSTAGE, FULL, COLSUM, CLAMP>;
   size_t smem = sizeof(typename K::Smem);
   static_assert(sizeof(typename K::Smem) <= 160 * 1024, "tile does not fit the 160 KB LDS of a compute unit");
   if (OP == kWeightGrad && p.image_pitch > 0) {
@@ -62,6 +62,16 @@ static hipError_t launch_tile(GemmParams p, const WeightGradPlan* plan, const Sp
   constexpr int TR = 128 / ElemTraits<T>::kBytes;
   const bool full = (p.I % TILE == 0) && (p.J % TILE == 0) && (p.R % TR == 0);
   if (full) return launch_one<T, OP, TILE, TILE, WI, WJ, NSTAGE, true, COLSUM>(p, plan, split, stream);
+  // Ragged tile grid but a complete contracted dimension: 16-bit tiles can still be staged
+  // directly, with edge pieces fetched from inside the operand (weight-grad: the plain operands'
+  // 16-byte pieces must not straddle their row ends).
+  if constexpr (sizeof(T) == 2 && NSTAGE == 2 && TILE >= 128) {
+    constexpr int VEC = ElemTraits<T>::kVec;
+    const bool pieces_ok = OP != kWeightGrad || (p.I % VEC == 0 && p.J % VEC == 0 && p.I >= VEC && p.J >= VEC);
+    // (weight-grad clears the rows of a partial last R step in LDS, so any R will do there)
+    if ((p.R % TR == 0 || OP == kWeightGrad) && pieces_ok && getenv("RZLINEAR_NO_CLAMP") == nullptr)
+      return launch_one<T, OP, TILE, TILE, WI, WJ, NSTAGE, false, COLSUM, true>(p, plan, split, stream);
+  }
   return launch_one<T, OP, TILE, TILE, WI, WJ, NSTAGE, false, COLSUM>(p, plan, split, stream);
 }
 

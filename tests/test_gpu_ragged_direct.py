@@ -1,0 +1,68 @@
+"""Ragged tile grids with a complete contracted dimension: the 16-bit kernels keep their direct
+global-to-LDS staging and fetch edge pieces from inside the operands.  Checked against the CPU
+oracle for every op, both large tiles, with and without the bias-gradient column sums."""
+import sys
+
+import pytest
+import torch
+
+from helpers import SEED_CONSTANTS, TOL, make_inputs, rargs, rel_err
+
+pytestmark = pytest.mark.gpu
+
+R1024 = SEED_CONSTANTS[1024]
+
+# (M, K, N, H, BK, BN)
+CASES = [
+    (1000, 512, 1000, 9000, 64, 64),     # forward contracts K = 8 steps; M, N ragged
+    (1000, 1000, 512, 9000, 64, 64),     # input-grad contracts N
+    (1024, 1000, 520, 9000, 64, 64),     # weight-grad contracts M; K, N multiples of 8 only
+    (320, 136, 264, 70000, 32, 64),      # one ragged tile each way, atomic scatter
+    (640, 1001, 520, 9000, 64, 64),      # K not a multiple of 8: weight-grad must use the checked kernel
+    (129, 128, 129, 3000, 16, 16),       # a single row / column beyond a tile
+    (1000, 512, 520, 9000, 64, 64),      # weight-grad: the last of 16 R steps holds 40 rows
+    (70, 256, 256, 9000, 64, 64),        # two R steps, the second with 6 rows
+    (40, 256, 384, 9000, 64, 64),        # a single, partial R step
+    (4100, 192, 160, 30000, 64, 64),     # sliced M: only the last slice ends in a partial step
+    (65, 1024, 1024, 200000, 64, 64),    # one row into the second step, atomic scatter
+]
+_id = lambda s: "x".join(map(str, s))
+
+
+def _say(*a):
+    print(*a, flush=True)
+    sys.stdout.flush()
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=lambda d: str(d).split(".")[-1])
+@pytest.mark.parametrize("tile", ["128", "256"])
+@pytest.mark.parametrize("shape", CASES, ids=_id)
+def test_ragged_edges_with_direct_staging(oracle, monkeypatch, shape, tile, dtype):
+    from rzlinear_amd.impl.RzLinearBackward import (rz_linear_backward_input_grad_tl,
+                                                    rz_linear_backward_weight_bias_grad_tl,
+                                                    rz_linear_backward_weight_grad_tl)
+    from rzlinear_amd.impl.RzLinearForward import rz_linear_forward_bias_tl
+    monkeypatch.setenv("RZLINEAR_TILE", tile)
+    M, K, N, H, BK, BN = shape
+    _say("ragged direct", shape, tile, dtype)
+    (x, hw, dy), (x64, hw64, dy64) = make_inputs(M, K, N, H, dtype, seed=41)
+    bias = torch.linspace(-1, 1, N).to(dtype).cuda()
+    kw = dict(BLOCK_SIZE_K=BK, BLOCK_SIZE_N=BN)
+    y = rz_linear_forward_bias_tl(x, hw, bias, 1.0, M, K, N, H, *rargs(R1024), **kw)
+    dx = rz_linear_backward_input_grad_tl(dy, hw, 1.0, M, K, N, H, *rargs(R1024), **kw)
+    dhw = rz_linear_backward_weight_grad_tl(x, dy, 1.0, M, K, N, H, *rargs(R1024), **kw)
+    dhw2, dbias = rz_linear_backward_weight_bias_grad_tl(x, dy, 1.0, M, K, N, H, *rargs(R1024), **kw)
+    torch.cuda.synchronize()
+    f = lambda t: t.float().cpu().numpy()
+    assert rel_err(f(y), oracle.forward(x64, hw64, N, BK, BN, R1024) + bias.double().cpu().numpy()) <= TOL[dtype]
+    assert rel_err(f(dx), oracle.input_grad(dy64, hw64, K, BK, BN, R1024)) <= TOL[dtype]
+    ref = oracle.weight_grad(x64, dy64, H, BK, BN, R1024)
+    assert rel_err(f(dhw), ref) <= TOL[dtype]
+    assert rel_err(f(dhw2), ref) <= TOL[dtype]
+    assert rel_err(f(dbias), dy64.sum(axis=0)) <= TOL[dtype]
+    # the bounds-checked kernels give the same results
+    monkeypatch.setenv("RZLINEAR_NO_CLAMP", "1")
+    y2 = rz_linear_forward_bias_tl(x, hw, bias, 1.0, M, K, N, H, *rargs(R1024), **kw)
+    dx2 = rz_linear_backward_input_grad_tl(dy, hw, 1.0, M, K, N, H, *rargs(R1024), **kw)
+    torch.cuda.synchronize()
+    assert torch.equal(y, y2) and torch.equal(dx, dx2)
