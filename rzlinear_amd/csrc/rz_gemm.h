@@ -1,15 +1,16 @@
 // One MFMA-tiled kernel template for the three RzLinear contractions on gfx950.
 //
 // A workgroup of WI*WJ wavefronts owns a TI x TJ tile of C and walks the contracted
-// dimension R in steps of TR (128 bytes of R per step).  Per step the A and B tiles go
-// global -> registers (issued one or two steps ahead) -> LDS (one or two stages) -> MFMA
-// fragments.  The hashed operand
-// (W) is fetched as 16-byte pieces of hashed_weight at off(tk,tn) + kk*BN + nn; the pieces may
-// start at any element, so the loads are unaligned and rely on the hardware's unaligned
-// global access.  Tile offsets are hashed by a few threads into a small LDS table, several
-// steps ahead of their use, so the integer modulos stay off the critical path.
+// dimension R in steps of TR (128 bytes of R per step).  Per step the A and B tiles are staged
+// in LDS and read from there as MFMA fragments.  The hashed operand (W) is fetched as 16-byte
+// pieces of hashed_weight at off(tk,tn) + kk*BN + nn; the pieces may start at any element, so
+// the loads are unaligned and rely on the hardware's unaligned global access.  Tile offsets
+// are hashed by a few threads into a small LDS table, several steps ahead of their use, so
+// the integer modulos stay off the critical path.
 //
-// LDS layouts (X = I or J extent of the operand)
+// Register staging (fp32, the 64 tile, ragged contracted dimension): global -> registers (issued
+// one or two steps ahead) -> LDS (one or two stages).  LDS layouts (X = I or J extent of the
+// operand)
 //   16-bit, R contiguous in the source : [X][TR + 8]   fragment = one ds_read_b128 per lane
 //   16-bit, X contiguous in the source : [TR][X + 32]  fragment = two ds_read_b64_tr_b16
 //       (the LDS transpose read returns, to lane c of a 16-lane group, column c of a 4 x 16
@@ -18,7 +19,8 @@
 //   fp32                                : [TR][X + pad], one ds_read_b32 per lane; a source
 //       with R contiguous is transposed while it is written (pad 1), else copied (pad 4)
 //
-// Direct staging (16-bit types, complete tiles, two stages): the tiles go global -> LDS with
+// Direct staging (16-bit types, 128 and 256 tiles, two stages; complete tiles, or ragged ones
+// with CLAMP below): the tiles go global -> LDS with
 // direct-to-LDS loads, no registers and no LDS write instructions in between.  Such a load
 // puts the 64 lanes' 16-byte pieces at consecutive LDS addresses, so rows cannot be padded;
 // the stages are unpadded and swizzled instead, and the swizzle is applied on the global side
