@@ -112,8 +112,9 @@ __device__ __forceinline__ u32x4_t mask_tail(u32x4_t v, int col, int col_lim) {
 }
 
 // COLSUM (weight-grad only): also sum the columns of B (dY) for the bias gradient.
-// CLAMP (with FULL = false): the contracted dimension is complete (R a multiple of the R step;
-// weight-grad: any R, its last step is cleared in LDS) but the C tile grid has ragged edges.  Tiles are then still staged directly: a piece that
+// CLAMP (with FULL = false): ragged shapes.  The last R step may be partial (its excess is
+// cleared in LDS; where R is contiguous in an operand it must be a multiple of the 16-byte
+// piece) and the C tile grid may have ragged edges.  Tiles are then still staged directly: a piece that
 // would start outside the operand is fetched from the nearest row / piece inside it (hashed
 // pieces need nothing: every tile index hashes to a valid slice).  What such a piece holds
 // only reaches rows or columns of C that the bounds-checked epilogue never stores.
@@ -467,10 +468,14 @@ struct GemmKernel {
         const int gi = (A_LAYOUT == kRContig) ? i0 + row : i0 + col;
         const int ci = !CLAMP ? gi : (A_LAYOUT == kRContig) ? (gi < p.I ? gi : p.I - 1) : (gi < p.I ? gi : p.I - VEC);
         // (CLAMP weight-grad: rows of the last, partial R step beyond R come from row R - 1 and
-        //  are cleared in LDS before they are used, see clear_tail_rows)
+        //  are cleared in LDS before they are used, see clear_tail)
         const int gr = r0 + row;
         const int cr = (CLAMP && OP == kWeightGrad && gr >= p.R) ? p.R - 1 : gr;
-        const T* src = (A_LAYOUT == kRContig) ? gA + (int64_t)ci * p.lda + r0 + col
+        // (CLAMP forward / input-grad: pieces of the last, partial R step beyond R come from the
+        //  last piece inside and are cleared in LDS as well)
+        const int gc = r0 + col;
+        const int cc = (CLAMP && gc >= p.R) ? p.R - VEC : gc;
+        const T* src = (A_LAYOUT == kRContig) ? gA + (int64_t)ci * p.lda + cc
                                               : gA + (int64_t)cr * p.lda + ci;
         direct_load(src, sm.a[st], q, LA::kPieces);
       }
@@ -501,20 +506,33 @@ struct GemmKernel {
         for (int q = 0; q < LB::kPieces; q++) direct_load(gHW + idx[q], sm.b[st], q, LB::kPieces);
       }
     };
-    // CLAMP weight-grad, last R step with fewer than TR rows: once every wavefront's loads of
-    // that step have landed (the caller has just passed a barrier), the rows beyond R — whole
-    // LDS rows of both operands, fetched from row R - 1 — are set to zero; a second barrier
-    // makes that visible.  Happens at most once per workgroup.
-    const int tail_rows = (CLAMP && OP == kWeightGrad) ? steps * TR - (r_end - r_begin) : 0;
-    auto clear_tail_rows = [&](int st) {
-      if constexpr (CLAMP && OP == kWeightGrad) {
-        if (tail_rows > 0) {
+    // CLAMP, last R step with fewer than TR elements of R: once every wavefront's loads of that
+    // step have landed (the caller has just passed a barrier), the part of both stages beyond R
+    // — fetched from inside the operands, or from tiles beyond the tile grid — is set to zero:
+    // whole rows where X is contiguous, the trailing 16-byte pieces of every row where R is
+    // (R is then a multiple of the piece width).  A second barrier makes that visible.  Happens
+    // at most once per workgroup.
+    const int tail = CLAMP ? steps * TR - (r_end - r_begin) : 0;
+    auto clear_tail = [&](int st) {
+      if constexpr (CLAMP) {
+        if (tail > 0) {
           const u32x4_t z = {0u, 0u, 0u, 0u};
-          const int first = TR - tail_rows;
-          for (int i = tid; i < tail_rows * (LA::kPitch / VEC); i += kThreads)
-            *reinterpret_cast<u32x4_t*>(sm.a[st] + first * LA::kPitch + i * VEC) = z;
-          for (int i = tid; i < tail_rows * (LB::kPitch / VEC); i += kThreads)
-            *reinterpret_cast<u32x4_t*>(sm.b[st] + first * LB::kPitch + i * VEC) = z;
+          auto clear = [&](auto L, int layout, T* stage) {
+            typedef decltype(L) LL;
+            if (layout == kRStrided) {
+              const int first = TR - tail;
+              for (int i = tid; i < tail * (LL::kPitch / VEC); i += kThreads)
+                *reinterpret_cast<u32x4_t*>(stage + first * LL::kPitch + i * VEC) = z;
+            } else {
+              const int pieces = tail / VEC, first = TR / VEC - pieces;
+              for (int i = tid; i < LL::kRows * pieces; i += kThreads) {
+                const int row = i / pieces, pz = first + i % pieces;
+                *reinterpret_cast<u32x4_t*>(stage + row * LL::kPitch + ((pz ^ ((row >> 1) & 7)) << 3)) = z;
+              }
+            }
+          };
+          clear(LA{}, A_LAYOUT, sm.a[st]);
+          clear(LB{}, B_LAYOUT, sm.b[st]);
           __syncthreads();
         }
       }
@@ -636,7 +654,7 @@ struct GemmKernel {
               // stage st has been read for the last time: refill it for step s+2
               if constexpr (decltype(do_fetch)::value) direct_issue(s + 2, st);
               // (no refill left = the next step is the last one: it may be a partial step)
-              if constexpr (decltype(has_next)::value && !decltype(do_fetch)::value) clear_tail_rows(st ^ 1);
+              if constexpr (decltype(has_next)::value && !decltype(do_fetch)::value) clear_tail(st ^ 1);
             }
             if constexpr (decltype(has_next)::value) frags(st ^ 1, 0, (ks + 1) & 1);
           }
@@ -681,7 +699,7 @@ struct GemmKernel {
         }
         __syncthreads();
         if constexpr (kDirect) {
-          if (steps == 1) clear_tail_rows(0);
+          if (steps == 1) clear_tail(0);
         }
         frags(0, 0, 0);
         // wavefronts w and w + 4 of a workgroup share a SIMD

@@ -62,14 +62,14 @@ static hipError_t launch_tile(GemmParams p, const WeightGradPlan* plan, const Sp
   constexpr int TR = 128 / ElemTraits<T>::kBytes;
   const bool full = (p.I % TILE == 0) && (p.J % TILE == 0) && (p.R % TR == 0);
   if (full) return launch_one<T, OP, TILE, TILE, WI, WJ, NSTAGE, true, COLSUM>(p, plan, split, stream);
-  // Ragged tile grid but a complete contracted dimension: 16-bit tiles can still be staged
-  // directly, with edge pieces fetched from inside the operand (weight-grad: the plain operands'
-  // 16-byte pieces must not straddle their row ends).
+  // Ragged shapes: 16-bit tiles can still be staged directly, with edge pieces fetched from
+  // inside the operands.  A plain operand's 16-byte pieces must not straddle the end of its
+  // rows: forward / input-grad need R, weight-grad needs I and J, to be multiples of the piece.
   if constexpr (sizeof(T) == 2 && NSTAGE == 2 && TILE >= 128) {
     constexpr int VEC = ElemTraits<T>::kVec;
-    const bool pieces_ok = OP != kWeightGrad || (p.I % VEC == 0 && p.J % VEC == 0 && p.I >= VEC && p.J >= VEC);
-    // (weight-grad clears the rows of a partial last R step in LDS, so any R will do there)
-    if ((p.R % TR == 0 || OP == kWeightGrad) && pieces_ok && getenv("RZLINEAR_NO_CLAMP") == nullptr)
+    const bool pieces_ok = OP == kWeightGrad ? (p.I % VEC == 0 && p.J % VEC == 0 && p.I >= VEC && p.J >= VEC)
+                                             : (p.R % VEC == 0 && p.R >= VEC);
+    if (pieces_ok && getenv("RZLINEAR_NO_CLAMP") == nullptr)
       return launch_one<T, OP, TILE, TILE, WI, WJ, NSTAGE, false, COLSUM, true>(p, plan, split, stream);
   }
   return launch_one<T, OP, TILE, TILE, WI, WJ, NSTAGE, false, COLSUM>(p, plan, split, stream);

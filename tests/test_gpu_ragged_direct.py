@@ -1,6 +1,7 @@
-"""Ragged tile grids with a complete contracted dimension: the 16-bit kernels keep their direct
-global-to-LDS staging and fetch edge pieces from inside the operands.  Checked against the CPU
-oracle for every op, both large tiles, with and without the bias-gradient column sums."""
+"""Ragged shapes: the 16-bit kernels keep their direct global-to-LDS staging, fetch edge pieces
+from inside the operands and clear the excess of a partial last contraction step in LDS.
+Checked against the CPU oracle for every op, both large tiles, with and without the
+bias-gradient column sums."""
 import sys
 
 import pytest
@@ -25,6 +26,9 @@ CASES = [
     (40, 256, 384, 9000, 64, 64),        # a single, partial R step
     (4100, 192, 160, 30000, 64, 64),     # sliced M: only the last slice ends in a partial step
     (65, 1024, 1024, 200000, 64, 64),    # one row into the second step, atomic scatter
+    (300, 72, 200, 9000, 16, 16),        # forward: one complete R step and one piece of the next
+    (256, 8, 136, 3000, 16, 16),         # forward: a single R step holding one piece
+    (200, 264, 8, 3000, 32, 64),         # input-grad: the same
 ]
 _id = lambda s: "x".join(map(str, s))
 
