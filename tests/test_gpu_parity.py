@@ -286,3 +286,50 @@ def test_random_shapes_fp32(oracle, shape):
     assert rel_err(y.cpu().numpy(), oracle.forward(x64, hw64, N, BK, BN, R, 1.5)) <= 1e-4
     assert rel_err(dx.cpu().numpy(), oracle.input_grad(dy64, hw64, K, BK, BN, R, 1.5)) <= 1e-4
     assert rel_err(dhw.cpu().numpy(), oracle.weight_grad(x64, dy64, H, BK, BN, R, 1.5)) <= 1e-4
+
+
+def _random_cases_16bit(n, seed):
+    """Shapes for the 16-bit kernels: larger than the fp32 sweep (so that the 128 and 256 tiles
+    with direct staging are picked), mostly multiples of 8 (edge-clamped staging), some
+    multiples of 64 or 256 (no bounds checks), some odd (bounds-checked register staging)."""
+    rng = np.random.default_rng(seed)
+    cases = []
+    for _ in range(n):
+        BK, BN = (int(2 ** rng.integers(4, 8)) for _ in range(2))
+        kind = rng.random()
+        if kind < 0.5:
+            M, K, N = (8 * int(rng.integers(1, 160)) for _ in range(3))
+        elif kind < 0.7:
+            M, K, N = (64 * int(rng.integers(1, 20)) for _ in range(3))
+        elif kind < 0.8:
+            M, K, N = (256 * int(rng.integers(1, 5)) for _ in range(3))
+        else:
+            M, K, N = (int(rng.integers(1, 1300)) for _ in range(3))
+        H = BK * BN + int(rng.integers(1, 120000))
+        cases.append((M, K, N, H, BK, BN))
+    return cases
+
+
+@pytest.mark.parametrize("shape", _random_cases_16bit(40, 4242), ids=lambda s: "x".join(map(str, s)))
+def test_random_shapes_16bit(oracle, shape):
+    """Seeded random shapes for bf16 (even cases) and fp16 (odd cases), with the bias and the
+    bias gradient in the same calls."""
+    from rzlinear_amd.impl.RzLinearBackward import (rz_linear_backward_input_grad_tl,
+                                                    rz_linear_backward_weight_bias_grad_tl)
+    from rzlinear_amd.impl.RzLinearForward import rz_linear_forward_bias_tl
+    M, K, N, H, BK, BN = shape
+    dtype = torch.bfloat16 if (M + K + N) % 2 == 0 else torch.float16
+    _say("random 16-bit", shape, dtype)
+    (x, hw, dy), (x64, hw64, dy64) = make_inputs(M, K, N, H, dtype, seed=M + 3 * K + 5 * N)
+    bias = torch.linspace(-2, 2, N).to(dtype).cuda()
+    R = SEED_CONSTANTS[0]
+    kw = dict(BLOCK_SIZE_K=BK, BLOCK_SIZE_N=BN)
+    y = rz_linear_forward_bias_tl(x, hw, bias, 0.75, M, K, N, H, *rargs(R), **kw)
+    dx = rz_linear_backward_input_grad_tl(dy, hw, 0.75, M, K, N, H, *rargs(R), **kw)
+    dhw, dbias = rz_linear_backward_weight_bias_grad_tl(x, dy, 0.75, M, K, N, H, *rargs(R), **kw)
+    torch.cuda.synchronize()
+    f = lambda t: t.float().cpu().numpy()
+    assert rel_err(f(y), oracle.forward(x64, hw64, N, BK, BN, R, 0.75) + bias.double().cpu().numpy()) <= TOL[dtype]
+    assert rel_err(f(dx), oracle.input_grad(dy64, hw64, K, BK, BN, R, 0.75)) <= TOL[dtype]
+    assert rel_err(f(dhw), oracle.weight_grad(x64, dy64, H, BK, BN, R, 0.75)) <= TOL[dtype]
+    assert rel_err(f(dbias), dy64.sum(axis=0)) <= TOL[dtype]
