@@ -138,7 +138,9 @@ int rz_input_grad_ws(const void* dY, const void* HW, void* dX, void* workspace,
  * When hashed_weight is small enough for an fp32 image of dHW to fit the LDS of a compute
  * unit, every workgroup stores one partial image ([workgroups][H rounded up to 4] floats) that
  * a second kernel adds up; otherwise the 16-bit types need an fp32 image of dHW (H floats)
- * for the atomic adds and fp32 needs nothing.
+ * for the atomic adds and fp32 needs nothing — unless M is small against K*N, when dHW is
+ * computed in windows (no atomics) and the workspace holds one int32 offset per W tile.
+ * The size depends on M: ask again when the batch size changes.
  */
 size_t rz_weight_grad_workspace_bytes(int M, int K, int N, int H, int BK, int BN, int dtype);
 

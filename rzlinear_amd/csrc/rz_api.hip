@@ -270,7 +270,8 @@ static void launch_reduce_colsum(int out_dtype, const float* part, void* out, in
 static inline size_t round256(size_t b) { return (b + 255) & ~(size_t)255; }
 
 // Workspace layout of a weight-grad call: [main][column sums].  main = the partial images (LDS
-// image mode) or, for the atomic scatter into a 16-bit dHW, its fp32 image.
+// image mode), the table of tile offsets (window kernel) or, for the atomic scatter into a
+// 16-bit dHW, its fp32 image.
 struct WeightGradWorkspace {
   size_t main_bytes, total_bytes;
 };
@@ -377,7 +378,7 @@ extern "C" {
 
 #define RZ_API __attribute__((visibility("default")))
 
-RZ_API int rz_version(void) { return 100; }
+RZ_API int rz_version(void) { return 200; }
 
 RZ_API const char* rz_status_string(int status) {
   switch (status) {
