@@ -26,6 +26,7 @@
 // the stages are unpadded and swizzled instead, and the swizzle is applied on the global side
 // (each lane fetches the piece that belongs at its LDS slot):
 //   R contiguous : [X][TR], row = 8 pieces; piece p of row x sits at slot p ^ ((x >> 1) & 7)
+//                  (16 pieces with the 256-byte R step: slot p ^ (x & 15))
 //   X contiguous : [TR][X], row = X/32 chunks of 64 bytes; chunk c of row r sits at c ^ (r & 3)
 // Both keep the fragment reads above free of bank conflicts.
 #pragma once
@@ -128,7 +129,15 @@ struct GemmKernel {
   static constexpr int kThreads = 64 * WI * WJ;
   static constexpr int VEC = Tr::kVec;
   static constexpr bool k16 = (Tr::kBytes == 2);
-  static constexpr int TR = 128 / Tr::kBytes;
+  // R step: 128 bytes of R — except the directly staged 128 tile with eight wavefronts, which
+  // is used at about one workgroup per compute unit and has LDS to spare: it takes 256 bytes
+  // per step, halving the barriers per flop (8 % faster at 2048^3).
+  static constexpr bool kLongStep = Tr::kBytes == 2 && (FULL || CLAMP) && NSTAGE == 2 && TI == 128 && TJ == 128 &&
+                                    WI * WJ == 8;
+  static constexpr int TR = (kLongStep ? 256 : 128) / Tr::kBytes;
+  static constexpr int kPpr = TR / (16 / Tr::kBytes);   // 16-byte pieces per R-contiguous row (8 or 16)
+  // swizzle of an R-contiguous direct stage: piece p of row x sits at slot p ^ row_swizzle(x)
+  static __device__ __forceinline__ int row_swizzle(int row) { return kPpr == 16 ? (row & 15) : ((row >> 1) & 7); }
   static constexpr int KS = Tr::kMfmaK;
   static constexpr int A_LAYOUT = (OP == kWeightGrad) ? kRStrided : kRContig;
   static constexpr int B_LAYOUT = (OP == kInputGrad) ? kRContig : kRStrided;
@@ -197,7 +206,7 @@ struct GemmKernel {
     } else if constexpr (LAYOUT == kRContig) {
       const int row = x_base + (lane & 31), piece = ks * 2 + (lane >> 5);
       if constexpr (kDirect)
-        return *reinterpret_cast<const u32x4_t*>(lds + row * L::kPitch + ((piece ^ ((row >> 1) & 7)) << 3));
+        return *reinterpret_cast<const u32x4_t*>(lds + row * L::kPitch + ((piece ^ row_swizzle(row)) << 3));
       return *reinterpret_cast<const u32x4_t*>(lds + row * L::kPitch + piece * 8);
     } else {
       const int g = lane >> 4, jl = lane & 15;
@@ -440,8 +449,8 @@ struct GemmKernel {
       typedef decltype(L) LL;
       const int n = wave * LL::kPieces + q;
       if (layout == kRContig) {
-        row = n * 8 + (lane >> 3);
-        col = ((lane & 7) ^ ((row >> 1) & 7)) * 8;
+        row = n * (64 / kPpr) + lane / kPpr;
+        col = ((lane % kPpr) ^ row_swizzle(row)) * 8;
       } else {
         constexpr int kSlots = LL::kPitch / 8;          // 16-byte slots per row
         row = n * (64 / kSlots) + lane / kSlots;
@@ -527,7 +536,7 @@ struct GemmKernel {
               const int pieces = tail / VEC, first = TR / VEC - pieces;
               for (int i = tid; i < LL::kRows * pieces; i += kThreads) {
                 const int row = i / pieces, pz = first + i % pieces;
-                *reinterpret_cast<u32x4_t*>(stage + row * LL::kPitch + ((pz ^ ((row >> 1) & 7)) << 3)) = z;
+                *reinterpret_cast<u32x4_t*>(stage + row * LL::kPitch + ((pz ^ row_swizzle(row)) << 3)) = z;
               }
             }
           };

@@ -59,8 +59,11 @@ static hipError_t launch_one(GemmParams p, const WeightGradPlan* plan, const Spl
 template <typename T, int OP, int TILE, int WI, int WJ, int NSTAGE, bool COLSUM = false>
 static hipError_t launch_tile(GemmParams p, const WeightGradPlan* plan, const SplitPlan* split,
                               hipStream_t stream) {
-  constexpr int TR = 128 / ElemTraits<T>::kBytes;
-  const bool full = (p.I % TILE == 0) && (p.J % TILE == 0) && (p.R % TR == 0);
+  // (the unchecked kernel's R step; every slice of a split contraction must be whole steps too)
+  constexpr int TR = GemmKernel<T, OP, TILE, TILE, WI, WJ, NSTAGE, true>::TR;
+  const int chunk = (OP == kWeightGrad) ? (plan != nullptr ? plan->r_chunk : p.R)
+                                        : (split != nullptr && split->splits > 1 ? split->r_chunk : p.R);
+  const bool full = (p.I % TILE == 0) && (p.J % TILE == 0) && (p.R % TR == 0) && (chunk % TR == 0);
   if (full) return launch_one<T, OP, TILE, TILE, WI, WJ, NSTAGE, true, COLSUM>(p, plan, split, stream);
   // Ragged shapes: 16-bit tiles can still be staged directly, with edge pieces fetched from
   // inside the operands.  A plain operand's 16-byte pieces must not straddle the end of its
