@@ -15,8 +15,10 @@ module; the product package never does.  Two independent restatements live here:
 Parity status: pinned.  The reference holds no golden vectors for the two-level hash, so they
 were produced once by running its own Triton kernels under Triton's CPU interpreter
 (tests/golden/make_reference_vectors.py -> tests/golden/reference_vectors.npz); both
-restatements agree with them to fp32 rounding, and tests/test_oracle.py adds known-answer and
-invariant tests and checks the two restatements against each other.
+restatements agree with them to fp32 rounding (and with fp16 vectors made the same way,
+tests/golden/reference_vectors_16bit.npz, to fp16 rounding), and tests/test_oracle.py adds
+known-answer and invariant tests and checks the two restatements against each other.  The
+reference's bf16 behaviour is unpinned: the interpreter does not run bf16.
 """
 import ctypes
 import os

@@ -174,6 +174,31 @@ def test_kernels_match_vectors_produced_by_the_reference_kernels():
         assert rel_err(dhw.cpu().numpy(), d[name + "_dhw"]) <= 1e-4
 
 
+def test_fp16_kernels_match_fp16_vectors_produced_by_the_reference_kernels():
+    """fp16 HIP kernels against the reference's own kernels on fp16 tensors
+    (tests/golden/reference_vectors_16bit.npz).  Both accumulate the products in fp32 and round
+    the output once, so they may differ by an fp16 rounding; the reference adds the weight
+    gradient atomically in fp16, this build in fp32."""
+    import os
+    from rzlinear_amd.impl.RzLinearBackward import (rz_linear_backward_input_grad_tl,
+                                                    rz_linear_backward_weight_grad_tl)
+    from rzlinear_amd.impl.RzLinearForward import rz_linear_forward_tl
+    d = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "reference_vectors_16bit.npz"))
+    R = d["R"].tolist()
+    for name in "hi":
+        M, K, N, H, BK, BN = [int(v) for v in d[name + "_shape"]]
+        f = float(d[name + "_f"])
+        _say("reference fp16 vectors", name, (M, K, N, H, BK, BN))
+        x, hw, dy = (torch.from_numpy(d[name + s]).half().cuda() for s in ("_x", "_hw", "_dy"))
+        y = rz_linear_forward_tl(x, hw, f, M, K, N, H, *rargs(R), BLOCK_SIZE_K=BK, BLOCK_SIZE_N=BN)
+        dx = rz_linear_backward_input_grad_tl(dy, hw, f, M, K, N, H, *rargs(R), BLOCK_SIZE_K=BK, BLOCK_SIZE_N=BN)
+        dhw = rz_linear_backward_weight_grad_tl(x, dy, f, M, K, N, H, *rargs(R), BLOCK_SIZE_K=BK, BLOCK_SIZE_N=BN)
+        torch.cuda.synchronize()
+        assert rel_err(y.float().cpu().numpy(), d[name + "_y"]) <= 1e-3
+        assert rel_err(dx.float().cpu().numpy(), d[name + "_dx"]) <= 1e-3
+        assert rel_err(dhw.float().cpu().numpy(), d[name + "_dhw"]) <= 2e-3
+
+
 @pytest.mark.parametrize("dtype", DTYPES, ids=lambda d: str(d).split(".")[-1])
 def test_module_forward_backward_with_fused_bias(oracle, dtype):
     """The nn.Module end to end: N-D input, bias fused into the forward kernel, all gradients."""

@@ -271,6 +271,25 @@ def test_oracle_matches_vectors_produced_by_the_reference_kernels(oracle):
                 assert np.abs(ref - got).max() <= 2e-6 * np.abs(got).max()
 
 
+def test_oracle_against_fp16_vectors_of_the_reference_kernels(oracle):
+    """tests/golden/reference_vectors_16bit.npz: the reference's kernels on fp16 tensors (Triton's
+    CPU interpreter; it does not support bf16).  The float64 oracle on the same fp16 inputs must
+    agree to fp16 rounding: the reference accumulates tl.dot in fp32 and rounds the output once
+    (measured 2.4e-4 .. 4.0e-4), and adds the weight gradient atomically in fp16 (<= 7.6e-4)."""
+    d = np.load(os.path.join(GOLDEN, "reference_vectors_16bit.npz"))
+    R = d["R"].tolist()
+    for name in "hi":
+        assert str(d[name + "_dtype"]) == "float16"
+        M, K, N, H, BK, BN = [int(v) for v in d[name + "_shape"]]
+        f = float(d[name + "_f"])
+        x, hw, dy = (d[name + s].astype(np.float64) for s in ("_x", "_hw", "_dy"))
+        rel = lambda a, b: np.abs(a - b).max() / np.abs(b).max()
+        assert rel(d[name + "_y"], oracle.forward(x, hw, N, BK, BN, R, f)) <= 1e-3
+        assert rel(d[name + "_dx"], oracle.input_grad(dy, hw, K, BK, BN, R, f)) <= 1e-3
+        assert rel(d[name + "_dhw"], oracle.weight_grad(x, dy, H, BK, BN, R, f)) <= 2e-3
+        assert rel(d[name + "_y"], oracle.c_forward(x, hw, N, BK, BN, R, f)) <= 1e-3
+
+
 # ---------------------------------------------------------------- legacy generation hash
 # Row 1 of the output the reference's notebook recorded for hashed_weight = arange(1000),
 # input = eye(128), a 128 x 128 layer, seed 1024 (verify.ipynb, cell 3): with an identity
