@@ -92,3 +92,30 @@ def test_library_picks_the_window_path_for_skinny_batches(oracle):
     torch.cuda.synchronize()
     assert rel_err(a.float().cpu().numpy(), oracle.weight_grad(x64, dy64, H, BK, BN, R1024, 1.0)) <= TOL[torch.bfloat16]
     assert torch.equal(a, b)   # deterministic, unlike the atomic scatter
+
+
+def _random_window_cases(n, seed):
+    rng = np.random.default_rng(seed)
+    cases = []
+    for _ in range(n):
+        BK = int(rng.choice([32, 64]))
+        M = int(rng.integers(1, 300))
+        K, N = (int(rng.integers(8, 1500)) for _ in range(2))
+        H = int(rng.integers(40000, 3000000))
+        cases.append((M, K, N, H, BK, 64))
+    return cases
+
+
+@pytest.mark.parametrize("shape", _random_window_cases(24, 777), ids=_shape_id)
+def test_windowed_weight_grad_random_shapes(oracle, monkeypatch, shape):
+    """Seeded random shapes through the window kernel: fp32 for even M, bf16 for odd M."""
+    from rzlinear_amd.impl.RzLinearBackward import rz_linear_backward_weight_grad_tl
+    monkeypatch.setenv("RZLINEAR_WINDOW", "1")
+    M, K, N, H, BK, BN = shape
+    dtype = torch.float32 if M % 2 == 0 else torch.bfloat16
+    _say("windowed random", shape, dtype)
+    R = SEED_CONSTANTS[0]
+    (x, _, dy), (x64, _, dy64) = make_inputs(M, K, N, H, dtype, seed=M + K + N)
+    dhw = rz_linear_backward_weight_grad_tl(x, dy, 1.25, M, K, N, H, *rargs(R), BLOCK_SIZE_K=BK, BLOCK_SIZE_N=BN)
+    torch.cuda.synchronize()
+    assert rel_err(dhw.float().cpu().numpy(), oracle.weight_grad(x64, dy64, H, BK, BN, R, 1.25)) <= TOL[dtype]
