@@ -196,8 +196,9 @@ static inline SplitPlan plan_split(int I, int J, int R, int elem_bytes) {
   const int r_steps = (R + TR - 1) / TR;
   const int slots = (pl.tile == 256) ? 1 : (pl.tile == 128 ? 2 : 4);
   long long want = ((long long)kComputeUnits * slots + tiles - 1) / tiles;   // fill every CU slot
-  // a slice should run at least 16 steps (8 when most compute units would otherwise sit idle)
-  const int min_steps = (tiles * 2 < kComputeUnits) ? 8 : 16;
+  // a slice should run at least 16 steps (8 when most compute units would otherwise sit idle);
+  // an fp32 step is several times longer than a 16-bit one, so half as many will do
+  const int min_steps = ((tiles * 2 < kComputeUnits) ? 8 : 16) / (elem_bytes == 4 ? 2 : 1);
   if (want > r_steps / min_steps) want = r_steps / min_steps;
   if (want > 16) want = 16;
   if (tiles * 2 >= (long long)kComputeUnits * slots || want < 2 || getenv("RZLINEAR_NO_SPLIT") != nullptr)
