@@ -63,6 +63,25 @@ typedef enum rz_hash {
                              /rz_linear_kernel.cu:34-36,:56-64; R4..R7 unused; H >= BK*BN suffices */
 } rz_hash;
 
+/*
+ * Optional tuning overrides of the entry points that take a `const rz_tuning*` (NULL or an
+ * all-zero struct = the library decides everything, which is what callers want; the overrides
+ * exist so that tests and benchmarks can reach every kernel form).  The library reads no
+ * environment variable and keeps no settings between calls: what a call does is a function of
+ * its arguments alone, and a workspace query answers for the same tuning it is given.
+ * No counterpart in the reference, whose tile choice is the autotuner's.
+ */
+typedef struct rz_tuning {
+  int tile;       /* C-tile edge of the contraction kernels: 0 = automatic, 64, 128 or 256 */
+  int stages;     /* 0 = automatic, 1 = the single-stage form of the 128 tile */
+  int lds_image;  /* weight-grad: 0 = automatic, -1 = never sum tiles in an LDS image of dHW */
+  int window;     /* weight-grad: 0 = automatic, 1 = dHW by windows whenever possible, -1 = never */
+  int split;      /* forward / input-grad: 0 = automatic, -1 = never split the contraction */
+  int clamp;      /* ragged 16-bit shapes: 0 = automatic, -1 = always the bounds-checked kernels */
+  int resident;   /* forward / input-grad: 0 = automatic, -1 = never keep hashed_weight in LDS */
+  int reserved;   /* must be 0 */
+} rz_tuning;
+
 /* Library / ABI version (major*10000 + minor*100 + patch). */
 int rz_version(void);
 
@@ -187,24 +206,44 @@ int rz_weight_grad_ex(const void* X, const void* dY, void* dHW, void* dbias, voi
                       unsigned flags, void* stream);
 
 /*
- * The three contractions with an explicit tile hash (rz_hash).  hash_levels = RZ_HASH_TWO_LEVEL
- * gives rz_forward_ws / rz_input_grad_ws / rz_weight_grad_ex (same workspace sizes, same
- * flags).  RZ_HASH_LEGACY runs a hashed_weight laid out by the legacy generation — its
- * forward /rz_linear_kernel.cu:245-338 and backward :516-592 in tiled mode — with BK = BN = 16
- * and the constants of /RzLinear.py:70-75 (larger tiles follow the same formula).
+ * The three contractions with an explicit tile hash (rz_hash) and optional tuning overrides.
+ * hash_levels = RZ_HASH_TWO_LEVEL and tuning = NULL give rz_forward_ws / rz_input_grad_ws /
+ * rz_weight_grad_ex (same flags).  RZ_HASH_LEGACY runs a hashed_weight laid out by the legacy
+ * generation — its forward /rz_linear_kernel.cu:245-338 and backward :516-592 in tiled mode —
+ * with BK = BN = 16 and the constants of /RzLinear.py:70-75 (larger tiles follow the same
+ * formula).  The workspace size is asked with the same tuning (and flags) as the call.
  */
+size_t rz_forward_hashed_workspace_bytes(int M, int K, int N, int H, int BK, int BN, int dtype,
+                                         const rz_tuning* tuning);
 int rz_forward_hashed(const void* X, const void* HW, const void* bias, void* Y, void* workspace,
                       size_t workspace_bytes, int M, int K, int N, int H, int BK, int BN,
                       const int32_t R[8], int hash_levels, float init_factor, int64_t ldx, int64_t ldy,
-                      int dtype, void* stream);
+                      int dtype, const rz_tuning* tuning, void* stream);
+size_t rz_input_grad_hashed_workspace_bytes(int M, int K, int N, int H, int BK, int BN, int dtype,
+                                            const rz_tuning* tuning);
 int rz_input_grad_hashed(const void* dY, const void* HW, void* dX, void* workspace,
                          size_t workspace_bytes, int M, int K, int N, int H, int BK, int BN,
                          const int32_t R[8], int hash_levels, float init_factor, int64_t lddy,
-                         int64_t lddx, int dtype, void* stream);
+                         int64_t lddx, int dtype, const rz_tuning* tuning, void* stream);
+size_t rz_weight_grad_hashed_workspace_bytes(int M, int K, int N, int H, int BK, int BN, int dtype,
+                                             unsigned flags, int with_dbias, const rz_tuning* tuning);
 int rz_weight_grad_hashed(const void* X, const void* dY, void* dHW, void* dbias, void* workspace,
                           size_t workspace_bytes, int M, int K, int N, int H, int BK, int BN,
                           const int32_t R[8], int hash_levels, float init_factor, int64_t ldx,
-                          int64_t lddy, int dtype, unsigned flags, void* stream);
+                          int64_t lddy, int dtype, unsigned flags, const rz_tuning* tuning, void* stream);
+
+/*
+ * How a call would be carried out (host-side, touches no device): which C tile, how many
+ * slices of the contracted dimension and how long each, which kernel form.  op: 0 = forward,
+ * 1 = input-grad, 2 = weight-grad (flags / with_dbias as for rz_weight_grad_hashed, else 0).
+ * Fills out[8] = { C-tile edge, slices, contracted elements per slice, contracted elements per
+ * kernel step, mode, workgroups, 0, 0 } with mode 0 = plain store, 1 = split contraction with
+ * fp32 partial planes, 2 = weight-grad through LDS images of dHW, 3 = weight-grad by global
+ * atomics, 4 = weight-grad by windows of dHW, 5 = weight-grad through LDS images of segments of
+ * dHW.  For tests of the planning logic and for tuning; no counterpart in the reference.
+ */
+int rz_plan_query(int op, int M, int K, int N, int H, int BK, int BN, int dtype, unsigned flags,
+                  int with_dbias, const rz_tuning* tuning, int32_t out[8]);
 
 /*
  * Materialise W[K,N] (row pitch ldw) from hashed_weight; edge tiles are clipped.

@@ -10,8 +10,7 @@ import os
 import torch
 
 _PKG_DIR = os.path.dirname(os.path.abspath(__file__))
-# RZLINEAR_LIB selects another build of the same library (variant builds for tuning)
-LIB_PATH = os.environ.get("RZLINEAR_LIB") or os.path.join(_PKG_DIR, "librzlinear.so")
+LIB_PATH = os.path.join(_PKG_DIR, "librzlinear.so")
 
 RZ_F32, RZ_BF16, RZ_F16 = 0, 1, 2
 _DTYPES = {torch.float32: RZ_F32, torch.bfloat16: RZ_BF16, torch.float16: RZ_F16}
@@ -22,7 +21,45 @@ EXPORTS = (
     "rz_forward_bias", "rz_forward_workspace_bytes", "rz_forward_ws", "rz_input_grad",
     "rz_input_grad_workspace_bytes", "rz_input_grad_ws", "rz_weight_grad_workspace_bytes", "rz_weight_grad", "rz_weight_grad_ex_workspace_bytes",
     "rz_weight_grad_ex", "rz_forward_hashed", "rz_input_grad_hashed", "rz_weight_grad_hashed", "rz_materialize",
+    "rz_forward_hashed_workspace_bytes", "rz_input_grad_hashed_workspace_bytes",
+    "rz_weight_grad_hashed_workspace_bytes", "rz_plan_query",
 )
+
+
+class Tuning(ctypes.Structure):
+    """struct rz_tuning of include/rzlinear.h: overrides of the library's own choices (all zero =
+    automatic).  Only tests and benchmarks set any of it."""
+    _fields_ = [("tile", ctypes.c_int), ("stages", ctypes.c_int), ("lds_image", ctypes.c_int),
+                ("window", ctypes.c_int), ("split", ctypes.c_int), ("clamp", ctypes.c_int),
+                ("resident", ctypes.c_int), ("reserved", ctypes.c_int)]
+
+
+# What the launchers of this package pass as `tuning` (None = automatic).  The C library keeps no
+# settings of its own; this module-level value is the Python side's, set with `tuning(...)`.
+_tuning = None
+
+
+class tuning:
+    """Context manager: ``with _lib.tuning(tile=128, lds_image=-1): ...`` makes the launchers
+    called inside pass these overrides to the library (see struct rz_tuning)."""
+
+    def __init__(self, **fields):
+        self._new = Tuning(**fields) if fields else None
+
+    def __enter__(self):
+        global _tuning
+        self._old, _tuning = _tuning, self._new
+        return self._new
+
+    def __exit__(self, *exc):
+        global _tuning
+        _tuning = self._old
+        return False
+
+
+def current_tuning():
+    """ctypes argument for the `tuning` parameter of the *_hashed entry points."""
+    return ctypes.byref(_tuning) if _tuning is not None else None
 
 _lib = None
 
@@ -83,15 +120,24 @@ def load():
     lib.rz_weight_grad_ex.restype = c_int
     lib.rz_weight_grad_ex.argtypes = [c_vp, c_vp, c_vp, c_vp, c_vp, c_sz, c_int, c_int, c_int, c_int, c_int, c_int,
                                       i32p, c_f, c_i64, c_i64, c_int, ctypes.c_uint, c_vp]
+    tun = ctypes.POINTER(Tuning)
     lib.rz_forward_hashed.restype = c_int
     lib.rz_forward_hashed.argtypes = [c_vp, c_vp, c_vp, c_vp, c_vp, c_sz, c_int, c_int, c_int, c_int, c_int, c_int,
-                                      i32p, c_int, c_f, c_i64, c_i64, c_int, c_vp]
+                                      i32p, c_int, c_f, c_i64, c_i64, c_int, tun, c_vp]
     lib.rz_input_grad_hashed.restype = c_int
     lib.rz_input_grad_hashed.argtypes = [c_vp, c_vp, c_vp, c_vp, c_sz, c_int, c_int, c_int, c_int, c_int, c_int,
-                                         i32p, c_int, c_f, c_i64, c_i64, c_int, c_vp]
+                                         i32p, c_int, c_f, c_i64, c_i64, c_int, tun, c_vp]
     lib.rz_weight_grad_hashed.restype = c_int
     lib.rz_weight_grad_hashed.argtypes = [c_vp, c_vp, c_vp, c_vp, c_vp, c_sz, c_int, c_int, c_int, c_int, c_int,
-                                          c_int, i32p, c_int, c_f, c_i64, c_i64, c_int, ctypes.c_uint, c_vp]
+                                          c_int, i32p, c_int, c_f, c_i64, c_i64, c_int, ctypes.c_uint, tun, c_vp]
+    lib.rz_forward_hashed_workspace_bytes.restype = c_sz
+    lib.rz_forward_hashed_workspace_bytes.argtypes = [c_int] * 7 + [tun]
+    lib.rz_input_grad_hashed_workspace_bytes.restype = c_sz
+    lib.rz_input_grad_hashed_workspace_bytes.argtypes = [c_int] * 7 + [tun]
+    lib.rz_weight_grad_hashed_workspace_bytes.restype = c_sz
+    lib.rz_weight_grad_hashed_workspace_bytes.argtypes = [c_int] * 7 + [ctypes.c_uint, c_int, tun]
+    lib.rz_plan_query.restype = c_int
+    lib.rz_plan_query.argtypes = [c_int] * 8 + [ctypes.c_uint, c_int, tun, i32p]
     lib.rz_materialize.restype = c_int
     lib.rz_materialize.argtypes = [c_vp, c_vp, c_int, c_int, c_int, c_int, c_int, i32p, c_int, c_i64,
                                    c_int, c_vp]
@@ -155,3 +201,14 @@ def tile_offsets(K, N, H, BLOCK_SIZE_K, BLOCK_SIZE_N, random_numbers, hash_level
     check(lib.rz_tile_offsets(ctypes.cast(out.data_ptr(), ctypes.POINTER(ctypes.c_int32)), K, N, H,
                               BLOCK_SIZE_K, BLOCK_SIZE_N, R, hash_levels))
     return out
+
+
+PLAN_MODES = {0: "store", 1: "split", 2: "lds_image", 3: "atomics", 4: "window", 5: "segment_images"}
+
+
+def plan_query(op, M, K, N, H, BK, BN, dtype_code_, flags=0, with_dbias=False):
+    """How the library would carry out a call (rz_plan_query), under the current tuning:
+    dict(tile, slices, slice_len, step, mode, workgroups).  op: 0 forward, 1 input-grad, 2 weight-grad."""
+    out = (ctypes.c_int32 * 8)()
+    check(load().rz_plan_query(op, M, K, N, H, BK, BN, dtype_code_, flags, int(with_dbias), current_tuning(), out))
+    return dict(tile=out[0], slices=out[1], slice_len=out[2], step=out[3], mode=PLAN_MODES[out[4]], workgroups=out[5])

@@ -54,7 +54,7 @@ def build(keep_asm=False, jobs=None, verbose=True, extra_flags=(), out=None):
     """Compile every HIP source and link librzlinear.so; returns its path.
 
     extra_flags / out build a variant (e.g. with -D tuning switches) next to the default one;
-    RZLINEAR_LIB=<path> makes the package load it."""
+    set rzlinear_amd._lib.LIB_PATH to its path before the first call to load it."""
     out = out or LIB_PATH
     obj_dir = OBJ_DIR if out == LIB_PATH else os.path.join(OBJ_DIR, "variant_" + os.path.basename(out).replace(".", "_"))
     os.makedirs(obj_dir, exist_ok=True)

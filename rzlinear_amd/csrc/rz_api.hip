@@ -71,11 +71,11 @@ static int dtype_bytes(int dtype) {
 }
 
 static hipError_t launch_gemm(int dtype, int op, const GemmParams& p, const WeightGradPlan* plan,
-                              const SplitPlan* split, hipStream_t s) {
+                              const SplitPlan* split, const rz_tuning& tuning, hipStream_t s) {
   switch (dtype) {
-    case RZ_F32: return launch_gemm_f32(op, p, plan, split, s);
-    case RZ_BF16: return launch_gemm_bf16(op, p, plan, split, s);
-    case RZ_F16: return launch_gemm_f16(op, p, plan, split, s);
+    case RZ_F32: return launch_gemm_f32(op, p, plan, split, tuning, s);
+    case RZ_BF16: return launch_gemm_bf16(op, p, plan, split, tuning, s);
+    case RZ_F16: return launch_gemm_f16(op, p, plan, split, tuning, s);
     default: return hipErrorInvalidValue;
   }
 }
@@ -167,6 +167,40 @@ __global__ __launch_bounds__(256) void reduce_colsum_kernel(const float* __restr
   if (g == 0 && n < N) out[n] = ElemTraits<T>::from_float((sums[0][c] + sums[1][c]) + (sums[2][c] + sums[3][c]));
 }
 
+// dbias[n] = sum over the rows m of dY[m][n], for the weight-grad forms that do not stage dY
+// tile by tile (the window kernel: short M).  A workgroup owns 64 columns; four thread groups
+// each add up every fourth row, then the groups are combined through LDS in a fixed order.
+template <typename T, typename O>
+__global__ __launch_bounds__(256) void colsum_rows_kernel(const T* __restrict__ dY, int64_t ld, O* __restrict__ out,
+                                                          int N, int M) {
+  __shared__ float sums[4][64];
+  const int c = threadIdx.x & 63, g = threadIdx.x >> 6;
+  const int n = blockIdx.x * 64 + c;
+  float s = 0.f;
+  if (n < N) {
+#pragma unroll 8
+    for (int m = g; m < M; m += 4) s += ElemTraits<T>::to_float(dY[(int64_t)m * ld + n]);
+  }
+  sums[g][c] = s;
+  __syncthreads();
+  if (g == 0 && n < N) out[n] = ElemTraits<O>::from_float((sums[0][c] + sums[1][c]) + (sums[2][c] + sums[3][c]));
+}
+
+static void launch_colsum_rows(int dtype, int out_dtype, const void* dY, int64_t ld, void* out, int N, int M,
+                               hipStream_t s) {
+  const dim3 grid((N + 63) / 64), block(256);
+  if (dtype == RZ_F32)
+    hipLaunchKernelGGL((colsum_rows_kernel<float, float>), grid, block, 0, s, (const float*)dY, ld, (float*)out, N, M);
+  else if (dtype == RZ_BF16 && out_dtype == RZ_F32)
+    hipLaunchKernelGGL((colsum_rows_kernel<bf16_t, float>), grid, block, 0, s, (const bf16_t*)dY, ld, (float*)out, N, M);
+  else if (dtype == RZ_BF16)
+    hipLaunchKernelGGL((colsum_rows_kernel<bf16_t, bf16_t>), grid, block, 0, s, (const bf16_t*)dY, ld, (bf16_t*)out, N, M);
+  else if (out_dtype == RZ_F32)
+    hipLaunchKernelGGL((colsum_rows_kernel<f16_t, float>), grid, block, 0, s, (const f16_t*)dY, ld, (float*)out, N, M);
+  else
+    hipLaunchKernelGGL((colsum_rows_kernel<f16_t, f16_t>), grid, block, 0, s, (const f16_t*)dY, ld, (f16_t*)out, N, M);
+}
+
 // C[i][j] = sum over the slices of part[s][i][j] (+ bias[j]), converted to the element type.
 template <typename T>
 __global__ __launch_bounds__(256) void reduce_slices_kernel(const float* __restrict__ part,
@@ -206,20 +240,20 @@ static hipError_t reduce_slices_dtype(int dtype, const float* part, void* C, con
 // Forward (op kForward) or input-grad through one code path: p holds the operands; with a
 // workspace the contraction may be split over R (skinny problems).
 static int run_plain_op(int op, int dtype, GemmParams p, const void* bias, void* workspace,
-                        size_t workspace_bytes, bool may_split, hipStream_t s) {
+                        size_t workspace_bytes, bool may_split, const rz_tuning& tuning, hipStream_t s) {
   if (may_split) {
-    const SplitPlan sp = plan_split(p.I, p.J, p.R, dtype_bytes(dtype));
+    const SplitPlan sp = plan_split(p.I, p.J, p.R, dtype_bytes(dtype), tuning);
     if (sp.splits > 1) {
       if (workspace == nullptr || workspace_bytes < sp.workspace_bytes) return RZ_ERR_WORKSPACE;
       p.partial = (float*)workspace;
       p.bias = nullptr;
-      if (launch_gemm(dtype, op, p, nullptr, &sp, s) != hipSuccess) return RZ_ERR_LAUNCH;
+      if (launch_gemm(dtype, op, p, nullptr, &sp, tuning, s) != hipSuccess) return RZ_ERR_LAUNCH;
       return reduce_slices_dtype(dtype, p.partial, p.C, bias, p.I, p.J, p.ldc, sp.splits, s) == hipSuccess
                  ? RZ_OK : RZ_ERR_LAUNCH;
     }
   }
   p.bias = bias;
-  return launch_gemm(dtype, op, p, nullptr, nullptr, s) == hipSuccess ? RZ_OK : RZ_ERR_LAUNCH;
+  return launch_gemm(dtype, op, p, nullptr, nullptr, tuning, s) == hipSuccess ? RZ_OK : RZ_ERR_LAUNCH;
 }
 
 static hipError_t zero_words(void* p, size_t bytes, hipStream_t s) {
@@ -279,9 +313,10 @@ static WeightGradWorkspace weight_grad_workspace(const WeightGradPlan& plan, con
                                                  bool dhw_f32, bool with_dbias) {
   WeightGradWorkspace w;
   if (plan.image_pitch > 0) w.main_bytes = plan.workspace_bytes;
-  else if (window.use && !with_dbias) w.main_bytes = round256((size_t)window.tiles * sizeof(int32_t));  // tile offsets
+  else if (window.use) w.main_bytes = round256((size_t)window.tiles * sizeof(int32_t));  // tile offsets
   else w.main_bytes = dhw_f32 ? 0 : round256((size_t)H * sizeof(float));
-  w.total_bytes = w.main_bytes + (with_dbias ? plan.colsum_bytes : 0);
+  // (the window kernel does not stage dY by tile columns: its bias gradient is a pass of its own)
+  w.total_bytes = w.main_bytes + (with_dbias && !window.use ? plan.colsum_bytes : 0);
   return w;
 }
 
@@ -289,20 +324,23 @@ static WeightGradWorkspace weight_grad_workspace(const WeightGradPlan& plan, con
 static int weight_grad_impl(const void* X, const void* dY, void* dHW, void* dbias, void* workspace,
                             size_t workspace_bytes, int M, int K, int N, int H, int BK, int BN,
                             const int32_t R[8], float init_factor, int64_t ldx, int64_t lddy, int dtype,
-                            unsigned flags, void* stream, int hash_levels = RZ_HASH_TWO_LEVEL) {
+                            unsigned flags, void* stream, int hash_levels = RZ_HASH_TWO_LEVEL,
+                            const rz_tuning* tuning_arg = nullptr) {
   if (X == nullptr || dY == nullptr || dHW == nullptr) return RZ_ERR_NULL_POINTER;
   if (dtype_bytes(dtype) == 0) return RZ_ERR_BAD_DTYPE;
   if (M < 1 || ldx < K || lddy < N) return RZ_ERR_BAD_SHAPE;
   if (flags & ~(unsigned)(RZ_WG_ACCUMULATE | RZ_WG_DHW_F32 | RZ_WG_DBIAS_F32)) return RZ_ERR_BAD_ARGUMENT;
+  const rz_tuning tuning = tuning_or_default(tuning_arg);
+  if (!tuning_valid(tuning)) return RZ_ERR_BAD_ARGUMENT;
   GemmParams p = {};
   int st = make_hash(&p.h, K, N, H, BK, BN, R, hash_levels);
   if (st != RZ_OK) return st;
   const bool accumulate = (flags & RZ_WG_ACCUMULATE) != 0;
   const int dhw_dtype = (flags & RZ_WG_DHW_F32) ? RZ_F32 : dtype;
   const int dbias_dtype = (flags & RZ_WG_DBIAS_F32) ? RZ_F32 : dtype;
-  const WeightGradPlan plan = plan_weight_grad(M, K, N, H, dtype_bytes(dtype));
+  const WeightGradPlan plan = plan_weight_grad(M, K, N, H, dtype_bytes(dtype), tuning);
   WindowPlan wp = {};
-  if (plan.image_pitch == 0) wp = plan_window(M, K, N, H, BK, BN, dtype_bytes(dtype));
+  if (plan.image_pitch == 0) wp = plan_window(M, K, N, H, BK, BN, dtype_bytes(dtype), tuning);
   const WeightGradWorkspace ws = weight_grad_workspace(plan, wp, H, dhw_dtype == RZ_F32, dbias != nullptr);
   if (ws.total_bytes > 0 && (workspace == nullptr || workspace_bytes < ws.total_bytes)) return RZ_ERR_WORKSPACE;
   hipStream_t s = (hipStream_t)stream;
@@ -314,8 +352,8 @@ static int weight_grad_impl(const void* X, const void* dY, void* dHW, void* dbia
   p.lda = ldx;
   p.ldb = lddy;
   p.scale = init_factor;
-  if (dbias != nullptr) p.colsum = reinterpret_cast<float*>(static_cast<char*>(workspace) + ws.main_bytes);
-  if (plan.image_pitch == 0 && dbias == nullptr && wp.use) {
+  if (dbias != nullptr && !wp.use) p.colsum = reinterpret_cast<float*>(static_cast<char*>(workspace) + ws.main_bytes);
+  if (plan.image_pitch == 0 && wp.use) {
     // large hashed_weight, short contraction: windows of dHW instead of K*N atomics.  The
     // tile offsets are hashed once into the workspace; every workgroup scans them.
     {
@@ -338,14 +376,19 @@ static int weight_grad_impl(const void* X, const void* dY, void* dHW, void* dbia
       hipError_t e = dtype == RZ_F32 ? launch_window_f32(w, wp.windows, s)
                      : dtype == RZ_BF16 ? launch_window_bf16(w, wp.windows, s)
                                         : launch_window_f16(w, wp.windows, s);
-      return e == hipSuccess ? RZ_OK : RZ_ERR_LAUNCH;
+      if (e != hipSuccess) return RZ_ERR_LAUNCH;
+      if (dbias != nullptr) {
+        launch_colsum_rows(dtype, dbias_dtype, dY, lddy, dbias, N, M, s);
+        if (hipGetLastError() != hipSuccess) return RZ_ERR_LAUNCH;
+      }
+      return RZ_OK;
     }
   }
   if (plan.image_pitch > 0) {
     // every workgroup sums its tiles into an LDS image of dHW and stores it as a partial image;
     // the partial images are then added up (no global atomics, fixed summation order)
     p.scatter = (float*)workspace;
-    if (launch_gemm(dtype, kWeightGrad, p, &plan, nullptr, s) != hipSuccess) return RZ_ERR_LAUNCH;
+    if (launch_gemm(dtype, kWeightGrad, p, &plan, nullptr, tuning, s) != hipSuccess) return RZ_ERR_LAUNCH;
     if (accumulate) launch_reduce_partials<true>(dhw_dtype, p.scatter, dHW, H, plan.image_pitch, (int)plan.workgroups, s);
     else launch_reduce_partials<false>(dhw_dtype, p.scatter, dHW, H, plan.image_pitch, (int)plan.workgroups, s);
   } else {
@@ -356,7 +399,7 @@ static int weight_grad_impl(const void* X, const void* dY, void* dHW, void* dbia
         zero_words(image, (size_t)H * sizeof(float), s) != hipSuccess)
       return RZ_ERR_LAUNCH;
     p.scatter = image;
-    if (launch_gemm(dtype, kWeightGrad, p, &plan, nullptr, s) != hipSuccess) return RZ_ERR_LAUNCH;
+    if (launch_gemm(dtype, kWeightGrad, p, &plan, nullptr, tuning, s) != hipSuccess) return RZ_ERR_LAUNCH;
     if (dhw_dtype != RZ_F32) {
       if (accumulate) launch_convert<true>(dhw_dtype, image, dHW, H, s);
       else launch_convert<false>(dhw_dtype, image, dHW, H, s);
@@ -378,7 +421,7 @@ extern "C" {
 
 #define RZ_API __attribute__((visibility("default")))
 
-RZ_API int rz_version(void) { return 200; }
+RZ_API int rz_version(void) { return 300; }
 
 RZ_API const char* rz_status_string(int status) {
   switch (status) {
@@ -425,10 +468,12 @@ RZ_API int rz_tile_offsets_device(int32_t* d_out, int K, int N, int H, int BK, i
 static int forward_impl(const void* X, const void* HW, const void* bias, void* Y, void* workspace,
                         size_t workspace_bytes, bool may_split, int M, int K, int N, int H, int BK, int BN,
                         const int32_t R[8], float init_factor, int64_t ldx, int64_t ldy, int dtype,
-                        void* stream, int hash_levels = RZ_HASH_TWO_LEVEL) {
+                        void* stream, int hash_levels = RZ_HASH_TWO_LEVEL, const rz_tuning* tuning_arg = nullptr) {
   if (X == nullptr || HW == nullptr || Y == nullptr) return RZ_ERR_NULL_POINTER;
   if (dtype_bytes(dtype) == 0) return RZ_ERR_BAD_DTYPE;
   if (M < 1 || ldx < K || ldy < N) return RZ_ERR_BAD_SHAPE;
+  const rz_tuning tuning = tuning_or_default(tuning_arg);
+  if (!tuning_valid(tuning)) return RZ_ERR_BAD_ARGUMENT;
   GemmParams p = {};
   int st = make_hash(&p.h, K, N, H, BK, BN, R, hash_levels);
   if (st != RZ_OK) return st;
@@ -441,16 +486,18 @@ static int forward_impl(const void* X, const void* HW, const void* bias, void* Y
   p.lda = ldx;
   p.ldc = ldy;
   p.scale = init_factor;
-  return run_plain_op(kForward, dtype, p, bias, workspace, workspace_bytes, may_split, (hipStream_t)stream);
+  return run_plain_op(kForward, dtype, p, bias, workspace, workspace_bytes, may_split, tuning, (hipStream_t)stream);
 }
 
 static int input_grad_impl(const void* dY, const void* HW, void* dX, void* workspace, size_t workspace_bytes,
                            bool may_split, int M, int K, int N, int H, int BK, int BN, const int32_t R[8],
                            float init_factor, int64_t lddy, int64_t lddx, int dtype, void* stream,
-                           int hash_levels = RZ_HASH_TWO_LEVEL) {
+                           int hash_levels = RZ_HASH_TWO_LEVEL, const rz_tuning* tuning_arg = nullptr) {
   if (dY == nullptr || HW == nullptr || dX == nullptr) return RZ_ERR_NULL_POINTER;
   if (dtype_bytes(dtype) == 0) return RZ_ERR_BAD_DTYPE;
   if (M < 1 || lddy < N || lddx < K) return RZ_ERR_BAD_SHAPE;
+  const rz_tuning tuning = tuning_or_default(tuning_arg);
+  if (!tuning_valid(tuning)) return RZ_ERR_BAD_ARGUMENT;
   GemmParams p = {};
   int st = make_hash(&p.h, K, N, H, BK, BN, R, hash_levels);
   if (st != RZ_OK) return st;
@@ -463,7 +510,7 @@ static int input_grad_impl(const void* dY, const void* HW, void* dX, void* works
   p.lda = lddy;
   p.ldc = lddx;
   p.scale = init_factor;
-  return run_plain_op(kInputGrad, dtype, p, nullptr, workspace, workspace_bytes, may_split,
+  return run_plain_op(kInputGrad, dtype, p, nullptr, workspace, workspace_bytes, may_split, tuning,
                       (hipStream_t)stream);
 }
 
@@ -481,11 +528,17 @@ RZ_API int rz_forward(const void* X, const void* HW, void* Y, int M, int K, int 
                       dtype, stream);
 }
 
-RZ_API size_t rz_forward_workspace_bytes(int M, int K, int N, int H, int BK, int BN, int dtype) {
+RZ_API size_t rz_forward_hashed_workspace_bytes(int M, int K, int N, int H, int BK, int BN, int dtype,
+                                                const rz_tuning* tuning) {
   (void)H; (void)BK; (void)BN;
   const int eb = dtype_bytes(dtype);
-  if (eb == 0 || M < 1 || K < 1 || N < 1) return 0;
-  return plan_split(M, N, K, eb).workspace_bytes;
+  const rz_tuning t = tuning_or_default(tuning);
+  if (eb == 0 || M < 1 || K < 1 || N < 1 || !tuning_valid(t)) return 0;
+  return plan_split(M, N, K, eb, t).workspace_bytes;
+}
+
+RZ_API size_t rz_forward_workspace_bytes(int M, int K, int N, int H, int BK, int BN, int dtype) {
+  return rz_forward_hashed_workspace_bytes(M, K, N, H, BK, BN, dtype, nullptr);
 }
 
 RZ_API int rz_forward_ws(const void* X, const void* HW, const void* bias, void* Y, void* workspace,
@@ -503,11 +556,17 @@ RZ_API int rz_input_grad(const void* dY, const void* HW, void* dX, int M, int K,
                          dtype, stream);
 }
 
-RZ_API size_t rz_input_grad_workspace_bytes(int M, int K, int N, int H, int BK, int BN, int dtype) {
+RZ_API size_t rz_input_grad_hashed_workspace_bytes(int M, int K, int N, int H, int BK, int BN, int dtype,
+                                                   const rz_tuning* tuning) {
   (void)H; (void)BK; (void)BN;
   const int eb = dtype_bytes(dtype);
-  if (eb == 0 || M < 1 || K < 1 || N < 1) return 0;
-  return plan_split(M, K, N, eb).workspace_bytes;
+  const rz_tuning t = tuning_or_default(tuning);
+  if (eb == 0 || M < 1 || K < 1 || N < 1 || !tuning_valid(t)) return 0;
+  return plan_split(M, K, N, eb, t).workspace_bytes;
+}
+
+RZ_API size_t rz_input_grad_workspace_bytes(int M, int K, int N, int H, int BK, int BN, int dtype) {
+  return rz_input_grad_hashed_workspace_bytes(M, K, N, H, BK, BN, dtype, nullptr);
 }
 
 RZ_API int rz_input_grad_ws(const void* dY, const void* HW, void* dX, void* workspace,
@@ -530,15 +589,21 @@ RZ_API int rz_weight_grad(const void* X, const void* dY, void* dHW, void* worksp
                           init_factor, ldx, lddy, dtype, 0u, stream);
 }
 
-RZ_API size_t rz_weight_grad_ex_workspace_bytes(int M, int K, int N, int H, int BK, int BN, int dtype,
-                                                unsigned flags, int with_dbias) {
+RZ_API size_t rz_weight_grad_hashed_workspace_bytes(int M, int K, int N, int H, int BK, int BN, int dtype,
+                                                    unsigned flags, int with_dbias, const rz_tuning* tuning) {
   const int eb = dtype_bytes(dtype);
-  if (eb == 0 || M < 1 || K < 1 || N < 1 || H < 1) return 0;
-  const WeightGradPlan plan = plan_weight_grad(M, K, N, H, eb);
+  const rz_tuning t = tuning_or_default(tuning);
+  if (eb == 0 || M < 1 || K < 1 || N < 1 || H < 1 || !tuning_valid(t)) return 0;
+  const WeightGradPlan plan = plan_weight_grad(M, K, N, H, eb, t);
   const bool dhw_f32 = (flags & RZ_WG_DHW_F32) != 0 || dtype == RZ_F32;
   WindowPlan wp = {};
-  if (plan.image_pitch == 0 && check_tile(BK, BN) == RZ_OK) wp = plan_window(M, K, N, H, BK, BN, eb);
+  if (plan.image_pitch == 0 && check_tile(BK, BN) == RZ_OK) wp = plan_window(M, K, N, H, BK, BN, eb, t);
   return weight_grad_workspace(plan, wp, H, dhw_f32, with_dbias != 0).total_bytes;
+}
+
+RZ_API size_t rz_weight_grad_ex_workspace_bytes(int M, int K, int N, int H, int BK, int BN, int dtype,
+                                                unsigned flags, int with_dbias) {
+  return rz_weight_grad_hashed_workspace_bytes(M, K, N, H, BK, BN, dtype, flags, with_dbias, nullptr);
 }
 
 RZ_API int rz_weight_grad_ex(const void* X, const void* dY, void* dHW, void* dbias, void* workspace,
@@ -552,25 +617,62 @@ RZ_API int rz_weight_grad_ex(const void* X, const void* dY, void* dHW, void* dbi
 RZ_API int rz_forward_hashed(const void* X, const void* HW, const void* bias, void* Y, void* workspace,
                              size_t workspace_bytes, int M, int K, int N, int H, int BK, int BN,
                              const int32_t R[8], int hash_levels, float init_factor, int64_t ldx,
-                             int64_t ldy, int dtype, void* stream) {
+                             int64_t ldy, int dtype, const rz_tuning* tuning, void* stream) {
   return forward_impl(X, HW, bias, Y, workspace, workspace_bytes, true, M, K, N, H, BK, BN, R, init_factor,
-                      ldx, ldy, dtype, stream, hash_levels);
+                      ldx, ldy, dtype, stream, hash_levels, tuning);
 }
 
 RZ_API int rz_input_grad_hashed(const void* dY, const void* HW, void* dX, void* workspace,
                                 size_t workspace_bytes, int M, int K, int N, int H, int BK, int BN,
                                 const int32_t R[8], int hash_levels, float init_factor, int64_t lddy,
-                                int64_t lddx, int dtype, void* stream) {
+                                int64_t lddx, int dtype, const rz_tuning* tuning, void* stream) {
   return input_grad_impl(dY, HW, dX, workspace, workspace_bytes, true, M, K, N, H, BK, BN, R, init_factor,
-                         lddy, lddx, dtype, stream, hash_levels);
+                         lddy, lddx, dtype, stream, hash_levels, tuning);
 }
 
 RZ_API int rz_weight_grad_hashed(const void* X, const void* dY, void* dHW, void* dbias, void* workspace,
                                  size_t workspace_bytes, int M, int K, int N, int H, int BK, int BN,
                                  const int32_t R[8], int hash_levels, float init_factor, int64_t ldx,
-                                 int64_t lddy, int dtype, unsigned flags, void* stream) {
+                                 int64_t lddy, int dtype, unsigned flags, const rz_tuning* tuning, void* stream) {
   return weight_grad_impl(X, dY, dHW, dbias, workspace, workspace_bytes, M, K, N, H, BK, BN, R,
-                          init_factor, ldx, lddy, dtype, flags, stream, hash_levels);
+                          init_factor, ldx, lddy, dtype, flags, stream, hash_levels, tuning);
+}
+
+RZ_API int rz_plan_query(int op, int M, int K, int N, int H, int BK, int BN, int dtype, unsigned flags,
+                         int with_dbias, const rz_tuning* tuning, int32_t out[8]) {
+  (void)flags; (void)with_dbias;
+  if (out == nullptr) return RZ_ERR_NULL_POINTER;
+  const int eb = dtype_bytes(dtype);
+  if (eb == 0) return RZ_ERR_BAD_DTYPE;
+  if (M < 1 || K < 1 || N < 1 || H < 1) return RZ_ERR_BAD_SHAPE;
+  const rz_tuning t = tuning_or_default(tuning);
+  if (!tuning_valid(t)) return RZ_ERR_BAD_ARGUMENT;
+  int st = check_tile(BK, BN);
+  if (st != RZ_OK) return st;
+  for (int i = 0; i < 8; i++) out[i] = 0;
+  if (op == kWeightGrad) {
+    const WeightGradPlan plan = plan_weight_grad(M, K, N, H, eb, t);
+    WindowPlan wp = {};
+    if (plan.image_pitch == 0) wp = plan_window(M, K, N, H, BK, BN, eb, t);
+    if (wp.use) {
+      out[0] = 0; out[1] = 1; out[2] = M; out[3] = 32; out[4] = 4; out[5] = wp.windows;
+      return RZ_OK;
+    }
+    const KernelForm f = kernel_form(op, K, N, M, plan.r_chunk, plan.tile, plan.workgroups, eb, t);
+    out[0] = plan.tile; out[1] = plan.splits; out[2] = plan.r_chunk; out[3] = f.step;
+    out[4] = plan.image_pitch > 0 ? 2 : 3;
+    out[5] = (int32_t)plan.workgroups;
+    return RZ_OK;
+  }
+  if (op != kForward && op != kInputGrad) return RZ_ERR_BAD_ARGUMENT;
+  const int I = M, J = op == kForward ? N : K, R = op == kForward ? K : N;
+  const SplitPlan sp = plan_split(I, J, R, eb, t);
+  const bool cut = sp.splits > 1;
+  const int chunk = cut ? sp.r_chunk : R;
+  const KernelForm f = kernel_form(op, I, J, R, chunk, sp.tile, tile_count(I, J, sp.tile), eb, t);
+  out[0] = sp.tile; out[1] = sp.splits; out[2] = chunk; out[3] = f.step; out[4] = cut ? 1 : 0;
+  out[5] = (int32_t)(tile_count(I, J, sp.tile) * sp.splits);
+  return RZ_OK;
 }
 
 RZ_API int rz_materialize(const void* HW, void* W, int K, int N, int H, int BK, int BN,

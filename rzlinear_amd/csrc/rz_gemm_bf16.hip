@@ -3,8 +3,8 @@
 
 namespace rz {
 hipError_t launch_gemm_bf16(int op, GemmParams p, const WeightGradPlan* plan, const SplitPlan* split,
-                           hipStream_t stream) {
-  return launch_gemm_t<bf16_t>(op, p, plan, split, stream);
+                            const rz_tuning& tuning, hipStream_t stream) {
+  return launch_gemm_t<bf16_t>(op, p, plan, split, tuning, stream);
 }
 hipError_t launch_window_bf16(const WindowParams& p, int windows, hipStream_t stream) {
   return launch_window_t<bf16_t>(p, windows, stream);

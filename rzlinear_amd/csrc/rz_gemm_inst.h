@@ -1,15 +1,31 @@
 // Body shared by the per-dtype translation units: tile choice + launch.
 #pragma once
 
+#include <atomic>
+
 #include "rz_gemm.h"
 #include "rz_launch.h"
 #include "rz_window.h"
 
 namespace rz {
 
+// Kernels that use more than the default 64 KB of LDS need their limit raised once per kernel
+// and device; `done` is that kernel's bit set of devices already served.
+static inline hipError_t raise_lds_limit(const void* kernel, std::atomic<uint64_t>& done) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  const uint64_t bit = 1ull << (dev & 63);
+  if (done.load(std::memory_order_acquire) & bit) return hipSuccess;
+  e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+  if (e == hipSuccess) done.fetch_or(bit, std::memory_order_release);
+  return e;
+}
+
 template <typename T, int OP, int TI, int TJ, int WI, int WJ, int NSTAGE, bool FULL, bool COLSUM, bool CLAMP = false>
 static hipError_t launch_one(GemmParams p, const WeightGradPlan* plan, const SplitPlan* split,
                              hipStream_t stream) {
+  static std::atomic<uint64_t> lds_limit_raised{0};
   typedef GemmKernel<T, OP, TI, TJ, WI, WJ, NSTAGE, FULL, COLSUM, CLAMP> K;
   p.tiles_i = (p.I + TI - 1) / TI;
   p.tiles_j = (p.J + TJ - 1) / TJ;
@@ -33,6 +49,9 @@ static hipError_t launch_one(GemmParams p, const WeightGradPlan* plan, const Spl
     if (split->tile != TI || p.partial == nullptr) return hipErrorInvalidValue;
     splits = split->splits;
     p.r_chunk = split->r_chunk;
+    // a slice must begin on a step boundary: the offset table of a step assumes that the step
+    // lies inside one hashed tile or covers whole ones
+    if (p.r_chunk % K::TR != 0) return hipErrorInvalidValue;
   } else {
     p.r_chunk = r_steps * K::TR;
     p.partial = nullptr;
@@ -46,8 +65,7 @@ static hipError_t launch_one(GemmParams p, const WeightGradPlan* plan, const Spl
     if (need > smem) smem = need;
   }
   if (smem > 64 * 1024) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    hipError_t e = raise_lds_limit(reinterpret_cast<const void*>(kernel), lds_limit_raised);
     if (e != hipSuccess) return e;
   }
   dim3 grid((unsigned)tiles, (unsigned)splits, 1), block(K::kThreads, 1, 1);
@@ -55,39 +73,38 @@ static hipError_t launch_one(GemmParams p, const WeightGradPlan* plan, const Spl
   return hipGetLastError();
 }
 
-// FULL kernels carry no bounds checks: every tile and every R step must be complete.
+// FULL kernels carry no bounds checks: every tile and every R step must be complete.  Ragged
+// shapes: 16-bit tiles can still be staged directly, with edge pieces fetched from inside the
+// operands (CLAMP); everything else takes the bounds-checked kernel.
 template <typename T, int OP, int TILE, int WI, int WJ, int NSTAGE, bool COLSUM = false>
 static hipError_t launch_tile(GemmParams p, const WeightGradPlan* plan, const SplitPlan* split,
-                              hipStream_t stream) {
-  // (the unchecked kernel's R step; every slice of a split contraction must be whole steps too)
-  constexpr int TR = GemmKernel<T, OP, TILE, TILE, WI, WJ, NSTAGE, true>::TR;
-  const int chunk = (OP == kWeightGrad) ? (plan != nullptr ? plan->r_chunk : p.R)
-                                        : (split != nullptr && split->splits > 1 ? split->r_chunk : p.R);
-  const bool full = (p.I % TILE == 0) && (p.J % TILE == 0) && (p.R % TR == 0) && (chunk % TR == 0);
-  if (full) return launch_one<T, OP, TILE, TILE, WI, WJ, NSTAGE, true, COLSUM>(p, plan, split, stream);
-  // Ragged shapes: 16-bit tiles can still be staged directly, with edge pieces fetched from
-  // inside the operands.  A plain operand's 16-byte pieces must not straddle the end of its
-  // rows: forward / input-grad need R, weight-grad needs I and J, to be multiples of the piece.
-  if constexpr (sizeof(T) == 2 && NSTAGE == 2 && TILE >= 128) {
-    constexpr int VEC = ElemTraits<T>::kVec;
-    const bool pieces_ok = OP == kWeightGrad ? (p.I % VEC == 0 && p.J % VEC == 0 && p.I >= VEC && p.J >= VEC)
-                                             : (p.R % VEC == 0 && p.R >= VEC);
-    if (pieces_ok && getenv("RZLINEAR_NO_CLAMP") == nullptr)
-      return launch_one<T, OP, TILE, TILE, WI, WJ, NSTAGE, false, COLSUM, true>(p, plan, split, stream);
+                              const KernelForm& form, hipStream_t stream) {
+  // (the form was derived on the host from the same rules that select the instantiation here:
+  //  refuse to launch if the two ever disagree about the step length)
+  if (form.full) {
+    if (form.step != GemmKernel<T, OP, TILE, TILE, WI, WJ, NSTAGE, true>::TR) return hipErrorInvalidValue;
+    return launch_one<T, OP, TILE, TILE, WI, WJ, NSTAGE, true, COLSUM>(p, plan, split, stream);
   }
+  if constexpr (sizeof(T) == 2 && NSTAGE == 2 && TILE >= 128) {
+    if (form.clamp) {
+      if (form.step != GemmKernel<T, OP, TILE, TILE, WI, WJ, NSTAGE, false, false, true>::TR) return hipErrorInvalidValue;
+      return launch_one<T, OP, TILE, TILE, WI, WJ, NSTAGE, false, COLSUM, true>(p, plan, split, stream);
+    }
+  }
+  if (form.clamp || form.step != GemmKernel<T, OP, TILE, TILE, WI, WJ, NSTAGE, false>::TR) return hipErrorInvalidValue;
   return launch_one<T, OP, TILE, TILE, WI, WJ, NSTAGE, false, COLSUM>(p, plan, split, stream);
 }
 
 template <typename T, int TILE, int WI, int WJ, int NSTAGE>
 static hipError_t launch_op(int op, GemmParams p, const WeightGradPlan* plan, const SplitPlan* split,
-                            hipStream_t stream) {
+                            const KernelForm& form, hipStream_t stream) {
   switch (op) {
-    case kForward: return launch_tile<T, kForward, TILE, WI, WJ, NSTAGE>(p, plan, split, stream);
-    case kInputGrad: return launch_tile<T, kInputGrad, TILE, WI, WJ, NSTAGE>(p, plan, split, stream);
+    case kForward: return launch_tile<T, kForward, TILE, WI, WJ, NSTAGE>(p, plan, split, form, stream);
+    case kInputGrad: return launch_tile<T, kInputGrad, TILE, WI, WJ, NSTAGE>(p, plan, split, form, stream);
     case kWeightGrad:
       // with a column-sum target the kernel also produces the bias gradient's partial sums
-      if (p.colsum != nullptr) return launch_tile<T, kWeightGrad, TILE, WI, WJ, NSTAGE, true>(p, plan, split, stream);
-      return launch_tile<T, kWeightGrad, TILE, WI, WJ, NSTAGE>(p, plan, split, stream);
+      if (p.colsum != nullptr) return launch_tile<T, kWeightGrad, TILE, WI, WJ, NSTAGE, true>(p, plan, split, form, stream);
+      return launch_tile<T, kWeightGrad, TILE, WI, WJ, NSTAGE>(p, plan, split, form, stream);
     default: return hipErrorInvalidValue;
   }
 }
@@ -95,29 +112,25 @@ static hipError_t launch_op(int op, GemmParams p, const WeightGradPlan* plan, co
 // Tile shapes (all two LDS stages, software pipelined unless noted):
 //   256: 256 x 256, eight wavefronts of 128 x 64, one workgroup per compute unit
 //   128: 128 x 128, four wavefronts of 64 x 64 (up to two workgroups per compute unit) or
-//        eight of 64 x 32 when there is about one workgroup per compute unit
+//        eight of 64 x 32 when there is about one workgroup per compute unit; tuning.stages = 1
+//        selects a single-stage form that leans on several workgroups per compute unit
+//        instead of a pipeline (tuning aid)
 //    64:  64 x  64, four wavefronts of 32 x 32, for problems with few tiles
-// RZLINEAR_STAGES=1 selects a single-stage 128 x 128 form that leans on several workgroups
-// per compute unit instead of a pipeline (tuning aid).
 template <typename T>
 static hipError_t launch_gemm_t(int op, GemmParams p, const WeightGradPlan* plan, const SplitPlan* split,
-                                hipStream_t stream) {
-  const int tile = (op == kWeightGrad && plan != nullptr) ? plan->tile
-                   : (split != nullptr ? split->tile : pick_tile(p.I, p.J, (int)sizeof(T)));
-  const char* stages_env = getenv("RZLINEAR_STAGES");
-  const bool one_stage = stages_env != nullptr && atoi(stages_env) == 1;
-  switch (tile) {
-    case 256: return launch_op<T, 256, 2, 4, 2>(op, p, plan, split, stream);
-    case 64: return launch_op<T, 64, 2, 2, 2>(op, p, plan, split, stream);
-    case 128:
-      if (one_stage) return launch_op<T, 128, 2, 2, 1>(op, p, plan, split, stream);
-      // with about one workgroup per compute unit, eight wavefronts (two per SIMD, 64 x 32
-      // each) hide latency better than four of 64 x 64; with more workgroups resident the
-      // four-wavefront form does less LDS traffic per flop
-      if (tile_count(p.I, p.J, 128) * (op == kWeightGrad && plan != nullptr ? plan->splits : 1) <=
-          kComputeUnits * 3 / 2)
-        return launch_op<T, 128, 2, 4, 2>(op, p, plan, split, stream);
-      return launch_op<T, 128, 2, 2, 2>(op, p, plan, split, stream);
+                                const rz_tuning& tuning, hipStream_t stream) {
+  const bool wg = op == kWeightGrad && plan != nullptr;
+  const bool cut = !wg && split != nullptr && split->splits > 1;
+  const int tile = wg ? plan->tile : (split != nullptr ? split->tile : pick_tile(p.I, p.J, (int)sizeof(T), tuning));
+  const int chunk = wg ? plan->r_chunk : (cut ? split->r_chunk : p.R);
+  const long long workgroups = tile_count(p.I, p.J, tile) * (wg ? plan->splits : 1);
+  const KernelForm form = kernel_form(op, p.I, p.J, p.R, chunk, tile, workgroups, (int)sizeof(T), tuning);
+  switch (form.tile * 100 + form.waves * 10 + form.stages) {
+    case 25682: return launch_op<T, 256, 2, 4, 2>(op, p, plan, split, form, stream);
+    case 6442: return launch_op<T, 64, 2, 2, 2>(op, p, plan, split, form, stream);
+    case 12841: return launch_op<T, 128, 2, 2, 1>(op, p, plan, split, form, stream);
+    case 12882: return launch_op<T, 128, 2, 4, 2>(op, p, plan, split, form, stream);
+    case 12842: return launch_op<T, 128, 2, 2, 2>(op, p, plan, split, form, stream);
     default: return hipErrorInvalidValue;
   }
 }
@@ -130,9 +143,9 @@ static hipError_t launch_window_one(const WindowParams& p, int windows, hipStrea
   if ((long long)windows * p.window < p.H) return hipErrorInvalidValue;
   auto kernel = rz_window_kernel<T, TBK, TBN>;
   const size_t smem = K::kFixedBytes + sizeof(float) * (size_t)p.window;
+  static std::atomic<uint64_t> lds_limit_raised{0};
   if (smem > 64 * 1024) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    hipError_t e = raise_lds_limit(reinterpret_cast<const void*>(kernel), lds_limit_raised);
     if (e != hipSuccess) return e;
   }
   hipLaunchKernelGGL(kernel, dim3((unsigned)windows), dim3(K::kThreads), smem, stream, p);

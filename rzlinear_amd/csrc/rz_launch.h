@@ -1,22 +1,34 @@
 // Host-side launch of the contraction kernels; one translation unit per element type.
 #pragma once
 
+#include "../../include/rzlinear.h"
 #include "rz_common.h"
 
-#include <stdlib.h>
-
 namespace rz {
+
+// Every planning function takes the caller's tuning overrides (all zero = automatic); nothing
+// here reads the environment or keeps state, so a workspace query and the launch that follows
+// it decide alike.
+static inline rz_tuning tuning_or_default(const rz_tuning* t) {
+  rz_tuning d = {};
+  return t != nullptr ? *t : d;
+}
+static inline bool tuning_valid(const rz_tuning& t) {
+  return (t.tile == 0 || t.tile == 64 || t.tile == 128 || t.tile == 256) && (t.stages == 0 || t.stages == 1) &&
+         (t.lds_image == 0 || t.lds_image == -1) && (t.window >= -1 && t.window <= 1) &&
+         (t.split == 0 || t.split == -1) && (t.clamp == 0 || t.clamp == -1) &&
+         (t.resident == 0 || t.resident == -1) && t.reserved == 0;
+}
 
 static constexpr int kComputeUnits = 256;
 // Number of workgroups of the small tile that fills the compute units a few times over.
 static constexpr int kTargetWorkgroups = 1024;
 
-// C-tile edge for a contraction with an I x J result: the largest of 256, 128, 64 that still
-// yields about one workgroup per compute unit; RZLINEAR_TILE=64|128|256 forces one (tuning aid).
-static inline int forced_tile() {
-  const char* e = getenv("RZLINEAR_TILE");   // read per call, so a test can switch it
-  const int v = e ? atoi(e) : 0;
-  return (v == 64 || v == 128 || v == 256) ? v : 0;
+// Contracted elements per kernel step that every slice of a cut contraction must be a multiple
+// of: 128 bytes, and 256 for the 16-bit 128 tile, whose eight-wavefront form takes 256-byte steps
+// (a slice that began in the middle of such a step would start between two hashed tiles).
+static inline int slice_unit(int tile, int elem_bytes) {
+  return ((tile == 128 && elem_bytes == 2) ? 256 : 128) / elem_bytes;
 }
 
 static inline long long tile_count(int I, int J, int t) {
@@ -51,8 +63,9 @@ static inline double tile_score(int I, int J, int t, int elem_bytes) {
   return tile_score_full(I, J, t, elem_bytes) * ((double)I * (double)J) / (wgs * t * t);
 }
 
-static inline int pick_tile(int I, int J, int elem_bytes) {
-  if (forced_tile()) return forced_tile();
+// C-tile edge for a contraction with an I x J result: the best-scoring of 256, 128, 64.
+static inline int pick_tile(int I, int J, int elem_bytes, const rz_tuning& tuning) {
+  if (tuning.tile) return tuning.tile;
   int best = 256;
   double best_score = tile_score(I, J, 256, elem_bytes);
   const int others[2] = {128, 64};
@@ -91,14 +104,12 @@ static inline long long tile_cover(int K, int N, int t) {
   return (long long)((K + t - 1) / t) * ((N + t - 1) / t) * t * t;
 }
 
-static inline WeightGradPlan plan_weight_grad(int M, int K, int N, int H, int elem_bytes) {
+static inline WeightGradPlan plan_weight_grad(int M, int K, int N, int H, int elem_bytes, const rz_tuning& t) {
   WeightGradPlan pl;
-  const int TR = 128 / elem_bytes;
   const int pitch = (H + 3) & ~3;
-  const bool no_image = getenv("RZLINEAR_NO_LDS_IMAGE") != nullptr;   // tuning aid
-  const bool image = !no_image && (size_t)pitch * sizeof(float) <= kMaxImageBytes;
-  if (forced_tile()) {
-    pl.tile = forced_tile();
+  const bool image = t.lds_image != -1 && (size_t)pitch * sizeof(float) <= kMaxImageBytes;
+  if (t.tile) {
+    pl.tile = t.tile;
   } else if (image) {
     // with the LDS image the M loop can be cut freely (a slice costs one partial image), so
     // the pipelined 256 tile is used unless it would mostly compute padding
@@ -108,14 +119,16 @@ static inline WeightGradPlan plan_weight_grad(int M, int K, int N, int H, int el
     // a short M cut over many slices leaves a 256 workgroup a step or two between its prologue
     // and its scatter: the 128 tile then has less to set up and to scatter per workgroup
     const long long tiles256 = tile_count(K, N, 256);
+    const int step256 = slice_unit(256, elem_bytes);
     if (pl.tile == 256 && tiles256 < kComputeUnits &&
-        (long long)((M + TR - 1) / TR) * tiles256 < 4LL * kComputeUnits &&
+        (long long)((M + step256 - 1) / step256) * tiles256 < 4LL * kComputeUnits &&
         tile_cover(K, N, 128) * 10 <= tile_cover(K, N, 256) * 13)
       pl.tile = 128;
   } else {
-    pl.tile = pick_tile(K, N, elem_bytes);
+    pl.tile = pick_tile(K, N, elem_bytes, t);
   }
   const long long tiles = (long long)((K + pl.tile - 1) / pl.tile) * ((N + pl.tile - 1) / pl.tile);
+  const int TR = slice_unit(pl.tile, elem_bytes);
   const int r_steps = (M + TR - 1) / TR;
   // split the reduction over M when there are too few W tiles to fill the chip
   const long long target = (pl.tile >= 256) ? kComputeUnits : (pl.tile == 128 ? 2 * kComputeUnits : kTargetWorkgroups);
@@ -151,11 +164,9 @@ static constexpr int kWindowFloats = 25600;   // LDS floats a workgroup can hold
 
 static inline bool window_tile_supported(int BK, int BN) { return BN == 64 && (BK == 64 || BK == 32); }
 
-static inline WindowPlan plan_window(int M, int K, int N, int H, int BK, int BN, int elem_bytes) {
+static inline WindowPlan plan_window(int M, int K, int N, int H, int BK, int BN, int elem_bytes, const rz_tuning& t) {
   WindowPlan pl = {false, 0, 0, 0};
-  const char* env = getenv("RZLINEAR_WINDOW");   // tuning aid: 0 = never, 1 = whenever possible
-  const int forced = env ? atoi(env) : -1;
-  if (forced == 0 || !window_tile_supported(BK, BN)) return pl;
+  if (t.window == -1 || !window_tile_supported(BK, BN)) return pl;
   const long long tiles = (long long)((K + BK - 1) / BK) * ((N + BN - 1) / BN);
   if (tiles > (1 << 20)) return pl;              // every workgroup scans every tile's offset
   pl.tiles = tiles;
@@ -175,7 +186,7 @@ static inline WindowPlan plan_window(int M, int K, int N, int H, int BK, int BN,
   const double wg_rounds = (double)((pl.windows + kComputeUnits - 1) / kComputeUnits);
   const double t_window = wg_rounds * per_wg * (0.72 + (elem_bytes == 4 ? 1.2 : 0.32) * chunks) + 30.0;
   const double t_scatter = 0.9 * (double)K * N / 184e3 + 2.0 * M * (double)K * N / 800e6;
-  pl.use = forced == 1 || t_window * 1.2 < t_scatter;
+  pl.use = t.window == 1 || t_window * 1.2 < t_scatter;
   return pl;
 }
 
@@ -188,20 +199,20 @@ struct SplitPlan {
   size_t workspace_bytes;
 };
 
-static inline SplitPlan plan_split(int I, int J, int R, int elem_bytes) {
+static inline SplitPlan plan_split(int I, int J, int R, int elem_bytes, const rz_tuning& t) {
   SplitPlan pl;
-  const int TR = 128 / elem_bytes;
-  pl.tile = pick_tile(I, J, elem_bytes);
+  pl.tile = pick_tile(I, J, elem_bytes, t);
+  const int TR = slice_unit(pl.tile, elem_bytes);
   const long long tiles = tile_count(I, J, pl.tile);
   const int r_steps = (R + TR - 1) / TR;
   const int slots = (pl.tile == 256) ? 1 : (pl.tile == 128 ? 2 : 4);
   long long want = ((long long)kComputeUnits * slots + tiles - 1) / tiles;   // fill every CU slot
   // a slice should run at least 16 steps (8 when most compute units would otherwise sit idle);
   // an fp32 step is several times longer than a 16-bit one, so half as many will do
-  const int min_steps = ((tiles * 2 < kComputeUnits) ? 8 : 16) / (elem_bytes == 4 ? 2 : 1);
+  const int min_steps = ((tiles * 2 < kComputeUnits) ? 8 : 16) / ((elem_bytes == 4 ? 2 : 1) * (TR * elem_bytes / 128));
   if (want > r_steps / min_steps) want = r_steps / min_steps;
   if (want > 16) want = 16;
-  if (tiles * 2 >= (long long)kComputeUnits * slots || want < 2 || getenv("RZLINEAR_NO_SPLIT") != nullptr)
+  if (tiles * 2 >= (long long)kComputeUnits * slots || want < 2 || t.split == -1)
     want = 1;
   const int steps_per = (int)((r_steps + want - 1) / want);
   pl.splits = (r_steps + steps_per - 1) / steps_per;
@@ -210,15 +221,49 @@ static inline SplitPlan plan_split(int I, int J, int R, int elem_bytes) {
   return pl;
 }
 
+// Which instantiation of the contraction kernel runs a launch: C tile, wavefronts, LDS stages,
+// whether every tile and step is complete (no bounds checks), whether a ragged shape still
+// takes direct staging with edge pieces fetched from inside the operands, and the contracted
+// elements per step that follow from those.  One function decides for the launch and for
+// rz_plan_query.
+struct KernelForm {
+  int tile, waves, stages;
+  bool full, clamp;
+  int step;
+};
+
+static inline KernelForm kernel_form(int op, int I, int J, int R, int chunk, int tile, long long workgroups,
+                                     int elem_bytes, const rz_tuning& t) {
+  KernelForm f;
+  f.tile = tile;
+  f.stages = (tile == 128 && t.stages == 1) ? 1 : 2;
+  // 128 tile: with about one workgroup per compute unit, eight wavefronts (two per SIMD, 64 x 32
+  // each) hide latency better than four of 64 x 64; with more workgroups resident the
+  // four-wavefront form does less LDS traffic per flop
+  f.waves = tile == 256 ? 8 : tile == 64 ? 4 : (f.stages == 1 ? 4 : (workgroups <= kComputeUnits * 3 / 2 ? 8 : 4));
+  const bool direct_capable = elem_bytes == 2 && f.stages == 2 && tile >= 128;
+  const int step_plain = 128 / elem_bytes;
+  const int step_direct = (direct_capable && tile == 128 && f.waves == 8) ? 256 / elem_bytes : step_plain;
+  f.full = (I % tile == 0) && (J % tile == 0) && (R % step_direct == 0) && (chunk % step_direct == 0);
+  // a plain operand's 16-byte pieces must not straddle the end of its rows: forward / input-grad
+  // need R, weight-grad needs I and J, to be multiples of the piece
+  const int vec = 16 / elem_bytes;
+  const bool pieces_ok = op == kWeightGrad ? (I % vec == 0 && J % vec == 0 && I >= vec && J >= vec)
+                                           : (R % vec == 0 && R >= vec);
+  f.clamp = !f.full && direct_capable && pieces_ok && t.clamp != -1;
+  f.step = (f.full || f.clamp) ? step_direct : step_plain;
+  return f;
+}
+
 // Fills in the tiling fields of `p` and enqueues the kernel for `op` on `stream`; weight-grad
 // takes its plan (tile, split of M, scatter mode) from `plan`, the others ignore it.
 // (forward / input-grad take tile and split from `split`, or pick a tile and do not split).
 hipError_t launch_gemm_f32(int op, GemmParams p, const WeightGradPlan* plan, const SplitPlan* split,
-                           hipStream_t stream);
+                           const rz_tuning& tuning, hipStream_t stream);
 hipError_t launch_gemm_bf16(int op, GemmParams p, const WeightGradPlan* plan, const SplitPlan* split,
-                            hipStream_t stream);
+                            const rz_tuning& tuning, hipStream_t stream);
 hipError_t launch_gemm_f16(int op, GemmParams p, const WeightGradPlan* plan, const SplitPlan* split,
-                           hipStream_t stream);
+                           const rz_tuning& tuning, hipStream_t stream);
 
 struct WindowParams;
 // Enqueues the windowed weight-grad kernel; p.window and the tile grid must come from plan_window.

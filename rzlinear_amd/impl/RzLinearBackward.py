@@ -53,13 +53,14 @@ def weight_grad_hashed(input, output_grad, init_factor, M, K, N, H, R, BLOCK_SIZ
         if accumulate:
             flags |= _lib.WG_ACCUMULATE
     bias_grad = torch.empty((N,), device=output_grad.device, dtype=output_grad.dtype) if with_bias_grad else None
-    need = lib.rz_weight_grad_ex_workspace_bytes(M, K, N, H, BLOCK_SIZE_K, BLOCK_SIZE_N, code, flags,
-                                                 int(with_bias_grad))
+    tuning = _lib.current_tuning()
+    need = lib.rz_weight_grad_hashed_workspace_bytes(M, K, N, H, BLOCK_SIZE_K, BLOCK_SIZE_N, code, flags,
+                                                     int(with_bias_grad), tuning)
     ws = _lib.workspace(need, output_grad.device)
     _lib.check(lib.rz_weight_grad_hashed(
         x.data_ptr(), dy.data_ptr(), out.data_ptr(), bias_grad.data_ptr() if with_bias_grad else None,
         ws.data_ptr() if need else None, need, M, K, N, H, BLOCK_SIZE_K, BLOCK_SIZE_N, R, hash_levels,
-        float(init_factor), ldx, lddy, code, flags, stream))
+        float(init_factor), ldx, lddy, code, flags, tuning, stream))
     return out, bias_grad
 
 
@@ -133,9 +134,10 @@ def input_grad_hashed(output_grad, hashed_weight, init_factor, M, K, N, H, R, BK
     input_grad = torch.empty((M, K), device=output_grad.device, dtype=output_grad.dtype)
     lib = _lib.load()
     code = _lib.dtype_code(output_grad)
-    need = lib.rz_input_grad_workspace_bytes(M, K, N, H, BK, BN, code)
+    tuning = _lib.current_tuning()
+    need = lib.rz_input_grad_hashed_workspace_bytes(M, K, N, H, BK, BN, code, tuning)
     ws = _lib.workspace(need, output_grad.device)
     _lib.check(lib.rz_input_grad_hashed(
         dy.data_ptr(), hw.data_ptr(), input_grad.data_ptr(), ws.data_ptr() if need else None, need,
-        M, K, N, H, BK, BN, R, hash_levels, float(init_factor), lddy, K, code, stream))
+        M, K, N, H, BK, BN, R, hash_levels, float(init_factor), lddy, K, code, tuning, stream))
     return input_grad

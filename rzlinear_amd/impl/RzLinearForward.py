@@ -57,10 +57,11 @@ def forward_hashed(input, hashed_weight, bias, init_factor, M, K, N, H, R, BK, B
     lib = _lib.load()
     code = _lib.dtype_code(input)
     # skinny problems split the contraction and need a scratch buffer for the partial results
-    need = lib.rz_forward_workspace_bytes(M, K, N, H, BK, BN, code)
+    tuning = _lib.current_tuning()
+    need = lib.rz_forward_hashed_workspace_bytes(M, K, N, H, BK, BN, code, tuning)
     ws = _lib.workspace(need, input.device)
     _lib.check(lib.rz_forward_hashed(
         x.data_ptr(), hw.data_ptr(), bias.data_ptr() if bias is not None else None, output.data_ptr(),
         ws.data_ptr() if need else None, need, M, K, N, H, BK, BN, R, hash_levels, float(init_factor),
-        ldx, N, code, stream))
+        ldx, N, code, tuning, stream))
     return output

@@ -17,3 +17,19 @@ def oracle():
     from oracle import rz_oracle
     rz_oracle.build_c()
     return rz_oracle
+
+
+@pytest.fixture
+def tuned():
+    """tuned(tile=128, lds_image=-1, ...) makes the package's launchers pass these rz_tuning
+    overrides for the rest of the test (a later call replaces them); undone at teardown."""
+    import contextlib
+    from rzlinear_amd import _lib
+    stack = contextlib.ExitStack()
+
+    def apply(**fields):
+        stack.close()
+        stack.enter_context(_lib.tuning(**fields))
+
+    yield apply
+    stack.close()

@@ -21,6 +21,44 @@ def rel_err(out, ref):
     return float(np.abs(out - ref).max() / (scale if scale > 0 else 1.0))
 
 
+# Element-wise bound for the 16-bit kernels, next to the normalised bound above.  The kernels
+# multiply exactly (16-bit products fit fp32), accumulate in fp32 and round ONCE to the output
+# type, so against the float64 oracle on the same rounded inputs every element must satisfy
+#     |out - ref| <= ulp(type) * |ref|  +  1e-5 * max|ref|
+# (one output rounding: 2^-8 relative for bf16, 2^-10 for fp16 covers a whole unit in the last
+#  place; the second term is the fp32 accumulation over the contracted dimension).  This is
+# much tighter than 2e-2 of the tensor maximum and it is what exposes a polluted edge row or
+# column: the reference's own tests compare element-wise too (allclose(rtol=1e-3) in fp32,
+# python/tests/test_rz_linear.py:73,:113,:141).
+ULP = {torch.bfloat16: 2.0 ** -8, torch.float16: 2.0 ** -10, torch.float32: 2.0 ** -22}
+
+
+def elementwise_excess(out, ref, dtype, floor=1e-5):
+    """Largest |out - ref| / (ulp*|ref| + floor*max|ref|) over all elements: <= 1 passes."""
+    out = np.asarray(out, dtype=np.float64)
+    ref = np.asarray(ref, dtype=np.float64)
+    assert out.shape == ref.shape, (out.shape, ref.shape)
+    assert np.isfinite(out).all(), "non-finite values in the kernel output"
+    scale = np.abs(ref).max()
+    bound = ULP[dtype] * np.abs(ref) + floor * (scale if scale > 0 else 1.0)
+    return float((np.abs(out - ref) / bound).max()) if out.size else 0.0
+
+
+def assert_close(out, ref, dtype, what=""):
+    """Both bounds: the stated normalised tolerance and, element by element, the rounding bound."""
+    e = rel_err(out, ref)
+    assert e <= TOL[dtype], "%s: normalised max error %.3g > %.3g" % (what, e, TOL[dtype])
+    x = elementwise_excess(out, ref, dtype)
+    if x > 1.0:
+        out = np.asarray(out, dtype=np.float64)
+        ref = np.asarray(ref, dtype=np.float64)
+        scale = np.abs(ref).max()
+        bad = np.abs(out - ref) / (ULP[dtype] * np.abs(ref) + 1e-5 * (scale if scale > 0 else 1.0))
+        at = np.unravel_index(int(bad.argmax()), bad.shape)
+        raise AssertionError("%s: element %s is %.6g, expected %.6g (%.2f x the element-wise bound; %d elements "
+                             "beyond it)" % (what, at, out[at], ref[at], x, int((bad > 1.0).sum())))
+
+
 def make_inputs(M, K, N, H, dtype, seed, device="cuda"):
     """X ~ N(0,1), hashed_weight ~ U(-1/sqrt(K), 1/sqrt(K)), dY ~ N(0,1), rounded to dtype.
     Returns the device tensors and their exact float64 images for the oracle."""

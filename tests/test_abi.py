@@ -111,7 +111,44 @@ def test_status_codes(lib):
     assert lib.rz_weight_grad_workspace_bytes(8, 128, 128, 65536, 64, 64, 0) == 0
     assert lib.rz_weight_grad_workspace_bytes(8, 128, 128, 65536, 64, 64, 1) == 65536 * 4
     assert lib.rz_forward_hashed(one, one, None, one, None, 0, 8, 128, 128, 65536, 64, 64, _R(R1024), 5, 1.0,
-                                 128, 128, 0, None) == -9
+                                 128, 128, 0, None, None) == -9
+    # tuning overrides are validated
+    from rzlinear_amd import _lib
+    bad = _lib.Tuning(tile=96)
+    assert lib.rz_forward_hashed(one, one, None, one, None, 0, 8, 128, 128, 65536, 64, 64, _R(R1024), 2, 1.0,
+                                 128, 128, 0, ctypes.byref(bad), None) == -9
+    assert lib.rz_plan_query(0, 8, 128, 128, 65536, 64, 64, 0, 0, 0, ctypes.byref(bad), (ctypes.c_int32 * 8)()) == -9
     for code in range(0, -10, -1):
         assert lib.rz_status_string(code) not in (None, b"", b"unknown status")
     assert lib.rz_status_string(-99) == b"unknown status"
+
+
+def test_plan_slices_begin_on_step_boundaries(lib):
+    """Every slice of a cut contraction must start on a boundary of the kernel's step: a step's
+    table of tile offsets assumes that the step lies inside one hashed tile or covers whole
+    ones (a slice that began half-way into a 256-byte step would straddle two 128-row tiles).
+    Swept over shapes, element types and forced tiles through rz_plan_query."""
+    from rzlinear_amd import _lib
+    rng = np.random.default_rng(2024)
+    shapes = [(1024, 4352, 2048), (1024, 2176, 2048), (32, 10240, 10240), (128, 10240, 1024), (512, 8320, 1536)]
+    for _ in range(300):
+        shapes.append((int(rng.integers(1, 2048)), int(rng.integers(64, 12000)), int(rng.integers(64, 12000))))
+    seen_cut = 0
+    for (M, K, N) in shapes:
+        for code in (_lib.RZ_F32, _lib.RZ_BF16):
+            for tile in (0, 64, 128, 256):
+                with _lib.tuning(tile=tile):
+                    for op, R in ((0, K), (1, N), (2, M)):
+                        q = _lib.plan_query(op, M, K, N, 1 << 20, 128, 128, code)
+                        assert q["step"] in (32, 64, 128), q
+                        if q["mode"] == "window":
+                            continue
+                        assert q["slices"] >= 1 and (q["slices"] - 1) * q["slice_len"] < R <= q["slices"] * q["slice_len"], (q, R)
+                        if q["slices"] > 1:
+                            seen_cut += 1
+                            assert q["slice_len"] % q["step"] == 0, (M, K, N, code, tile, op, q)
+    assert seen_cut > 100
+    # the case that used to cut 4352 = 4 x 1088 under a 128-element step
+    with _lib.tuning():
+        q = _lib.plan_query(0, 1024, 4352, 2048, 1 << 20, 128, 128, _lib.RZ_BF16)
+    assert q["tile"] == 128 and q["slices"] > 1 and q["slice_len"] % 128 == 0, q

@@ -6,7 +6,7 @@ import numpy as np
 import pytest
 import torch
 
-from helpers import SEED_CONSTANTS, TOL, make_inputs, rargs, rel_err
+from helpers import SEED_CONSTANTS, TOL, assert_close, make_inputs, rargs, rel_err
 
 pytestmark = pytest.mark.gpu
 
@@ -129,22 +129,22 @@ TILE_CASES = [
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=lambda d: str(d).split(".")[-1])
-@pytest.mark.parametrize("env", [{"RZLINEAR_TILE": "64"}, {"RZLINEAR_TILE": "128"}, {"RZLINEAR_TILE": "256"},
-                                 {"RZLINEAR_TILE": "128", "RZLINEAR_STAGES": "1"},
-                                 {"RZLINEAR_TILE": "256", "RZLINEAR_NO_LDS_IMAGE": "1"}],
-                         ids=lambda e: "-".join("%s=%s" % (k.replace("RZLINEAR_", ""), v) for k, v in e.items()))
+@pytest.mark.parametrize("env", [{"tile": 64}, {"tile": 128}, {"tile": 256}, {"tile": 128, "stages": 1},
+                                 {"tile": 256, "lds_image": -1}],
+                         ids=lambda e: "-".join("%s=%s" % (k, v) for k, v in e.items()))
 @pytest.mark.parametrize("shape", TILE_CASES, ids=lambda s: "x".join(map(str, s)))
-def test_every_tile_shape_and_scatter_mode(oracle, monkeypatch, shape, env, dtype):
-    """The library picks its C tile and scatter path from the problem size; force each one."""
+def test_every_tile_shape_and_scatter_mode(oracle, shape, env, dtype):
+    """The library picks its C tile and scatter path from the problem size; force each one
+    (rz_tuning overrides)."""
+    from rzlinear_amd import _lib
     from rzlinear_amd.impl.RzLinearBackward import rz_linear_backward_tl
     from rzlinear_amd.impl.RzLinearForward import rz_linear_forward_tl
-    for k, v in env.items():
-        monkeypatch.setenv(k, v)
     M, K, N, H, BK, BN = shape
     _say("tiles", shape, env, dtype)
     (x, hw, dy), (x64, hw64, dy64) = make_inputs(M, K, N, H, dtype, seed=4)
-    y = rz_linear_forward_tl(x, hw, 1.0, M, K, N, H, *rargs(R1024), BLOCK_SIZE_K=BK, BLOCK_SIZE_N=BN)
-    dx, dhw = rz_linear_backward_tl(x, hw, dy, 1.0, M, K, N, H, *rargs(R1024), BLOCK_SIZE_K=BK, BLOCK_SIZE_N=BN)
+    with _lib.tuning(**env):
+        y = rz_linear_forward_tl(x, hw, 1.0, M, K, N, H, *rargs(R1024), BLOCK_SIZE_K=BK, BLOCK_SIZE_N=BN)
+        dx, dhw = rz_linear_backward_tl(x, hw, dy, 1.0, M, K, N, H, *rargs(R1024), BLOCK_SIZE_K=BK, BLOCK_SIZE_N=BN)
     torch.cuda.synchronize()
     assert rel_err(y.float().cpu().numpy(), oracle.forward(x64, hw64, N, BK, BN, R1024)) <= TOL[dtype]
     assert rel_err(dx.float().cpu().numpy(), oracle.input_grad(dy64, hw64, K, BK, BN, R1024)) <= TOL[dtype]
@@ -282,6 +282,33 @@ def test_skinny_problems_split_the_contraction(oracle, shape, dtype):
     assert rel_err(dx.float().cpu().numpy(), oracle.input_grad(dy64, hw64, K, BK, BN, R1024, 0.5)) <= TOL[dtype]
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=lambda d: str(d).split(".")[-1])
+@pytest.mark.parametrize("shape", [(1024, 4352, 2048, 70000, 128, 128), (1024, 2048, 4352, 70000, 128, 128),
+                                   (1024, 2176, 2048, 300000, 256, 128), (1000, 4360, 2040, 70000, 128, 256)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_cut_contraction_on_the_long_step_tile(oracle, shape, dtype):
+    """The 16-bit 128 tile in its eight-wavefront form walks the contraction in 128-element
+    steps; a contraction cut into slices must cut on those steps, or a slice would start
+    between two hashed tiles of 128 (or 256) rows and read offsets that nobody hashed.
+    4352 = 34 x 128 and 2176 = 17 x 128 do not divide evenly over the slices."""
+    from rzlinear_amd import _lib
+    from rzlinear_amd.impl.RzLinearBackward import rz_linear_backward_input_grad_tl
+    from rzlinear_amd.impl.RzLinearForward import rz_linear_forward_tl
+    M, K, N, H, BK, BN = shape
+    _say("cut contraction, long step", shape, dtype)
+    code = _lib.dtype_code(torch.empty(0, dtype=dtype))
+    plans = [_lib.plan_query(op, M, K, N, H, BK, BN, code) for op in (0, 1)]
+    assert any(p["tile"] == 128 and p["slices"] > 1 for p in plans), plans
+    for p in plans:
+        assert p["slices"] == 1 or p["slice_len"] % p["step"] == 0, p
+    (x, hw, dy), (x64, hw64, dy64) = make_inputs(M, K, N, H, dtype, seed=21)
+    y = rz_linear_forward_tl(x, hw, 1.0, M, K, N, H, *rargs(R1024), BLOCK_SIZE_K=BK, BLOCK_SIZE_N=BN)
+    dx = rz_linear_backward_input_grad_tl(dy, hw, 1.0, M, K, N, H, *rargs(R1024), BLOCK_SIZE_K=BK, BLOCK_SIZE_N=BN)
+    torch.cuda.synchronize()
+    assert_close(y.float().cpu().numpy(), oracle.forward(x64, hw64, N, BK, BN, R1024), dtype, "Y")
+    assert_close(dx.float().cpu().numpy(), oracle.input_grad(dy64, hw64, K, BK, BN, R1024), dtype, "dX")
+
+
 def _random_cases(n, seed):
     rng = np.random.default_rng(seed)
     cases = []
@@ -354,7 +381,7 @@ def test_random_shapes_16bit(oracle, shape):
     dhw, dbias = rz_linear_backward_weight_bias_grad_tl(x, dy, 0.75, M, K, N, H, *rargs(R), **kw)
     torch.cuda.synchronize()
     f = lambda t: t.float().cpu().numpy()
-    assert rel_err(f(y), oracle.forward(x64, hw64, N, BK, BN, R, 0.75) + bias.double().cpu().numpy()) <= TOL[dtype]
-    assert rel_err(f(dx), oracle.input_grad(dy64, hw64, K, BK, BN, R, 0.75)) <= TOL[dtype]
-    assert rel_err(f(dhw), oracle.weight_grad(x64, dy64, H, BK, BN, R, 0.75)) <= TOL[dtype]
-    assert rel_err(f(dbias), dy64.sum(axis=0)) <= TOL[dtype]
+    assert_close(f(y), oracle.forward(x64, hw64, N, BK, BN, R, 0.75) + bias.double().cpu().numpy(), dtype, "Y")
+    assert_close(f(dx), oracle.input_grad(dy64, hw64, K, BK, BN, R, 0.75), dtype, "dX")
+    assert_close(f(dhw), oracle.weight_grad(x64, dy64, H, BK, BN, R, 0.75), dtype, "dHW")
+    assert_close(f(dbias), dy64.sum(axis=0), dtype, "dbias")

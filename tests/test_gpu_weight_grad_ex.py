@@ -22,9 +22,8 @@ CASES = [
     (4100, 192, 160, 30000, 64, 64),     # long M: the reduction is cut into slices
     (40, 1500, 140, 9000, 64, 64),       # more tile rows than R steps: some workgroups never sum
 ]
-ENVS = [{}, {"RZLINEAR_TILE": "64"}, {"RZLINEAR_TILE": "128"}, {"RZLINEAR_TILE": "256"},
-        {"RZLINEAR_TILE": "128", "RZLINEAR_STAGES": "1"}, {"RZLINEAR_NO_LDS_IMAGE": "1"}]
-_env_id = lambda e: "-".join("%s=%s" % (k.replace("RZLINEAR_", ""), v) for k, v in e.items()) or "auto"
+ENVS = [{}, {"tile": 64}, {"tile": 128}, {"tile": 256}, {"tile": 128, "stages": 1}, {"lds_image": -1}]   # rz_tuning overrides
+_env_id = lambda e: "-".join("%s=%s" % (k, v) for k, v in e.items()) or "auto"
 _dt_id = lambda d: str(d).split(".")[-1]
 _shape_id = lambda s: "x".join(map(str, s))
 
@@ -37,15 +36,15 @@ def _say(*a):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16], ids=_dt_id)
 @pytest.mark.parametrize("env", ENVS, ids=_env_id)
 @pytest.mark.parametrize("shape", CASES, ids=_shape_id)
-def test_bias_grad_from_the_weight_grad_pass(oracle, monkeypatch, shape, env, dtype):
+def test_bias_grad_from_the_weight_grad_pass(oracle, shape, env, dtype):
+    from rzlinear_amd import _lib
     from rzlinear_amd.impl.RzLinearBackward import rz_linear_backward_weight_bias_grad_tl
-    for k, v in env.items():
-        monkeypatch.setenv(k, v)
     M, K, N, H, BK, BN = shape
     _say("weight+bias grad", shape, env, dtype)
     (x, _, dy), (x64, _, dy64) = make_inputs(M, K, N, H, dtype, seed=11)
-    dhw, dbias = rz_linear_backward_weight_bias_grad_tl(x, dy, 0.5, M, K, N, H, *rargs(R1024),
-                                                        BLOCK_SIZE_K=BK, BLOCK_SIZE_N=BN)
+    with _lib.tuning(**env):
+        dhw, dbias = rz_linear_backward_weight_bias_grad_tl(x, dy, 0.5, M, K, N, H, *rargs(R1024),
+                                                            BLOCK_SIZE_K=BK, BLOCK_SIZE_N=BN)
     torch.cuda.synchronize()
     assert dhw.shape == (H,) and dhw.dtype == dtype
     assert dbias.shape == (N,) and dbias.dtype == dtype
@@ -56,13 +55,12 @@ def test_bias_grad_from_the_weight_grad_pass(oracle, monkeypatch, shape, env, dt
 
 @pytest.mark.parametrize("out_dtype", ["same", "f32"])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=_dt_id)
-@pytest.mark.parametrize("env", [{}, {"RZLINEAR_NO_LDS_IMAGE": "1"}], ids=_env_id)
+@pytest.mark.parametrize("env", [{}, {"lds_image": -1}], ids=_env_id)
 @pytest.mark.parametrize("shape", CASES[:4], ids=_shape_id)
-def test_accumulate_into_an_existing_gradient(oracle, monkeypatch, shape, env, dtype, out_dtype):
+def test_accumulate_into_an_existing_gradient(oracle, tuned, shape, env, dtype, out_dtype):
     from rzlinear_amd.impl.RzLinearBackward import (rz_linear_backward_weight_bias_grad_tl,
                                                     rz_linear_backward_weight_grad_tl)
-    for k, v in env.items():
-        monkeypatch.setenv(k, v)
+    tuned(**env)
     M, K, N, H, BK, BN = shape
     _say("accumulate", shape, env, dtype, out_dtype)
     (x, _, dy), (x64, _, dy64) = make_inputs(M, K, N, H, dtype, seed=12)

@@ -1,5 +1,5 @@
 """GPU parity of the windowed weight-grad (large hashed_weight, short contraction): every
-workgroup owns a range of dHW and pulls in the tiles that touch it.  RZLINEAR_WINDOW=1 forces
+workgroup owns a range of dHW and pulls in the tiles that touch it.  rz_tuning.window = 1 forces
 that path wherever it is possible; the last test lets the library choose it by itself."""
 import sys
 
@@ -33,9 +33,9 @@ def _say(*a):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16], ids=_dt_id)
 @pytest.mark.parametrize("shape", CASES, ids=_shape_id)
-def test_windowed_weight_grad(oracle, monkeypatch, shape, dtype):
+def test_windowed_weight_grad(oracle, tuned, shape, dtype):
     from rzlinear_amd.impl.RzLinearBackward import rz_linear_backward_weight_grad_tl
-    monkeypatch.setenv("RZLINEAR_WINDOW", "1")
+    tuned(window=1)
     M, K, N, H, BK, BN = shape
     _say("windowed weight grad", shape, dtype)
     (x, _, dy), (x64, _, dy64) = make_inputs(M, K, N, H, dtype, seed=31)
@@ -51,7 +51,7 @@ def test_windowed_weight_grad(oracle, monkeypatch, shape, dtype):
                                               BLOCK_SIZE_N=BN)
     assert torch.equal(dhw, again)
     # and the scatter kernel agrees
-    monkeypatch.setenv("RZLINEAR_WINDOW", "0")
+    tuned(window=-1)
     scatter = rz_linear_backward_weight_grad_tl(x, dy, 0.5, M, K, N, H, *rargs(R1024), BLOCK_SIZE_K=BK,
                                                 BLOCK_SIZE_N=BN)
     torch.cuda.synchronize()
@@ -59,9 +59,9 @@ def test_windowed_weight_grad(oracle, monkeypatch, shape, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=_dt_id)
-def test_windowed_accumulate_and_fp32_buffer(oracle, monkeypatch, dtype):
+def test_windowed_accumulate_and_fp32_buffer(oracle, tuned, dtype):
     from rzlinear_amd.impl.RzLinearBackward import rz_linear_backward_weight_grad_tl
-    monkeypatch.setenv("RZLINEAR_WINDOW", "1")
+    tuned(window=1)
     M, K, N, H, BK, BN = 64, 512, 256, 90000, 64, 64
     _say("windowed accumulate", dtype)
     (x, _, dy), (x64, _, dy64) = make_inputs(M, K, N, H, dtype, seed=32)
@@ -82,7 +82,7 @@ def test_windowed_accumulate_and_fp32_buffer(oracle, monkeypatch, dtype):
 
 
 def test_library_picks_the_window_path_for_skinny_batches(oracle):
-    """M = 32 against K = N = 4096 with a 2^20-element hashed_weight: no environment switch."""
+    """M = 32 against K = N = 4096 with a 2^20-element hashed_weight: no tuning override."""
     from rzlinear_amd.impl.RzLinearBackward import rz_linear_backward_weight_grad_tl
     M, K, N, H, BK, BN = 32, 4096, 4096, 1 << 20, 64, 64
     _say("window path chosen by the plan")
@@ -107,10 +107,10 @@ def _random_window_cases(n, seed):
 
 
 @pytest.mark.parametrize("shape", _random_window_cases(24, 777), ids=_shape_id)
-def test_windowed_weight_grad_random_shapes(oracle, monkeypatch, shape):
+def test_windowed_weight_grad_random_shapes(oracle, tuned, shape):
     """Seeded random shapes through the window kernel: fp32 for even M, bf16 for odd M."""
     from rzlinear_amd.impl.RzLinearBackward import rz_linear_backward_weight_grad_tl
-    monkeypatch.setenv("RZLINEAR_WINDOW", "1")
+    tuned(window=1)
     M, K, N, H, BK, BN = shape
     dtype = torch.float32 if M % 2 == 0 else torch.bfloat16
     _say("windowed random", shape, dtype)

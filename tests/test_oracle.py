@@ -322,3 +322,29 @@ def test_legacy_hash_is_64_bit_and_uses_range_plus_one(oracle):
     # H == BK*BN is legal there: every tile at offset 0
     assert not oracle.c_tile_offsets(64, 64, 256, 16, 16, R, 3).any()
     assert (oracle.c_tile_offsets(640, 640, 257, 16, 16, R, 3) <= 1).all()
+
+
+@pytest.mark.parametrize("shape", [(48, 200, 136, 9000, 32, 64, 1.0), (130, 64, 64, 4097, 64, 64, 0.5),
+                                   (17, 300, 77, 20000, 16, 32, 2.0)])
+def test_timed_cpu_path_equals_the_oracle(oracle, shape):
+    """oracle/cpu_path.py (the CPU baseline that bench.py times: gather W through the index map,
+    torch.matmul, index_add_) against the numpy and C restatements, in float64 where the three
+    must agree to rounding, and in its own fp32 at the fp32 tolerance."""
+    import torch
+    from oracle import cpu_path
+    M, K, N, H, BK, BN, f = shape
+    R = [45007, 29440, 22221, 32190, 14791, 1316, 35275, 26448]
+    rng = np.random.default_rng(5)
+    x, hw, dy = rng.standard_normal((M, K)), rng.uniform(-1, 1, H) / K ** 0.5, rng.standard_normal((M, N))
+    path = cpu_path.CpuPath(K, N, H, BK, BN, R, init_factor=f)
+    assert np.array_equal(path.index_map.numpy(), oracle.index_map(K, N, H, BK, BN, R))
+    refs = (oracle.forward(x, hw, N, BK, BN, R, f), oracle.input_grad(dy, hw, K, BK, BN, R, f),
+            oracle.weight_grad(x, dy, H, BK, BN, R, f))
+    crefs = (oracle.c_forward(x, hw, N, BK, BN, R, f), oracle.c_input_grad(dy, hw, K, BK, BN, R, f),
+             oracle.c_weight_grad(x, dy, H, BK, BN, R, f))
+    for dt, tol in ((torch.float64, 1e-12), (torch.float32, 1e-5)):
+        got = path.step(torch.from_numpy(x).to(dt), torch.from_numpy(hw).to(dt), torch.from_numpy(dy).to(dt))
+        for g, r, c in zip(got, refs, crefs):
+            scale = np.abs(r).max()
+            assert np.abs(g.double().numpy() - r).max() <= tol * scale
+            assert np.abs(g.double().numpy() - c).max() <= tol * scale
