@@ -9,7 +9,14 @@ C ABI of librzlinear.so with caller-owned, pre-allocated outputs.  The default w
 one the headline metric is quoted on: M = N = K = 4096, 1000x compression (H = 16778), bf16,
 64x64 hashed tiles.  Prints ONE JSON line: fwd+bwd TFLOP/s (6*M*N*K flop per step), the
 roofline of the slowest of the three kernels, the dense torch.matmul (hipBLASLt/rocBLAS) rate on
-the same GPU and the reference's CPU path timed on the host cores.
+the same GPU under the same warm-up / step counts, a short sweep over the other baseline
+configurations and the reference's CPU path timed on the host cores.
+
+Order of the GPU work (the GPU's clock governor needs some 30 ms of load to settle after an
+idle period, so what runs when is part of the protocol and is reported):
+  output check -> dense legs (W warm-up + K timed) -> rz legs (W warm-up + K timed: the headline)
+  -> dense legs again (W + K) -> sweep -> CPU baseline.
+The dense rate quoted against the headline is the mean of the two dense runs around it.
 """
 import argparse
 import ctypes
@@ -24,86 +31,61 @@ if ROOT not in sys.path:
 
 HASH_SEED_1024 = [45007, 20011, 38363, 15263, 24507, 36489, 12234, 43027]
 
-# name -> (M, K, N, H, default dtype); tiles are 64x64 throughout
+# name -> (M, K, N, H, default dtype, input distributions); tiles are 64x64 throughout.
+# "normal": X ~ N(0,1), dY ~ N(0,1); "relu": X = relu(N(0,1)), dY ~ N(0, variance 1e-2).
 WORKLOADS = {
-    "square4096": (4096, 4096, 4096, 16778, "bf16"),      # the metric's configuration
-    "square2048": (2048, 2048, 2048, 16384, "bf16"),
-    "square1024": (1024, 1024, 1024, 16384, "bf16"),
-    "cpu_ref_1024": (1024, 1024, 1024, 65536, "fp32"),
-    "rec_mlp": (16384, 512, 1024, 5243, "bf16"),
-    "ffn": (8192, 4096, 16384, 67109, "bf16"),
-    "collision": (32768, 2048, 2048, 32768, "fp32"),
+    "square4096": (4096, 4096, 4096, 16778, "bf16", "normal"),      # the metric's configuration
+    "square2048": (2048, 2048, 2048, 16384, "bf16", "normal"),
+    "square1024": (1024, 1024, 1024, 16384, "bf16", "normal"),
+    "cpu_ref_1024": (1024, 1024, 1024, 65536, "fp32", "normal"),
+    "rec_mlp": (16384, 512, 1024, 5243, "bf16", "relu"),
+    "ffn": (8192, 4096, 16384, 67109, "bf16", "normal"),
+    "collision": (32768, 2048, 2048, 32768, "fp32", "normal"),
     # the shape grid of the reference's own benchmark script (python/bench/bench.py:10-11),
     # with its default compress_ratio 0.0625
-    "grid_32_1024": (32, 1024, 1024, 65536, "fp32"),
-    "grid_128_1024": (128, 1024, 1024, 65536, "fp32"),
-    "grid_1024_1024": (1024, 1024, 1024, 65536, "fp32"),
-    "grid_32_10240": (32, 10240, 10240, 6553600, "fp32"),
-    "grid_128_10240": (128, 10240, 10240, 6553600, "fp32"),
-    "grid_1024_10240": (1024, 10240, 10240, 6553600, "fp32"),
+    "grid_32_1024": (32, 1024, 1024, 65536, "fp32", "normal"),
+    "grid_128_1024": (128, 1024, 1024, 65536, "fp32", "normal"),
+    "grid_1024_1024": (1024, 1024, 1024, 65536, "fp32", "normal"),
+    "grid_32_10240": (32, 10240, 10240, 6553600, "fp32", "normal"),
+    "grid_128_10240": (128, 10240, 10240, 6553600, "fp32", "normal"),
+    "grid_1024_10240": (1024, 10240, 10240, 6553600, "fp32", "normal"),
 }
+# the baseline configurations beside the headline one: (workload, dtype) rows of the sweep
+SWEEP = [("cpu_ref_1024", "fp32"), ("square1024", "fp32"), ("square1024", "bf16"), ("square2048", "fp32"),
+         ("square2048", "bf16"), ("square4096", "fp32"), ("square4096", "bf16"), ("rec_mlp", "bf16"),
+         ("ffn", "bf16"), ("collision", "fp32")]
 # dense MFMA peaks of MI355X, TFLOP/s
 PEAK = {"bf16": 2500.0, "fp16": 2500.0, "fp32": 157.3}
-# HBM bytes per launch, measured once with rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE (KiB per
-# dispatch) and scaled by what the same counters read for a plain 256 MiB copy (FETCH_SIZE x2.0,
-# WRITE_SIZE x1.0); the rocprof summary with the raw readings is committed with the profiles.
-TRAFFIC_BYTES = {
+# HBM bytes per launch of each leg, from rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE (KiB per
+# dispatch, one run each), scaled by what the same counters read for a plain 256 MiB copy
+# (FETCH_SIZE x2.0, WRITE_SIZE x1.0).  A counter run cannot be taken inside this script, so the
+# figures are read off the committed summary named here; they describe the kernels of that
+# summary and are dropped (null) for a workload that has none.
+TRAFFIC = {
     ("square4096", "bf16"): {
-        "forward": int((16672.7 * 2.0 + 32768.0) * 1024),       # algorithmic: 64.03 MiB
-        "input_grad": int((16672.7 * 2.0 + 32768.0) * 1024),
-        "weight_grad": int((98457.7 * 2.0 + 16785.8) * 1024),   # X, dY re-read by 3 XCD groups; + partial images
+        "profile": "profiles/rz_gemm_bf16_square4096.txt",
+        "bytes": {"forward": int((16672.7 * 2.0 + 32768.0) * 1024),       # algorithmic: 64.03 MiB
+                  "input_grad": int((16672.7 * 2.0 + 32768.0) * 1024),
+                  "weight_grad": int((98457.7 * 2.0 + 16785.8) * 1024)},  # X, dY re-read by 3 XCD groups; + partial images
     },
 }
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=50)
-    ap.add_argument("--workload", default="square4096", choices=sorted(WORKLOADS))
-    ap.add_argument("--dtype", default=None, choices=["bf16", "fp16", "fp32"])
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--no-dense", action="store_true")
-    ap.add_argument("--cpu-budget", type=float, default=15.0, help="seconds of CPU-path timing")
-    ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MiB",
-                    help="only run a plain device-to-device copy of this many MiB (five launches) and exit: "
-                         "the known traffic against which rocprofv3's FETCH_SIZE / WRITE_SIZE are scaled")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        sys.exit("bench.py: this build measures one GPU only (no collectives, no sharding); run with --gpus 1")
-
-    import torch
-    from rzlinear_amd import _lib
-
-    if not torch.cuda.is_available():
-        sys.exit("bench.py: no GPU visible")
-    lib = _lib.load()   # raises if librzlinear.so is not built: there is no fallback
-    dev = torch.device("cuda:0")
-    torch.cuda.set_device(dev)
-
-    if args.calibrate_copy > 0:
-        n = args.calibrate_copy * 1024 * 1024
-        src = torch.empty((n,), dtype=torch.uint8, device=dev).random_(0, 255)
-        dst = torch.empty_like(src)
-        torch.cuda.synchronize()
-        for _ in range(5):
-            dst.copy_(src)
-        torch.cuda.synchronize()
-        print(json.dumps({"calibrate_copy_bytes_read": n, "calibrate_copy_bytes_written": n, "launches": 5}))
-        return
-
-    M, K, N, H, dflt = WORKLOADS[args.workload]
-    dname = args.dtype or dflt
+def make_workload(torch, _lib, name, dname, dev):
+    """Resident inputs, outputs and workspaces of one workload and its three legs."""
+    M, K, N, H, _, dist = WORKLOADS[name]
     dtype = {"bf16": torch.bfloat16, "fp16": torch.float16, "fp32": torch.float32}[dname]
     code = {"bf16": _lib.RZ_BF16, "fp16": _lib.RZ_F16, "fp32": _lib.RZ_F32}[dname]
+    lib = _lib.load()
     BK = BN = 64
     R = (ctypes.c_int32 * 8)(*HASH_SEED_1024)
-
     g = torch.Generator().manual_seed(1024)
-    x = torch.randn((M, K), generator=g).to(dtype).to(dev)
+    x = torch.randn((M, K), generator=g)
     hw = ((torch.rand((H,), generator=g) * 2 - 1) / K ** 0.5).to(dtype).to(dev)
-    dy = torch.randn((M, N), generator=g).to(dtype).to(dev)
+    dy = torch.randn((M, N), generator=g)
+    if dist == "relu":
+        x, dy = torch.relu(x), dy * 0.1
+    x, dy = x.to(dtype).to(dev), dy.to(dtype).to(dev)
     y = torch.empty((M, N), dtype=dtype, device=dev)
     dx = torch.empty((M, K), dtype=dtype, device=dev)
     dhw = torch.empty((H,), dtype=dtype, device=dev)
@@ -128,34 +110,138 @@ def main():
         _lib.check(lib.rz_weight_grad(x.data_ptr(), dy.data_ptr(), dhw.data_ptr(), ws.data_ptr(), ws_bytes,
                                       M, K, N, H, BK, BN, R, 1.0, K, N, code, stream))
 
-    legs = (("forward", fwd), ("input_grad", igrad), ("weight_grad", wgrad))
+    # the dense products of the same shapes, each in the operand layout that is fastest for
+    # the library (all "NN"), into pre-allocated outputs
+    w = torch.randn((K, N), generator=g).to(dtype).to(dev)
+    wt = w.t().contiguous()
+    xt = x.t().contiguous()
+    yd = torch.empty((M, N), dtype=dtype, device=dev)
+    dxd = torch.empty((M, K), dtype=dtype, device=dev)
+    dwd = torch.empty((K, N), dtype=dtype, device=dev)
+    dense_legs = (("forward", lambda: torch.matmul(x, w, out=yd)),
+                  ("input_grad", lambda: torch.matmul(dy, wt, out=dxd)),
+                  ("weight_grad", lambda: torch.matmul(xt, dy, out=dwd)))
+    wl = dict(M=M, K=K, N=N, H=H, BK=BK, BN=BN, R=R, code=code, dtype=dtype, dname=dname, x=x, hw=hw, dy=dy, y=y,
+              dx=dx, dhw=dhw, legs=(("forward", fwd), ("input_grad", igrad), ("weight_grad", wgrad)),
+              dense_legs=dense_legs, flop_gemm=2.0 * M * N * K)
+    return wl
 
-    for _ in range(args.warmup):
+
+def run_legs(torch, legs, warmup, steps):
+    """`warmup` untimed steps, then exactly `steps` timed ones between two synchronisations, with
+    HIP events on the launch stream around every leg.  Returns (ms per step by the host clock,
+    {leg: mean ms by the events})."""
+    for _ in range(warmup):
         for _, f in legs:
             f()
-    torch.cuda.synchronize()
-
-    # timed region: exactly `steps` steps; HIP events on the launch stream around every leg
-    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(len(legs) + 1)] for _ in range(args.steps)]
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(len(legs) + 1)] for _ in range(steps)]
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for s in range(args.steps):
+    for s in range(steps):
         ev[s][0].record()
         for i, (_, f) in enumerate(legs):
             f()
             ev[s][i + 1].record()
     torch.cuda.synchronize()
     t1 = time.perf_counter()
-    ms_per_step = (t1 - t0) * 1e3 / args.steps
-    flop_gemm = 2.0 * M * N * K
-    value = 3 * flop_gemm / (ms_per_step * 1e-3) / 1e12
+    leg_ms = {name: sum(ev[s][i].elapsed_time(ev[s][i + 1]) for s in range(steps)) / steps
+              for i, (name, _) in enumerate(legs)}
+    return (t1 - t0) * 1e3 / steps, leg_ms
 
-    leg_ms = {}
-    for i, (name, _) in enumerate(legs):
-        leg_ms[name] = sum(ev[s][i].elapsed_time(ev[s][i + 1]) for s in range(args.steps)) / args.steps
-    leg_tflops = {k: flop_gemm / (v * 1e-3) / 1e12 for k, v in leg_ms.items()}
-    slowest = max(leg_ms, key=leg_ms.get)
+
+def output_check(torch, _lib, wl):
+    """One pass of the three legs checked on the GPU against W materialised by rz_materialize and
+    torch's own products (float32 accumulate): a guard against timing a broken kernel, not the
+    parity test (that is tests/, against the oracle).  Returns the normalised max errors."""
+    lib = _lib.load()
+    M, K, N, H, BK, BN = (wl[k] for k in ("M", "K", "N", "H", "BK", "BN"))
+    stream = torch.cuda.current_stream().cuda_stream
+    idx = torch.empty((K, N), dtype=torch.float32, device=wl["x"].device)
+    ar = torch.arange(H, dtype=torch.float32, device=wl["x"].device)
+    _lib.check(lib.rz_materialize(ar.data_ptr(), idx.data_ptr(), K, N, H, BK, BN, wl["R"], 2, N, _lib.RZ_F32, stream))
+    idx = idx.long()
+    for _, f in wl["legs"]:
+        f()
+    W = wl["hw"].float()[idx]
+    xf, dyf = wl["x"].float(), wl["dy"].float()
+    rel = lambda out, ref: float((out.float() - ref).abs().max() / ref.abs().max())
+    errs = {"forward": rel(wl["y"], xf @ W), "input_grad": rel(wl["dx"], dyf @ W.t())}
+    dW = xf.t() @ dyf
+    ref = torch.zeros((H,), dtype=torch.float32, device=dW.device).index_add_(0, idx.reshape(-1), dW.reshape(-1))
+    errs["weight_grad"] = rel(wl["dhw"], ref)
+    torch.cuda.synchronize()
+    tol = 1e-3 if wl["dname"] == "fp32" else 2e-2   # (the fp32 comparator is itself an fp32 product)
+    bad = {k: v for k, v in errs.items() if not v <= tol}
+    if bad:
+        sys.exit("bench.py: output check failed, refusing to time: %s" % bad)
+    return {k: float("%.3g" % v) for k, v in errs.items()}
+
+
+def tflops(flop, ms):
+    return flop / (ms * 1e-3) / 1e12
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=50)
+    ap.add_argument("--workload", default="square4096", choices=sorted(WORKLOADS))
+    ap.add_argument("--dtype", default=None, choices=["bf16", "fp16", "fp32"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-dense", action="store_true")
+    ap.add_argument("--no-sweep", action="store_true")
+    ap.add_argument("--no-check", action="store_true")
+    ap.add_argument("--cpu-budget", type=float, default=15.0, help="seconds of CPU-path timing")
+    ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MiB",
+                    help="only run a plain device-to-device copy of this many MiB (five launches) and exit: "
+                         "the known traffic against which rocprofv3's FETCH_SIZE / WRITE_SIZE are scaled")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build measures one GPU only (no collectives, no sharding); run with --gpus 1")
+
+    import torch
+    from rzlinear_amd import _lib
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    _lib.load()   # raises if librzlinear.so is not built: there is no fallback
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    if args.calibrate_copy > 0:
+        n = args.calibrate_copy * 1024 * 1024
+        src = torch.empty((n,), dtype=torch.uint8, device=dev).random_(0, 255)
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"calibrate_copy_bytes_read": n, "calibrate_copy_bytes_written": n, "launches": 5}))
+        return
+
+    dname = args.dtype or WORKLOADS[args.workload][4]
+    wl = make_workload(torch, _lib, args.workload, dname, dev)
+    M, K, N, H, BK, BN = (wl[k] for k in ("M", "K", "N", "H", "BK", "BN"))
+    flop_gemm = wl["flop_gemm"]
     peak = PEAK[dname]
+
+    check = None if args.no_check else output_check(torch, _lib, wl)
+
+    dense_runs = []
+    if not args.no_dense:
+        dense_runs.append(run_legs(torch, wl["dense_legs"], args.warmup, args.steps))
+
+    # ---- the headline: W warm-up steps, then exactly K timed steps ----------------------------
+    ms_per_step, leg_ms = run_legs(torch, wl["legs"], args.warmup, args.steps)
+    value = tflops(3 * flop_gemm, ms_per_step)
+
+    if not args.no_dense:
+        dense_runs.append(run_legs(torch, wl["dense_legs"], args.warmup, args.steps))
+
+    leg_tflops = {k: tflops(flop_gemm, v) for k, v in leg_ms.items()}
+    slowest = max(leg_ms, key=leg_ms.get)
+    traffic = TRAFFIC.get((args.workload, dname))
     roofline = {
         "kernel": "rz_gemm_kernel<%s> (%s)" % (dname, slowest),
         "bound": "mfma",
@@ -163,52 +249,68 @@ def main():
         "peak": peak,
         "unit": "TFLOP/s",
         "frac": round(leg_tflops[slowest] / peak, 4),
-        "traffic": TRAFFIC_BYTES.get((args.workload, dname), {}).get(slowest),
+        "traffic": traffic["bytes"][slowest] if traffic else None,
+        "traffic_source": traffic["profile"] if traffic else None,
         "per_kernel_tflops": {k: round(v, 2) for k, v in leg_tflops.items()},
         "per_kernel_ms": {k: round(v, 4) for k, v in leg_ms.items()},
     }
 
     dense = None
-    if not args.no_dense:
-        w = torch.randn((K, N), generator=g).to(dtype).to(dev)
-        wt = w.t().contiguous()
-        xt = x.t().contiguous()
-
-        def timeit(fn, n=100):
-            for _ in range(20):
-                fn()
-            torch.cuda.synchronize()
-            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            a.record()
-            for _ in range(n):
-                fn()
-            b.record()
-            torch.cuda.synchronize()
-            return a.elapsed_time(b) / n
-
-        yd = torch.empty((M, N), dtype=dtype, device=dev)
-        dxd = torch.empty((M, K), dtype=dtype, device=dev)
-        dwd = torch.empty((K, N), dtype=dtype, device=dev)
-        # each dense product in the operand layout that is fastest for the library (all "NN")
-        d_ms = {
-            "forward": timeit(lambda: torch.matmul(x, w, out=yd)),
-            "input_grad": timeit(lambda: torch.matmul(dy, wt, out=dxd)),
-            "weight_grad": timeit(lambda: torch.matmul(xt, dy, out=dwd)),
-        }
-        d_tf = {k: flop_gemm / (v * 1e-3) / 1e12 for k, v in d_ms.items()}
-        dense_step = 3 * flop_gemm / (sum(d_ms.values()) * 1e-3) / 1e12
+    if dense_runs:
+        d_ms = {k: sum(r[1][k] for r in dense_runs) / len(dense_runs) for k in leg_ms}
+        d_step = sum(r[0] for r in dense_runs) / len(dense_runs)
+        dense_step_tf = tflops(3 * flop_gemm, d_step)
         dense = {
             "library": "torch.matmul (hipBLASLt/rocBLAS), operands pre-laid-out NN",
-            "per_kernel_tflops": {k: round(v, 2) for k, v in d_tf.items()},
-            "fwd_bwd_tflops": round(dense_step, 2),
-            "rz_over_dense": round(value / dense_step, 4),
+            "protocol": "same --warmup/--steps as the rz legs, once before and once after them; mean of the two",
+            "per_kernel_tflops": {k: round(tflops(flop_gemm, v), 2) for k, v in d_ms.items()},
+            "fwd_bwd_tflops": round(dense_step_tf, 2),
+            "fwd_bwd_tflops_before_after": [round(tflops(3 * flop_gemm, r[0]), 2) for r in dense_runs],
+            "rz_over_dense": round(value / dense_step_tf, 4),
+            "rz_over_dense_per_kernel": {k: round(d_ms[k] / leg_ms[k], 4) for k in leg_ms},
         }
-        del w, wt, xt, yd, dxd, dwd
+
+    # ---- the other baseline configurations, short runs outside the headline's timed region ----
+    sweep = None
+    if not args.no_sweep:
+        sweep = []
+        sw_warm, sw_steps = 5, 20
+        for name, dn in SWEEP:
+            if (name, dn) == (args.workload, dname):
+                row_rz, row_d = (ms_per_step, leg_ms), None
+                if dense_runs:
+                    row_d = (d_step, d_ms)
+                w2 = wl
+            else:
+                w2 = make_workload(torch, _lib, name, dn, dev)
+                row_d = run_legs(torch, w2["dense_legs"], sw_warm, sw_steps) if not args.no_dense else None
+                row_rz = run_legs(torch, w2["legs"], sw_warm, sw_steps)
+            fg = w2["flop_gemm"]
+            row = {"workload": name, "dtype": dn, "M": w2["M"], "K": w2["K"], "N": w2["N"], "H": w2["H"],
+                   "rz_tflops": {k: round(tflops(fg, v), 2) for k, v in row_rz[1].items()},
+                   "rz_fwd_bwd_tflops": round(tflops(3 * fg, row_rz[0]), 2),
+                   "pct_mfma_peak": round(100.0 * tflops(3 * fg, row_rz[0]) / PEAK[dn], 2)}
+            if row_d is not None:
+                row["dense_tflops"] = {k: round(tflops(fg, v), 2) for k, v in row_d[1].items()}
+                row["rz_over_dense"] = {k: round(row_d[1][k] / row_rz[1][k], 3) for k in row_rz[1]}
+                row["rz_over_dense"]["fwd_bwd"] = round(row_d[0] / row_rz[0], 3)
+            sweep.append(row)
+            if w2 is not wl:
+                del w2
+                torch.cuda.empty_cache()
+        sweep = {"protocol": "warm-up %d + %d timed steps per configuration (dense legs first, then rz); the headline "
+                             "configuration's row repeats the headline run" % (sw_warm, sw_steps), "rows": sweep}
 
     cpu_baseline = None
     if not args.no_cpu_baseline:
         from oracle import cpu_path   # checker/baseline only: never on the measured GPU path
-        torch.set_num_threads(min(os.cpu_count() or 1, 16))
+        # every host core this job may use: the machine's, unless the job was given a smaller
+        # share through OMP_NUM_THREADS (GPU boxes hand one GPU's job a share of the host)
+        share = os.environ.get("OMP_NUM_THREADS")
+        cores = os.cpu_count() or 1
+        if share and share.isdigit() and int(share) > 0:
+            cores = min(cores, int(share))
+        torch.set_num_threads(cores)
         sec, reps = cpu_path.time_cpu_path(M, K, N, H, BK, BN, HASH_SEED_1024, budget_s=args.cpu_budget)
         cpu_baseline = {
             "value": round(3 * flop_gemm / sec / 1e12, 4),
@@ -216,11 +318,13 @@ def main():
             "cores": torch.get_num_threads(),
             "kind": "port",
             "sample": "same shape M=%d K=%d N=%d H=%d in fp32: hash-gather W + torch.matmul fwd+bwd, median of %d "
-                      "steps (%.2f s each)" % (M, K, N, H, reps, sec),
+                      "steps (%.2f s each) on %d threads (host has %d cores, OMP_NUM_THREADS=%s)"
+                      % (M, K, N, H, reps, sec, torch.get_num_threads(), os.cpu_count() or 1, share),
         }
 
     out = {
-        "metric": "fwd+bwd TFLOP/s at M=N=K=4096, 1000x compression; % MFMA peak",
+        "metric": "fwd+bwd TFLOP/s at M=%d K=%d N=%d, %.0fx compression; %% MFMA peak" % (M, K, N, K * N / H)
+                  if args.workload != "square4096" else "fwd+bwd TFLOP/s at M=N=K=4096, 1000x compression; % MFMA peak",
         "value": round(value, 2),
         "unit": "TFLOP/s",
         "n_gpus": 1,
@@ -236,9 +340,11 @@ def main():
                                % (args.workload, M, K, N, H, BK, BN, dname),
                    "hash_seed": 1024, "init_factor": 1.0},
         "pct_mfma_peak": round(100.0 * value / peak, 2),
+        "output_check": check,
         "roofline": roofline,
         "dense_gemm": dense,
         "cpu_baseline": cpu_baseline,
+        "sweep": sweep,
     }
     print(json.dumps(out))
 
