@@ -45,7 +45,8 @@ typedef enum rz_status {
   RZ_ERR_HASH_OVERFLOW = -6,   /* hash intermediates would leave int32 (reference computes in int32) */
   RZ_ERR_WORKSPACE = -7,       /* workspace missing or too small */
   RZ_ERR_LAUNCH = -8,          /* HIP reported a launch error */
-  RZ_ERR_BAD_ARGUMENT = -9
+  RZ_ERR_BAD_ARGUMENT = -9,
+  RZ_ERR_SCRATCH_LIMIT = -10   /* rz_weight_grad_static: the problem needs more than the static scratch */
 } rz_status;
 
 typedef enum rz_dtype {
@@ -176,6 +177,24 @@ int rz_weight_grad(const void* X, const void* dY, void* dHW, void* workspace,
                    size_t workspace_bytes, int M, int K, int N, int H, int BK, int BN,
                    const int32_t R[8], float init_factor, int64_t ldx, int64_t lddy, int dtype,
                    void* stream);
+
+/*
+ * rz_weight_grad without a workspace argument and without any allocation: the partial images,
+ * the offset table or the fp32 image that rz_weight_grad keeps in the caller's workspace live in
+ * a 32 MiB device array that is part of the library (every GPU that loads the library holds its
+ * own copy until the process ends).  No counterpart in the reference; it is for callers that
+ * cannot allocate: code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc.  Same arguments, results and status codes as rz_weight_grad otherwise; a problem
+ * whose rz_weight_grad_workspace_bytes exceeds 32 MiB is refused with RZ_ERR_SCRATCH_LIMIT (at
+ * M = N = K = 4096, H = 16778 the need is 17 MB).  The first call on a device looks the array's
+ * address up (make that call outside a graph capture).  All calls on one GPU share the one array:
+ * calls that overlap in time on the same GPU — different streams, or different host threads —
+ * race on it and must be serialised by the caller; calls on one stream are ordered and safe.
+ * Nothing in the array needs to survive between calls, and each call writes what it reads.
+ */
+int rz_weight_grad_static(const void* X, const void* dY, void* dHW, int M, int K, int N, int H, int BK,
+                          int BN, const int32_t R[8], float init_factor, int64_t ldx, int64_t lddy,
+                          int dtype, void* stream);
 
 /*
  * Weight gradient for training loops that own their gradient buffers, optionally with the

@@ -22,7 +22,7 @@ EXPORTS = (
     "rz_input_grad_workspace_bytes", "rz_input_grad_ws", "rz_weight_grad_workspace_bytes", "rz_weight_grad", "rz_weight_grad_ex_workspace_bytes",
     "rz_weight_grad_ex", "rz_forward_hashed", "rz_input_grad_hashed", "rz_weight_grad_hashed", "rz_materialize",
     "rz_forward_hashed_workspace_bytes", "rz_input_grad_hashed_workspace_bytes",
-    "rz_weight_grad_hashed_workspace_bytes", "rz_plan_query",
+    "rz_weight_grad_hashed_workspace_bytes", "rz_plan_query", "rz_weight_grad_static",
 )
 
 
@@ -115,6 +115,9 @@ def load():
     lib.rz_weight_grad.restype = c_int
     lib.rz_weight_grad.argtypes = [c_vp, c_vp, c_vp, c_vp, c_sz, c_int, c_int, c_int, c_int, c_int, c_int,
                                    i32p, c_f, c_i64, c_i64, c_int, c_vp]
+    lib.rz_weight_grad_static.restype = c_int
+    lib.rz_weight_grad_static.argtypes = [c_vp, c_vp, c_vp, c_int, c_int, c_int, c_int, c_int, c_int,
+                                          i32p, c_f, c_i64, c_i64, c_int, c_vp]
     lib.rz_weight_grad_ex_workspace_bytes.restype = c_sz
     lib.rz_weight_grad_ex_workspace_bytes.argtypes = [c_int] * 7 + [ctypes.c_uint, c_int]
     lib.rz_weight_grad_ex.restype = c_int

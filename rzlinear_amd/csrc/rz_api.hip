@@ -3,6 +3,8 @@
 // the contraction kernels.
 #include "../../include/rzlinear.h"
 
+#include <atomic>
+
 #include "rz_common.h"
 #include "rz_launch.h"
 #include "rz_window.h"
@@ -417,6 +419,35 @@ static int weight_grad_impl(const void* X, const void* dY, void* dHW, void* dbia
 
 using namespace rz;
 
+// ---- scratch memory of the entry point that allocates nothing ---------------------------------
+// A file-scope device array stands in for the caller's workspace.  Every GPU that loads the
+// library holds its own copy, at its own address, until the process ends.  In host code the
+// array's NAME is only a handle for hipGetSymbolAddress — never a device address; the address
+// is looked up once per device (with that device current) and kept here.
+static constexpr size_t kScratchBytes = 32u << 20;
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+static constexpr int kMaxDevices = 64;
+static std::atomic<void*> scratch_ptr[kMaxDevices];
+
+// Device address of this device's scratch array, or null (status in *st) if it cannot be had.
+static void* scratch_of_current_device(int* st) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    *st = RZ_ERR_LAUNCH;
+    return nullptr;
+  }
+  void* p = scratch_ptr[dev].load(std::memory_order_acquire);
+  if (p == nullptr) {
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || p == nullptr) {
+      *st = RZ_ERR_LAUNCH;
+      return nullptr;
+    }
+    scratch_ptr[dev].store(p, std::memory_order_release);   // (a racing thread stores the same value)
+  }
+  *st = RZ_OK;
+  return p;
+}
+
 extern "C" {
 
 #define RZ_API __attribute__((visibility("default")))
@@ -435,6 +466,7 @@ RZ_API const char* rz_status_string(int status) {
     case RZ_ERR_WORKSPACE: return "workspace missing or smaller than rz_weight_grad_workspace_bytes";
     case RZ_ERR_LAUNCH: return "HIP kernel launch failed";
     case RZ_ERR_BAD_ARGUMENT: return "bad argument";
+    case RZ_ERR_SCRATCH_LIMIT: return "problem needs more scratch memory than the library's static 32 MiB: use the entry point that takes a workspace";
     default: return "unknown status";
   }
 }
@@ -587,6 +619,20 @@ RZ_API int rz_weight_grad(const void* X, const void* dY, void* dHW, void* worksp
                           int dtype, void* stream) {
   return weight_grad_impl(X, dY, dHW, nullptr, workspace, workspace_bytes, M, K, N, H, BK, BN, R,
                           init_factor, ldx, lddy, dtype, 0u, stream);
+}
+
+RZ_API int rz_weight_grad_static(const void* X, const void* dY, void* dHW, int M, int K, int N, int H, int BK,
+                                 int BN, const int32_t R[8], float init_factor, int64_t ldx, int64_t lddy,
+                                 int dtype, void* stream) {
+  // the same plan, kernels and checks as rz_weight_grad; only the workspace differs
+  if (dtype_bytes(dtype) != 0 && M >= 1 && K >= 1 && N >= 1 && H >= 1 &&
+      rz_weight_grad_workspace_bytes(M, K, N, H, BK, BN, dtype) > kScratchBytes)
+    return RZ_ERR_SCRATCH_LIMIT;
+  int st = RZ_OK;
+  void* ws = scratch_of_current_device(&st);
+  if (ws == nullptr) return st;
+  return weight_grad_impl(X, dY, dHW, nullptr, ws, kScratchBytes, M, K, N, H, BK, BN, R, init_factor, ldx, lddy,
+                          dtype, 0u, stream);
 }
 
 RZ_API size_t rz_weight_grad_hashed_workspace_bytes(int M, int K, int N, int H, int BK, int BN, int dtype,
