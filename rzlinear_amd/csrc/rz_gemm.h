@@ -5,8 +5,11 @@
 // in LDS and read from there as MFMA fragments.  The hashed operand (W) is fetched as 16-byte
 // pieces of hashed_weight at off(tk,tn) + kk*BN + nn; the pieces may start at any element, so
 // the loads are unaligned and rely on the hardware's unaligned global access.  Tile offsets
-// are hashed by a few threads into a small LDS table, several steps ahead of their use, so
-// the integer modulos stay off the critical path.
+// are hashed into an LDS table sixteen steps at a time, all threads sharing the work, so the
+// integer modulos cost every wavefront the same small share and stay off the critical path.
+// With direct staging everything a load address needs apart from the step is computed once per
+// thread (a 32-bit byte offset per piece); the step only moves a uniform base in scalar
+// registers, and a hashed piece adds its tile's table entry.
 //
 // Register staging (fp32, the 64 tile, ragged contracted dimension): global -> registers (issued
 // one or two steps ahead) -> LDS (one or two stages).  LDS layouts (X = I or J extent of the
@@ -168,9 +171,11 @@ struct GemmKernel {
   typedef Lds<A_LAYOUT, TI> LA;
   typedef Lds<B_LAYOUT, TJ> LB;
 
-  // offset table: kOffSlots windows (one per R step in flight) of kOffWindow entries; the
-  // weight-grad epilogue reuses it for the (TI/16) x (TJ/16) tiles of its C tile
-  static constexpr int kOffSlots = 4;
+  // offset table: kOffSlots windows (one per R step; two banks of kOffBank steps, one in use
+  // while the other is refilled) of kOffWindow entries; the weight-grad epilogue reuses it for
+  // the (TI/16) x (TJ/16) tiles of its C tile
+  static constexpr int kOffSlots = 32;    // two banks of kOffBank steps
+  static constexpr int kOffBank = 16;
   static constexpr int kOffWindow = (TR / 16) * (TJ / 16);
   static constexpr int kOffEntries =
       (OP == kWeightGrad) ? (TI / 16) * (TJ / 16) : kOffSlots * kOffWindow;
@@ -262,7 +267,7 @@ struct GemmKernel {
   static __device__ void run(const GemmParams& p, Smem& sm) {
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = tid >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // (uniform: lives in a scalar register)
     const int wave_i = wave / WJ, wave_j = wave % WJ;
     // Offset in the C tile of a wavefront's 32x32 block (a, b).  Forward and input-grad give a
     // wavefront one contiguous WTI x WTJ sub-tile (whole cache lines per store).  Weight-grad
@@ -309,6 +314,8 @@ struct GemmKernel {
         for (int e = 0; e < 16; e++) acc[a][b][e] = 0.f;
 
     u32x4_t ra[LA::kPieces], rb[LB::kPieces];
+    // elements of the last R step that lie beyond R (ragged contraction, direct staging)
+    const int tail = CLAMP ? steps * TR - (r_end - r_begin) : 0;
 
     // Bias gradient (COLSUM): the tiles_i workgroups of one tile column and slice stage the same
     // rows of dY, so they take turns: the workgroup whose turn it is adds the rows of that R
@@ -327,12 +334,37 @@ struct GemmKernel {
       else return off_window(p.h, j0, TJ, r0, TR);
     };
     // hash the tiles of R step `step` into its slot of the offset table
-    auto hash_step = [&](int step) {
+    // Hash the tiles of the kOffBank steps from `first` on into their slots of the offset table,
+    // all threads sharing the work (the integer modulos of the hash are long instruction
+    // sequences: done in bulk, every wavefront pays the same small share every kOffBank steps).
+    // With direct staging an entry is the tile offset plus the part of the within-tile offset
+    // that belongs to the step (a step inside a larger hashed tile starts r0 & (B - 1) rows /
+    // columns into it).
+    auto hash_bulk = [&](int first) {
       if constexpr (OP != kWeightGrad) {
-        if (step < steps) {
-          const OffWindow w = window(step);
-          off_fill(sm.off + (step & (kOffSlots - 1)) * kOffWindow, p.h, w, tid);
+        if (first < steps) {
+          const OffWindow w0 = window(first);              // count and ntn are the same for every step
+          const int cshift = __builtin_ctz(w0.count);     // (a power of two)
+          const int total = kOffBank << cshift;
+          for (int e = tid; e < total; e += kThreads) {
+            const int step = first + (e >> cshift), t = e & (w0.count - 1);
+            if (step < steps) {
+              const OffWindow w = window(step);
+              int v = (int)tile_offset(p.h, (uint32_t)(w.tk0 + t / w.ntn), (uint32_t)(w.tn0 + t % w.ntn));
+              if constexpr (kDirect) {
+                const int r0 = r_begin + step * TR;
+                v += (OP == kForward) ? (r0 & (p.h.BK - 1) & ~(TR - 1)) * p.h.BN : (r0 & (p.h.BN - 1) & ~(TR - 1));
+              }
+              sm.off[(step & (kOffSlots - 1)) * kOffWindow + t] = v;
+            }
+          }
         }
+      }
+    };
+    // in the main loops: at the first step of a bank, refill the other bank for the steps after it
+    auto hash_ahead = [&](int s) {
+      if constexpr (OP != kWeightGrad) {
+        if (s > 0 && (s & (kOffBank - 1)) == 0) hash_bulk(s + kOffBank);
       }
     };
     // Which 16-byte pieces of a source tile a thread moves.  A thread owns kPieces consecutive
@@ -466,8 +498,18 @@ struct GemmKernel {
       asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(dst), "v"(src)
                    : "memory", "m0");
     };
-    // all tiles of R step `step` -> LDS stage `st`
-    auto direct_issue = [&](int step, int st) {
+    // the same load with the address split into a uniform 64-bit base (scalar registers) and a
+    // per-lane 32-bit byte offset: the offsets are computed once, the base moves with the step
+    auto direct_load_so = [&](const void* base, uint32_t voff, const T* stage, int q, int pieces) {
+      typedef const T __attribute__((address_space(3)))* lds_ptr;
+      const uint32_t dst = __builtin_amdgcn_readfirstlane(
+          (uint32_t)(uintptr_t)(lds_ptr)(stage) + (uint32_t)((wave * pieces + q) * 1024));
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(voff), "s"(base)
+                   : "memory", "m0");
+    };
+    // the plain tiles of R step `step` -> LDS stage `st`, addresses computed in full (used for
+    // the last, partial step of a ragged contraction, whose pieces beyond R are redirected)
+    auto direct_issue_plain_slow = [&](int step, int st) {
       const int r0 = r_begin + step * TR;
 #pragma unroll
       for (int q = 0; q < LA::kPieces; q++) {
@@ -499,20 +541,82 @@ struct GemmKernel {
           const int cr = (CLAMP && gr >= p.R) ? p.R - 1 : gr;
           direct_load(gB + (int64_t)cr * p.ldb + cj, sm.b[st], q, LB::kPieces);
         }
-      } else {
-        const OffWindow w = window(step);
-        const int* tab = sm.off + (step & (kOffSlots - 1)) * kOffWindow;
-        int idx[LB::kPieces];
+      }
+    };
+    // Step-invariant part of every direct load of this thread, computed once.
+    //   plain operand : byte offset of the piece from the tile's first element of the step
+    //                   (edge clamping of ragged tile grids included: it does not depend on the step)
+    //   hashed operand: which entry of the step's offset window the piece's tile is, and the
+    //                   byte offset of the piece inside its tile.  A step starts on a multiple of
+    //                   TR, so with the hashed tile's extent along R a power of two, (r0 + x) &
+    //                   (B - 1) = (r0 & (B - 1)) + (x & (B - 1)) when B >= TR, and r0 drops out
+    //                   when B < TR; the step's part is uniform and is added to the table entries
+    //                   when they are hashed (see hash_bulk).
+    uint32_t a_voff[kDirect ? LA::kPieces : 1], b_voff[kDirect ? LB::kPieces : 1];
+    int b_tab[kDirect ? LB::kPieces : 1];
+    if constexpr (kDirect) {
 #pragma unroll
-        for (int q = 0; q < LB::kPieces; q++) {   // all table lookups first, then the loads
-          int row, col;
-          direct_src(LB{}, B_LAYOUT, q, row, col);
-          const int k = (OP == kForward) ? r0 + row : j0 + row;
-          const int n = (OP == kForward) ? j0 + col : r0 + col;
-          idx[q] = hashed_index(p.h, tab, w, k, n);
+      for (int q = 0; q < LA::kPieces; q++) {
+        int row, col;
+        direct_src(LA{}, A_LAYOUT, q, row, col);
+        if constexpr (A_LAYOUT == kRContig) {
+          const int gi = i0 + row;
+          const int ci = (!CLAMP || gi < p.I) ? row : p.I - 1 - i0;
+          a_voff[q] = (uint32_t)(((int64_t)ci * p.lda + col) * (int64_t)sizeof(T));
+        } else {
+          const int gi = i0 + col;
+          const int ci = (!CLAMP || gi < p.I) ? col : p.I - VEC - i0;
+          a_voff[q] = (uint32_t)(((int64_t)row * p.lda + ci) * (int64_t)sizeof(T));
         }
+      }
 #pragma unroll
-        for (int q = 0; q < LB::kPieces; q++) direct_load(gHW + idx[q], sm.b[st], q, LB::kPieces);
+      for (int q = 0; q < LB::kPieces; q++) {
+        int row, col;
+        direct_src(LB{}, B_LAYOUT, q, row, col);
+        if constexpr (OP == kWeightGrad) {
+          const int gj = j0 + col;
+          const int cj = (!CLAMP || gj < p.J) ? col : p.J - VEC - j0;
+          b_voff[q] = (uint32_t)(((int64_t)row * p.ldb + cj) * (int64_t)sizeof(T));
+          b_tab[q] = 0;
+        } else {
+          // (k, n) of the piece relative to the step's first row / column of W
+          // (forward: k = r0 + row, n = j0 + col; input-grad: k = j0 + row, n = r0 + col)
+          const int dk = row, dn = col;
+          const int kk = (OP == kForward) ? (p.h.BK >= TR ? dk : (dk & (p.h.BK - 1))) : ((j0 + dk) & (p.h.BK - 1));
+          const int nn = (OP == kForward) ? ((j0 + dn) & (p.h.BN - 1)) : (p.h.BN >= TR ? dn : (dn & (p.h.BN - 1)));
+          b_voff[q] = (uint32_t)((kk * p.h.BN + nn) * (int)sizeof(T));
+          const int tk_rel = (OP == kForward) ? (p.h.BK >= TR ? 0 : (dk >> p.h.bk_shift)) : (((j0 + dk) >> p.h.bk_shift) - (j0 >> p.h.bk_shift));
+          const int tn_rel = (OP == kForward) ? (((j0 + dn) >> p.h.bn_shift) - (j0 >> p.h.bn_shift)) : (p.h.BN >= TR ? 0 : (dn >> p.h.bn_shift));
+          const int ntn = (OP == kForward) ? ((TJ >> p.h.bn_shift) > 0 ? (TJ >> p.h.bn_shift) : 1)
+                                           : ((TR >> p.h.bn_shift) > 0 ? (TR >> p.h.bn_shift) : 1);
+          b_tab[q] = tk_rel * ntn + tn_rel;
+        }
+      }
+    }
+    // all tiles of R step `step` -> LDS stage `st`
+    auto direct_issue = [&](int step, int st) {
+      const int r0 = r_begin + step * TR;
+      if (CLAMP && tail > 0 && step == steps - 1) {   // (uniform) the partial last step
+        direct_issue_plain_slow(step, st);
+      } else {
+        // first element of the A tile of this step (uniform)
+        const T* a_base = (A_LAYOUT == kRContig) ? gA + (int64_t)i0 * p.lda + r0 : gA + (int64_t)r0 * p.lda + i0;
+#pragma unroll
+        for (int q = 0; q < LA::kPieces; q++) direct_load_so(a_base, a_voff[q], sm.a[st], q, LA::kPieces);
+        if constexpr (OP == kWeightGrad) {
+          const T* b_base = gB + (int64_t)r0 * p.ldb + j0;
+#pragma unroll
+          for (int q = 0; q < LB::kPieces; q++) direct_load_so(b_base, b_voff[q], sm.b[st], q, LB::kPieces);
+        }
+      }
+      if constexpr (OP != kWeightGrad) {
+        const int* tab = sm.off + (step & (kOffSlots - 1)) * kOffWindow;
+        uint32_t off[LB::kPieces];
+#pragma unroll
+        for (int q = 0; q < LB::kPieces; q++) off[q] = (uint32_t)tab[b_tab[q]];   // all lookups first, then the loads
+#pragma unroll
+        for (int q = 0; q < LB::kPieces; q++)
+          direct_load_so(gHW, off[q] * (uint32_t)sizeof(T) + b_voff[q], sm.b[st], q, LB::kPieces);
       }
     };
     // CLAMP, last R step with fewer than TR elements of R: once every wavefront's loads of that
@@ -521,7 +625,6 @@ struct GemmKernel {
     // whole rows where X is contiguous, the trailing 16-byte pieces of every row where R is
     // (R is then a multiple of the piece width).  A second barrier makes that visible.  Happens
     // at most once per workgroup.
-    const int tail = CLAMP ? steps * TR - (r_end - r_begin) : 0;
     auto clear_tail = [&](int st) {
       if constexpr (CLAMP) {
         if (tail > 0) {
@@ -591,9 +694,8 @@ struct GemmKernel {
     };
 
     if (steps > 0) {
-      hash_step(0);
-      hash_step(1);
-      hash_step(2);
+      hash_bulk(0);
+      hash_bulk(kOffBank);
       if constexpr (OP != kWeightGrad) __syncthreads();
       if constexpr (!kDirect) fetch(0);
     }
@@ -604,7 +706,7 @@ struct GemmKernel {
         commit(0);
         __syncthreads();
         if (s + 1 < steps) fetch(s + 1);
-        hash_step(s + 3);
+        hash_ahead(s);
         compute(0);
         __syncthreads();
       }
@@ -648,7 +750,7 @@ struct GemmKernel {
         constexpr int kFetchAt = kCommitAt;   // right behind the LDS writes that free the registers
         const int st = s & 1;
         // (its few threads branch, which ends a scheduling region: keep it out of the MFMA stream)
-        if constexpr (decltype(do_fetch)::value) hash_step(s + 4);
+        if constexpr (decltype(do_fetch)::value) hash_ahead(s);
 #pragma unroll
         for (int ks = 0; ks < NKS; ks++) {
           if (ks + 1 < NKS) {
@@ -695,7 +797,6 @@ struct GemmKernel {
           direct_issue(0, 0);
           if (steps > 1) {
             direct_issue(1, 1);
-            hash_step(3);
             // loads complete in order: all but the last step's worth have landed
             asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LA::kPieces + LB::kPieces) : "memory");
           } else {
@@ -704,7 +805,6 @@ struct GemmKernel {
         } else {
           commit(0);
           if (steps > 1) fetch(1);
-          hash_step(3);
         }
         __syncthreads();
         if constexpr (kDirect) {
