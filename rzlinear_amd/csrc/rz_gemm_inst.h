@@ -135,13 +135,13 @@ static hipError_t launch_gemm_t(int op, GemmParams p, const WeightGradPlan* plan
   }
 }
 
-template <typename T, int TBK, int TBN>
-static hipError_t launch_window_one(const WindowParams& p, int windows, hipStream_t stream) {
-  typedef WindowKernel<T, TBK, TBN> K;
+template <typename T, int TBK, int TBN, bool STAGED>
+static hipError_t launch_window_form(const WindowParams& p, int windows, hipStream_t stream) {
+  typedef WindowKernel<T, TBK, TBN, STAGED> K;
   static_assert(K::kFixedBytes + sizeof(float) * kWindowFloats <= 160 * 1024, "window does not fit the LDS");
   if (p.window < 4 || p.window > kWindowFloats || (p.window & 3) || windows < 1) return hipErrorInvalidValue;
   if ((long long)windows * p.window < p.H) return hipErrorInvalidValue;
-  auto kernel = rz_window_kernel<T, TBK, TBN>;
+  auto kernel = rz_window_kernel<T, TBK, TBN, STAGED>;
   const size_t smem = K::kFixedBytes + sizeof(float) * (size_t)p.window;
   static std::atomic<uint64_t> lds_limit_raised{0};
   if (smem > 64 * 1024) {
@@ -150,6 +150,15 @@ static hipError_t launch_window_one(const WindowParams& p, int windows, hipStrea
   }
   hipLaunchKernelGGL(kernel, dim3((unsigned)windows), dim3(K::kThreads), smem, stream, p);
   return hipGetLastError();
+}
+
+// 16-bit operands whose rows hold whole 16-byte pieces go through the staged form.
+template <typename T, int TBK, int TBN>
+static hipError_t launch_window_one(const WindowParams& p, int windows, hipStream_t stream) {
+  if constexpr (sizeof(T) == 2) {
+    if (p.K % 8 == 0 && p.N % 8 == 0) return launch_window_form<T, TBK, TBN, true>(p, windows, stream);
+  }
+  return launch_window_form<T, TBK, TBN, false>(p, windows, stream);
 }
 
 template <typename T>

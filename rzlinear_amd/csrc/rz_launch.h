@@ -179,12 +179,13 @@ static inline WindowPlan plan_window(int M, int K, int N, int H, int BK, int BN,
   pl.windows = (int)(((long long)H + w - 1) / w);
   // Rough times in microseconds, fitted to measurements at K = N = 10240, H = 6.5 M on MI355X.
   // Scatter kernel: K*N atomics at about 184 G/s plus the product.  Window kernel: every
-  // workgroup works through tiles * (window + tile) / H tiles; a tile costs about 0.7 us plus
-  // 0.3 us (16-bit) or 1.2 us (fp32) per 32 rows of M.
+  // workgroup works through tiles * (window + tile) / H tiles; a tile costs about 0.32 us plus
+  // 0.23 us (16-bit), or 0.7 us plus 1.0 us (fp32), per 32 rows of M (the operands of every tile come out of
+  // L2 again: tiles that share a window share no rows or columns of W).
   const double chunks = (double)((M + 31) / 32);
   const double per_wg = (double)tiles * ((double)w + (double)BK * BN) / (double)H;
   const double wg_rounds = (double)((pl.windows + kComputeUnits - 1) / kComputeUnits);
-  const double t_window = wg_rounds * per_wg * (0.72 + (elem_bytes == 4 ? 1.2 : 0.32) * chunks) + 30.0;
+  const double t_window = wg_rounds * per_wg * (elem_bytes == 4 ? 0.7 + 1.0 * chunks : 0.32 + 0.23 * chunks) + 28.0;
   const double t_scatter = 0.9 * (double)K * N / 184e3 + 2.0 * M * (double)K * N / 800e6;
   pl.use = t.window == 1 || t_window * 1.2 < t_scatter;
   return pl;

@@ -6,13 +6,21 @@
 // that takes microseconds).  Here a workgroup keeps dHW[w0, w0 + window) as an fp32 image in
 // LDS, finds the W tiles whose slice [off, off + BK*BN) meets that range by scanning the table
 // of tile offsets (hashed into the workspace by a small kernel of the same call; nothing is
-// kept between calls), computes each such tile's
-// X^T.dY product — operands are small and stay in L2 — and adds the part inside the window
-// with plain LDS read-add-write; barriers separate the adds of different tiles, whose slices
-// may overlap.  Finally the window is stored: every element of dHW is written exactly once, in
-// a fixed summation order (ascending tile id), with no atomics and no clearing pass.  A tile
-// that straddles a window boundary is computed by both neighbours.
+// kept between calls) and lists them, cut into strips of 32 rows, in ascending order.  Then
+// every WAVEFRONT takes strips from the list on its own: it computes the whole X^T.dY product
+// of a strip — the operands are small and stay in L2; a wavefront fetches its own operand
+// pieces (16-bit types: 16-byte pieces through a small LDS area of its own and the LDS
+// transpose read; otherwise the MFMA fragments element by element in their register layout),
+// so no wavefront waits for another — and adds the part inside the window with plain LDS
+// read-add-write.  Slices of different
+// tiles may overlap: a tile is added only after every earlier tile of the list whose slice
+// meets its own has been added (a flag per list entry, polled in LDS), so the summation order
+// of every element is the list order whatever the timing.  Finally the window is stored: every
+// element of dHW is written exactly once, with no atomics and no clearing pass.  A tile that
+// straddles a window boundary is computed by both neighbours.
 #pragma once
+
+#include <type_traits>
 
 #include "rz_gemm.h"
 
@@ -33,46 +41,86 @@ struct WindowParams {
   int out_f32;       // dHW is fp32 whatever T is
 };
 
-// TBK x TBN is the hashed tile (compile time).  A workgroup is kTeams teams of one wavefront
-// per 32x32 block of a tile.  The teams multiply different tiles at the same time (several
-// wavefronts per SIMD hide each other's latencies) and then add them into the window one
-// team after the other, in list order.
-template <typename T, int TBK, int TBN>
+// TBK x TBN is the hashed tile (compile time).  The unit of work is a strip of 32 rows of a tile
+// (its slice of hashed_weight is the 32 * TBN elements from off + 32 * TBN * strip on): a
+// wavefront holds the strip's 32x32 blocks in registers.
+// STAGED (16-bit types, K and N multiples of the 16-byte piece): operands travel as 16-byte
+// pieces through the wavefront's staging area; otherwise fragments are loaded element by element.
+template <typename T, int TBK, int TBN, bool STAGED>
 struct WindowKernel {
-  // the operand staging (padded LDS layouts, transpose reads) of the contraction kernel
-  typedef GemmKernel<T, kWeightGrad, TBK, TBN, TBK / 32, TBN / 32, 1, false> G;
-  typedef typename G::LA LA;
-  typedef typename G::LB LB;
+  static_assert(!STAGED || sizeof(T) == 2, "staging serves the LDS transpose read of the 16-bit types");
+  static_assert(TBK % 32 == 0 && TBN % 32 == 0, "a tile is whole 32x32 blocks");
+  typedef ElemTraits<T> Tr;
   typedef typename Mfma<T>::Frag Frag;
-  static constexpr int kTeamThreads = G::kThreads;
-  static constexpr int kTeams = sizeof(T) == 4 ? 2 : 4;
-  static constexpr int kThreads = kTeamThreads * kTeams;
+  static constexpr int kThreads = 1024;
   static constexpr int kWaves = kThreads / 64;
-  static constexpr int VEC = G::VEC;
-  static constexpr int kRows = 32;                 // rows of M per staged chunk
-  static constexpr int kPiecesA = kRows * LA::kCpr / kTeamThreads;
-  static constexpr int kPiecesB = kRows * LB::kCpr / kTeamThreads;
-  static_assert(kRows * LA::kCpr % kTeamThreads == 0 && kRows * LB::kCpr % kTeamThreads == 0, "chunk must split evenly");
-  static_assert(kRows % G::KS == 0 && kRows <= G::TR, "chunk rows must suit the fragment reads");
-  static constexpr int kList = kThreads;           // capacity of the list of tiles found
-  static constexpr int kBatch = 8;                 // tile offsets a thread loads at a time
+  static constexpr int kStrips = TBK / 32;               // strips of a tile
+  static constexpr int kStripElems = 32 * TBN;           // elements of hashed_weight under a strip
+  static constexpr int BI = 1, BJ = TBN / 32;            // blocks of a strip
+  static constexpr int KS = Tr::kMfmaK;                  // rows of M one MFMA contracts (16 or 2)
+  // rows of M loaded ahead as one group (16 wavefronts per compute unit leave 128 registers each)
+  static constexpr int kGroupRows = sizeof(T) == 4 ? 8 : 16;
+  static constexpr int GS = kGroupRows / KS;             // MFMA steps per group
+  static constexpr int kBatch = STAGED ? 8 : 4;           // tile offsets a lane loads at a time
+  static constexpr bool k16 = sizeof(T) == 2;
+  // 16-bit types: a wavefront's own staging area, 16 rows of X (32 columns) and of dY (TBN
+  // columns) per group; the list is kept shorter to make room for it next to the window
+  static constexpr int kStageX = 16 * 32, kStageElems = STAGED ? kStageX + 16 * TBN : 8;
+  static constexpr int kList = STAGED ? 960 : kThreads * kStrips;   // capacity of the list of strips found
+  static_assert(!STAGED || TBN == 64, "the staged dY rows are swizzled as two 64-byte chunks");
 
   struct Smem {
-    alignas(16) T a[kTeams][kRows * LA::kPitch];
-    alignas(16) T b[kTeams][kRows * LB::kPitch];
-    int list[kList];              // ids of the tiles found in this pass, ascending
-    int offs[kList];              // ... and their offsets in hashed_weight
+    int list[kList];              // strips found in this pass (tile id * kStrips + strip), ascending
+    int offs[kList];              // ... their offsets in hashed_weight
+    int done[kList];              // ... and whether they have been added to the window
     int count[2][kWaves];
+    alignas(16) T stage[kWaves][kStageElems];
     alignas(16) float window[4];  // the image of dHW[w0, w0 + window) starts here, then 64
                                   // dump slots
   };
   static constexpr size_t kFixedBytes = offsetof(Smem, window) + sizeof(float) * 64;   // + dump slots
 
+  // MFMA fragment of a 32-wide block of a row-major matrix (rows = the contracted dimension M).
+  //   16-bit: lane l holds rows m0 + r0 + (l >> 5) * 8 + j, j = 0..7, of column (l & 31)
+  //   fp32  : lane l holds row m0 + r0 + (l >> 5) of column (l & 31)
+  // `rows` points at row m0 (a row of the matrix) and the first column of the strip (clamped into
+  // the matrix); `lane_col` is the lane's column inside the strip, or 0 with col_ok = false when
+  // that column lies outside the matrix.  whole = every row of the group exists, the usual
+  // case.  Whatever is outside reads an element inside the matrix instead and is replaced by zero.
+  static __device__ __forceinline__ Frag load_frag(const T* __restrict__ rows, int64_t ld, int r0, int m0, int M,
+                                                   int lane, int lane_col, bool col_ok, bool whole) {
+    const int mg = lane >> 5;
+    if constexpr (sizeof(T) == 4) {
+      const bool ok = col_ok && (whole || m0 + r0 + mg < M);
+      const float v = reinterpret_cast<const float*>(rows)[ok ? (uint32_t)((r0 + mg) * (int)ld + lane_col) : 0u];
+      return ok ? v : 0.f;
+    } else {
+      const uint16_t* r16 = reinterpret_cast<const uint16_t*>(rows);
+      u32x4_t f = {0u, 0u, 0u, 0u};
+      if (whole) {
+        // the rows j are a uniform distance apart: uniform base per row, one lane offset
+        // (a lane outside the matrix has lane_col = 0: it reads the strip's first column)
+        const uint32_t off = (uint32_t)(mg * 8 * (int)ld + lane_col);
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+          const uint32_t v = (r16 + (int64_t)(r0 + j) * ld)[off];
+          f[j >> 1] |= (col_ok ? v : 0u) << (16 * (j & 1));
+        }
+      } else {
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+          const bool ok = col_ok && (m0 + r0 + mg * 8 + j < M);
+          const uint32_t v = r16[ok ? (uint32_t)((r0 + mg * 8 + j) * (int)ld + lane_col) : 0u];
+          f[j >> 1] |= (ok ? v : 0u) << (16 * (j & 1));
+        }
+      }
+      return f;
+    }
+  }
+
   static __device__ void run(const WindowParams& p, Smem& sm) {
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int team = wave / (kTeamThreads / 64), ttid = tid % kTeamThreads;
-    const int twave = wave % (kTeamThreads / 64);
-    const int wave_i = twave / (TBN / 32), wave_j = twave % (TBN / 32);
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     float* __restrict__ win = sm.window;
     const long long w0 = (long long)blockIdx.x * p.window;
     const int wlen = (p.H - w0) < p.window ? (int)(p.H - w0) : p.window;
@@ -85,186 +133,308 @@ struct WindowKernel {
     }
 
     const int total = p.tiles_k * p.tiles_n;
-    const int nchunks = (p.M + kRows - 1) / kRows;
-    f32x16_t acc;
-#pragma unroll
-    for (int e = 0; e < 16; e++) acc[e] = 0.f;
-    u32x4_t ra[kPiecesA], rb[kPiecesB];
+    const int ngroups = (p.M + kGroupRows - 1) / kGroupRows;
 
-    // 16 bytes at (row, col) of a row-major matrix, zero outside it.  When the column limit is a
-    // multiple of the vector width (`aligned`, the same for all threads) a piece is inside or
-    // outside as a whole: the load is then issued unconditionally from a clamped address, and
-    // the zero is selected only when the piece goes to LDS — nothing between the load and the
-    // next commit touches the loaded registers, so the load stays in flight that long.
-    auto piece = [&](const T* base, int64_t ld, int row, int row_lim, int col, int col_lim, bool aligned,
-                     bool& ok) -> u32x4_t {
-      ok = true;
-      if (!aligned) return load_plain<T, false>(base, ld, row, row_lim, col, col_lim);
-      ok = row < row_lim && col < col_lim;
-      u32x4_t v;
-      __builtin_memcpy(&v, base + (ok ? (int64_t)row * ld + col : 0), 16);
-      return v;
-    };
-    const bool aligned = (p.K % VEC == 0) && (p.N % VEC == 0);
-    bool oka[kPiecesA], okb[kPiecesB];
-    // global -> registers: chunk c (rows of M) of the X and dY tiles of W tile `id`
-    auto fetch = [&](int id, int c) {
-      const int tk = id / p.tiles_n, tn = id - tk * p.tiles_n;
-      const int m0 = c * kRows;
+    f32x16_t acc[BI][BJ];
 #pragma unroll
-      for (int q = 0; q < kPiecesA; q++) {
-        const int pc = ttid + q * kTeamThreads;
-        ra[q] = piece(gX, p.ldx, m0 + pc / LA::kCpr, p.M, tk * TBK + (pc % LA::kCpr) * VEC, p.K, aligned, oka[q]);
-      }
+    for (int a = 0; a < BI; a++)
 #pragma unroll
-      for (int q = 0; q < kPiecesB; q++) {
-        const int pc = ttid + q * kTeamThreads;
-        rb[q] = piece(gdY, p.lddy, m0 + pc / LB::kCpr, p.M, tn * TBN + (pc % LB::kCpr) * VEC, p.N, aligned, okb[q]);
-      }
-    };
-    auto commit = [&]() {
-      const u32x4_t z = {0u, 0u, 0u, 0u};
+      for (int b = 0; b < BJ; b++)
 #pragma unroll
-      for (int q = 0; q < kPiecesA; q++) {
-        const int pc = ttid + q * kTeamThreads;
-        G::template lds_put<kRStrided, LA>(sm.a[team], pc / LA::kCpr, pc % LA::kCpr, oka[q] ? ra[q] : z);
-      }
-#pragma unroll
-      for (int q = 0; q < kPiecesB; q++) {
-        const int pc = ttid + q * kTeamThreads;
-        G::template lds_put<kRStrided, LB>(sm.b[team], pc / LB::kCpr, pc % LB::kCpr, okb[q] ? rb[q] : z);
-      }
-    };
-    auto compute = [&]() {
-#pragma unroll
-      for (int ks = 0; ks < kRows / G::KS; ks++) {
-        const Frag fa = G::template lds_frag<kRStrided, LA>(sm.a[team], wave_i * 32, ks, lane);
-        const Frag fb = G::template lds_frag<kRStrided, LB>(sm.b[team], wave_j * 32, ks, lane);
-        acc = Mfma<T>::run(fa, fb, acc);
-      }
-    };
-    // add this wavefront's finished 32x32 block of the tile at offset `tile_off` into the
-    // window and clear it; all reads first, then the adds, then all writes (the 16 addresses of
-    // a lane are distinct)
-    auto add_to_window = [&](int tile_off) {
-      // (offsets and window starts are below 2^31, so their difference fits an int)
-      const int base = (int)((long long)tile_off - w0) + (wave_i * 32 + (lane >> 5) * 4) * TBN + wave_j * 32 + (lane & 31);
-      // elements outside the window go to a dump slot behind it: no branches, so
-      // the 16 reads and the 16 writes each go out back to back
-      const int dump = p.window + lane;   // (shared between wavefronts: its contents are never used)
-      int at[16];
-      float cur[16];
-#pragma unroll
-      for (int e = 0; e < 16; e++) {
-        const int a = base + ((e >> 2) * 8 + (e & 3)) * TBN;
-        at[e] = (a >= 0 && a < wlen) ? a : dump;
-        cur[e] = win[at[e]];
-      }
-#pragma unroll
-      for (int e = 0; e < 16; e++) {
-        win[at[e]] = cur[e] + acc[e] * p.scale;
-        acc[e] = 0.f;
-      }
-    };
+        for (int e = 0; e < 16; e++) acc[a][b][e] = 0.f;
+    // two register sets: the fragments of the next group are loaded while this one is multiplied
+    Frag fa[2][GS][BI], fb[2][GS][BJ];
+    // 16-bit staged path: the raw 16-byte pieces instead (one of X, two of dY per lane and group)
+    u32x4_t px[2], py[2][2];
+    bool okx[2], oky[2][2];
 
-    // The tile ids are examined kThreads at a time; the tiles that meet the window are appended
-    // to the list in ascending order (ballot + prefix inside a wavefront, counts across them).
-    // With a hash that spreads the tiles evenly the list holds every hit after one sweep; if
-    // it could overflow, the tiles found so far are worked through first.
-    int next_id = 0;
-    int parity = 0;   // the counts are double-buffered: one barrier per batch of ids
-    while (next_id < total) {
-      int found = 0;
-      while (next_id < total && found + kThreads <= kList) {
-        // a thread's next kBatch offsets are loaded together (one memory latency, not kBatch)
-        int batch_off[kBatch];
+    // Listing the strips that meet the window, in ascending (tile, strip) order.  The tile ids of
+    // a range [lo, hi) are dealt to the wavefronts in contiguous chunks; every wavefront first
+    // counts the strips of its chunk that meet the window, the counts are added up (one
+    // barrier), then it examines its chunk again and writes its strips behind those of the
+    // wavefronts before it.  Normally the range is the whole table and the list (kList entries)
+    // takes every hit; if it would overflow, the range is halved until its hits fit, and the
+    // rest of the table follows in further rounds.  (A range of one tile has at most kStrips
+    // hits, so the halving ends.)
+    auto strips_of = [&](int id, int off, unsigned long long* mask) -> int {
+      // ballots of "strip s of tile id meets the window" over the wavefront; returns their total
+      int n = 0;
 #pragma unroll
-        for (int j = 0; j < kBatch; j++) {
-          const int id = next_id + j * kThreads + tid;
-          batch_off[j] = p.offsets[id < total ? id : total - 1];
-        }
-#pragma unroll
-        for (int j = 0; j < kBatch; j++) {
-          if (!(next_id < total && found + kThreads <= kList)) break;   // (the same for all threads)
-          const int my_id = next_id + tid;
-          const long long my_off = batch_off[j];
-          const bool hit = my_id < total && my_off < w0 + wlen && my_off + TBK * TBN > w0;
-          const unsigned long long mask = __ballot(hit);
-          if (lane == 0) sm.count[parity][wave] = __popcll(mask);
-          __syncthreads();   // (first time round: also the cleared window, the finished list)
-          int before = 0, batch = 0;
-#pragma unroll
-          for (int w = 0; w < kWaves; w++) {
-            const int c = __builtin_amdgcn_readfirstlane(sm.count[parity][w]);
-            before += (w < wave) ? c : 0;
-            batch += c;
-          }
-          if (hit) {
-            const int at = found + before + __popcll(mask & ((1ull << lane) - 1ull));
-            sm.list[at] = my_id;
-            sm.offs[at] = (int)my_off;
-          }
-          found += batch;
-          next_id += kThreads;
-          parity ^= 1;
-        }
+      for (int s = 0; s < kStrips; s++) {
+        const long long so = (long long)off + (long long)s * kStripElems;
+        mask[s] = __ballot(id >= 0 && so < w0 + wlen && so + kStripElems > w0);
+        n += __popcll(mask[s]);
       }
-      __syncthreads();   // list complete
-
-      // Round r: team t takes list entry r * kTeams + t.  Every team runs the same number of
-      // chunks per round, so the barriers below are reached by all wavefronts together; a team
-      // without a tile only keeps step.
-      const int rounds = (found + kTeams - 1) / kTeams;
-      int entry = team;                                     // this team's current list entry
-      if (entry < found) fetch(sm.list[entry], 0);
-      for (int r = 0; r < rounds; r++) {
-        const bool have = entry < found;
-        const int tile_off = have ? __builtin_amdgcn_readfirstlane(sm.offs[entry]) : 0;
-        for (int c = 0; c < nchunks; c++) {
-          if (have) commit();
-          __syncthreads();   // staged chunks visible
-          // the next chunk's global loads fly during this chunk's product
-          if (c + 1 < nchunks) {
-            if (have) fetch(sm.list[entry], c + 1);
-          } else if (entry + kTeams < found) {
-            fetch(sm.list[entry + kTeams], 0);
+      return n;
+    };
+    int lo = 0;
+    while (lo < total) {
+      int hi = total, found = 0, chunk = 0;
+      for (;;) {
+        chunk = (hi - lo + kWaves - 1) / kWaves;
+        const int begin = lo + wave * chunk, end = begin + chunk < hi ? begin + chunk : hi;
+        int mine = 0;
+        for (int id0 = begin; id0 < end; id0 += 64 * kBatch) {
+          // a lane's next kBatch offsets are loaded together (one memory latency, not kBatch)
+          int offv[kBatch];
+#pragma unroll
+          for (int u = 0; u < kBatch; u++) {
+            const int id = id0 + u * 64 + lane;
+            offv[u] = id < end ? p.offsets[id] : 0;
           }
-          if (have) compute();
-          if (c + 1 < nchunks) __syncthreads();   // fragments read: the stages may be overwritten
+#pragma unroll
+          for (int u = 0; u < kBatch; u++) {
+            const int id = id0 + u * 64 + lane;
+            unsigned long long mask[kStrips];
+            mine += strips_of(id < end ? id : -1, offv[u], mask);
+          }
         }
-        // Tiles whose slices overlap must not be added at the same time.  With a large
-        // hashed_weight the kTeams tiles of a round rarely overlap: then all teams add at once;
-        // otherwise one team after the other.  (The decision depends on the offsets alone, so
-        // the summation order stays a function of the problem.)
-        bool overlap = false;
-        {
-          int round_off[kTeams];
+        __syncthreads();   // (the counts of the previous attempt or round have been read)
+        if (lane == 0) sm.count[0][wave] = mine;
+        __syncthreads();
+        found = 0;
 #pragma unroll
-          for (int t = 0; t < kTeams; t++) {
-            const int e = r * kTeams + t;
-            round_off[t] = e < found ? __builtin_amdgcn_readfirstlane(sm.offs[e]) : -1;
+        for (int w = 0; w < kWaves; w++) found += __builtin_amdgcn_readfirstlane(sm.count[0][w]);
+        if (found <= kList) break;
+        hi = lo + (hi - lo) / 2;   // (found > kList >= kStrips, so the range holds at least two tiles)
+      }
+      {
+        int at = 0;
+#pragma unroll
+        for (int w = 0; w < kWaves; w++) at += (w < wave) ? __builtin_amdgcn_readfirstlane(sm.count[0][w]) : 0;
+        const int begin = lo + wave * chunk, end = begin + chunk < hi ? begin + chunk : hi;
+        for (int id0 = begin; id0 < end; id0 += 64 * kBatch) {
+          int offv[kBatch];
+#pragma unroll
+          for (int u = 0; u < kBatch; u++) {
+            const int id = id0 + u * 64 + lane;
+            offv[u] = id < end ? p.offsets[id] : 0;
           }
 #pragma unroll
-          for (int t = 0; t < kTeams; t++)
+          for (int u = 0; u < kBatch; u++) {
+            const int id = id0 + u * 64 + lane;
+            unsigned long long mask[kStrips];
+            const int n = strips_of(id < end ? id : -1, offv[u], mask);
+            // the strips of the lanes below me, then my own in order
+            int mine = at;
 #pragma unroll
-            for (int u = t + 1; u < kTeams; u++) {
-              const int d = round_off[t] - round_off[u];
-              overlap |= round_off[t] >= 0 && round_off[u] >= 0 && d < TBK * TBN && d > -TBK * TBN;
+            for (int s = 0; s < kStrips; s++) mine += __popcll(mask[s] & ((1ull << lane) - 1ull));
+#pragma unroll
+            for (int s = 0; s < kStrips; s++) {
+              if ((mask[s] >> lane) & 1ull) {
+                sm.list[mine] = id * kStrips + s;
+                sm.offs[mine] = offv[u] + s * kStripElems;
+                sm.done[mine] = 0;
+                mine++;
+              }
             }
-        }
-        if (!overlap) {
-          if (have) add_to_window(tile_off);
-          __syncthreads();
-        } else {
-          for (int turn = 0; turn < kTeams; turn++) {
-            if (turn == team && have) add_to_window(tile_off);
-            __syncthreads();
+            at += n;
           }
         }
-        entry += kTeams;
       }
+      lo = hi;
+      __syncthreads();   // list complete, flags cleared
+
+      // ---- every wavefront works through list entries wave, wave + kWaves, ... on its own ----
+      // An item is one group of rows of M of one tile.  No barrier in here: a wavefront that
+      // waits for an earlier tile's flag must never be waited for by the owner of that tile.
+      const int my_tiles = found > wave ? (found - wave + kWaves - 1) / kWaves : 0;
+      const int items = my_tiles * ngroups;
+      int ft = 0, fg = 0;      // tile ordinal and group of the next item to load
+      auto fetch_next = [&](auto set) {
+        constexpr int S = decltype(set)::value;
+        if (ft < my_tiles) {
+          const int v = __builtin_amdgcn_readfirstlane(sm.list[wave + ft * kWaves]);
+          const int id = v / kStrips, strip = v % kStrips;
+          const int tk = id / p.tiles_n, tn = id - tk * p.tiles_n;
+          const int k0 = tk * TBK + strip * 32;              // the strip's first row of W
+          const int m0 = fg * kGroupRows;
+          const bool whole = m0 + kGroupRows <= p.M;
+          // (a strip that begins beyond K contributes nothing; its base is kept inside the matrix)
+          const T* rows_x = gX + (int64_t)m0 * p.ldx + (int64_t)(k0 < p.K ? k0 : p.K - 1);
+          const T* rows_y = gdY + (int64_t)m0 * p.lddy + (int64_t)tn * TBN;
+          if constexpr (STAGED) {
+            {
+              // X: lane -> row lane / 4, piece lane % 4; dY: rows lane / 8 and + 8, piece lane % 8.
+              // A piece outside the matrix is fetched from inside it and replaced by zero later.
+              {
+                const int r = lane >> 2, c = (lane & 3) * 8;
+                const bool ok = m0 + r < p.M && k0 + c < p.K;
+                const T* src = ok ? gX + (int64_t)(m0 + r) * p.ldx + (k0 + c) : gX + (int64_t)m0 * p.ldx;
+                __builtin_memcpy(&px[S], src, 16);
+                okx[S] = ok;
+              }
+#pragma unroll
+              for (int q = 0; q < 2; q++) {
+                const int r = (lane >> 3) + 8 * q, c = (lane & 7) * 8;
+                const bool ok = m0 + r < p.M && tn * TBN + c < p.N;
+                const T* src = ok ? rows_y + (int64_t)r * p.lddy + c : gdY + (int64_t)m0 * p.lddy;
+                __builtin_memcpy(&py[S][q], src, 16);
+                oky[S][q] = ok;
+              }
+              if (++fg == ngroups) {
+                fg = 0;
+                ft++;
+              }
+              return;
+            }
+          }
+#pragma unroll
+          for (int a = 0; a < BI; a++) {
+            const int col = a * 32 + (lane & 31);
+            const bool ok = k0 + col < p.K;
+#pragma unroll
+            for (int s = 0; s < GS; s++)
+              fa[S][s][a] = load_frag(rows_x, p.ldx, s * KS, m0, p.M, lane, ok ? col : 0, ok, whole);
+          }
+#pragma unroll
+          for (int b = 0; b < BJ; b++) {
+            const int col = b * 32 + (lane & 31);
+            const bool ok = tn * TBN + col < p.N;
+#pragma unroll
+            for (int s = 0; s < GS; s++)
+              fb[S][s][b] = load_frag(rows_y, p.lddy, s * KS, m0, p.M, lane, ok ? col : 0, ok, whole);
+          }
+          if (++fg == ngroups) {
+            fg = 0;
+            ft++;
+          }
+        }
+      };
+      // add the finished strip of list entry `e` into the window, after the earlier strips whose
+      // slices meet its own, and raise its flag
+      auto add_tile = [&](int e) {
+        const int tile_off = __builtin_amdgcn_readfirstlane(sm.offs[e]);
+        // lane l looks at the earlier entries l, l + 64, ...: straight-line LDS reads, no branches
+        for (;;) {
+          bool pending = false;
+          for (int f = lane; f < e; f += 64) {
+            const int d = sm.offs[f] - tile_off;
+            const int dn = __hip_atomic_load(&sm.done[f], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            pending |= (d < kStripElems) & (d > -kStripElems) & (dn == 0);
+          }
+          if (!__any(pending)) break;
+          __builtin_amdgcn_s_sleep(1);
+        }
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+        const int rel = (int)((long long)tile_off - w0);   // (offsets and window starts are below 2^31)
+        if (rel >= 0 && rel + kStripElems <= wlen) {
+          // the whole strip lies inside the window (the usual case): no checks, constant offsets
+#pragma unroll
+          for (int b = 0; b < BJ; b++) {
+            float* at = win + rel + ((lane >> 5) * 4) * TBN + b * 32 + (lane & 31);
+#pragma unroll
+            for (int half = 0; half < 2; half++) {
+              float cur[8];
+#pragma unroll
+              for (int q = 0; q < 8; q++) {
+                const int i = half * 8 + q;
+                cur[q] = at[((i >> 2) * 8 + (i & 3)) * TBN];
+              }
+#pragma unroll
+              for (int q = 0; q < 8; q++) {
+                const int i = half * 8 + q;
+                at[((i >> 2) * 8 + (i & 3)) * TBN] = cur[q] + acc[0][b][i] * p.scale;
+                acc[0][b][i] = 0.f;
+              }
+            }
+          }
+        } else {
+          // elements outside the window go to a dump slot behind it: no branches, so the reads
+          // and the writes of a block go out back to back (the addresses of a lane are distinct;
+          // the dump slots are shared between wavefronts, their contents are never used)
+          const int dump = p.window + lane;
+#pragma unroll
+          for (int b = 0; b < BJ; b++) {
+            const int base = rel + ((lane >> 5) * 4) * TBN + b * 32 + (lane & 31);
+            // (eight elements at a time: 16 wavefronts per compute unit leave few registers)
+#pragma unroll
+            for (int half = 0; half < 2; half++) {
+              int at[8];
+              float cur[8];
+#pragma unroll
+              for (int q = 0; q < 8; q++) {
+                const int i = half * 8 + q;
+                const int x = base + ((i >> 2) * 8 + (i & 3)) * TBN;
+                at[q] = (x >= 0 && x < wlen) ? x : dump;
+                cur[q] = win[at[q]];
+              }
+#pragma unroll
+              for (int q = 0; q < 8; q++) {
+                const int i = half * 8 + q;
+                win[at[q]] = cur[q] + acc[0][b][i] * p.scale;
+                acc[0][b][i] = 0.f;
+              }
+            }
+          }
+        }
+        if (lane == 0) __hip_atomic_store(&sm.done[e], 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+      };
+      int pt = 0, pg = 0;      // tile ordinal and group of the item being multiplied
+      auto item = [&](auto set) {
+        constexpr int S = decltype(set)::value;
+        fetch_next(std::integral_constant<int, S ^ 1>{});   // the next item's loads fly meanwhile
+        if constexpr (STAGED) {
+          {
+            // pieces -> this wavefront's staging area (LDS operations of one wavefront are carried
+            // out in order, so neither the reads below nor the next group's writes need a barrier)
+            T* st = sm.stage[wave];
+            const u32x4_t z = {0u, 0u, 0u, 0u};
+            *reinterpret_cast<u32x4_t*>(st + (lane >> 2) * 32 + (lane & 3) * 8) = okx[S] ? px[S] : z;
+#pragma unroll
+            for (int q = 0; q < 2; q++) {
+              const int r = (lane >> 3) + 8 * q, pc = lane & 7;
+              // dY rows are two 64-byte chunks, swapped in every other pair of rows, so that the four
+              // rows of a transpose read fall on different banks
+              *reinterpret_cast<u32x4_t*>(st + kStageX + r * TBN + ((((pc >> 2) ^ ((r >> 1) & 1)) << 5) | ((pc & 3) << 3))) =
+                  oky[S][q] ? py[S][q] : z;
+            }
+            // fragments by the LDS transpose read: within 16 lanes, lane c receives column c of a
+            // 4 x 16 block whose rows the lanes address four-per-row
+            typedef s16x4_t __attribute__((address_space(3))) * lds_s16x4_ptr;
+            const int g = lane >> 4, jl = lane & 15;
+            const int row = 8 * (g >> 1) + (jl >> 2), col = 16 * (g & 1) + 4 * (jl & 3);
+            auto tr_frag = [&](const T* at, int pitch) -> Frag {
+              const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(at));
+              const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(at + 4 * pitch));
+              const u32x2_t l2 = __builtin_bit_cast(u32x2_t, lo), h2 = __builtin_bit_cast(u32x2_t, hi);
+              u32x4_t f = {l2[0], l2[1], h2[0], h2[1]};
+              return f;
+            };
+            const Frag a = tr_frag(st + row * 32 + col, 32);
+            Frag b[BJ];
+#pragma unroll
+            for (int j = 0; j < BJ; j++)
+              b[j] = tr_frag(st + kStageX + row * TBN + (((j ^ ((row >> 1) & 1)) << 5) | col), TBN);
+#pragma unroll
+            for (int j = 0; j < BJ; j++) acc[0][j] = Mfma<T>::run(a, b[j], acc[0][j]);
+            if (++pg == ngroups) {
+              add_tile(wave + pt * kWaves);
+              pg = 0;
+              pt++;
+            }
+            return;
+          }
+        }
+#pragma unroll
+        for (int s = 0; s < GS; s++)
+#pragma unroll
+          for (int a = 0; a < BI; a++)
+#pragma unroll
+            for (int b = 0; b < BJ; b++) acc[a][b] = Mfma<T>::run(fa[S][s][a], fb[S][s][b], acc[a][b]);
+        if (++pg == ngroups) {
+          add_tile(wave + pt * kWaves);
+          pg = 0;
+          pt++;
+        }
+      };
+      fetch_next(std::integral_constant<int, 0>{});
+      for (int i = 0; i < items; i += 2) {
+        item(std::integral_constant<int, 0>{});
+        if (i + 1 < items) item(std::integral_constant<int, 1>{});
+      }
+      __syncthreads();   // every strip of the list has been added
     }
-    __syncthreads();
 
     // store the window: dHW[w0 + i] (+)= image[i], each element exactly once
     if (p.out_f32 || sizeof(T) == 4) {
@@ -273,14 +443,14 @@ struct WindowKernel {
     } else {
       T* out = static_cast<T*>(p.dHW) + w0;
       for (int i = tid; i < wlen; i += kThreads)
-        out[i] = ElemTraits<T>::from_float(win[i] + (p.accumulate ? ElemTraits<T>::to_float(out[i]) : 0.f));
+        out[i] = Tr::from_float(win[i] + (p.accumulate ? Tr::to_float(out[i]) : 0.f));
     }
   }
 };
 
-template <typename T, int TBK, int TBN>
-__global__ __launch_bounds__((WindowKernel<T, TBK, TBN>::kThreads)) void rz_window_kernel(WindowParams p) {
-  typedef WindowKernel<T, TBK, TBN> K;
+template <typename T, int TBK, int TBN, bool STAGED>
+__global__ __launch_bounds__((WindowKernel<T, TBK, TBN, STAGED>::kThreads)) void rz_window_kernel(WindowParams p) {
+  typedef WindowKernel<T, TBK, TBN, STAGED> K;
   extern __shared__ __attribute__((aligned(16))) unsigned char rz_window_smem[];
   K::run(p, *reinterpret_cast<typename K::Smem*>(rz_window_smem));
 }

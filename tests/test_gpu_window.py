@@ -21,6 +21,9 @@ CASES = [
     (200, 512, 512, 300000, 64, 64),      # 256 windows of about 1.2 K elements
     (31, 640, 640, 2000001, 64, 64),      # most of dHW untouched, odd H
     (130, 192, 128, 7000000, 64, 64),     # two rounds of windows; M spans several chunks
+    (40, 520, 264, 500000, 64, 64),       # 16-byte pieces whole, last tile row has one strip beyond K
+    (17, 96, 72, 100000, 32, 64),         # one partial group of rows of M
+    (8, 4096, 8192, 40000, 64, 64),       # more strips meet a window than its list holds (16-bit)
 ]
 _dt_id = lambda d: str(d).split(".")[-1]
 _shape_id = lambda s: "x".join(map(str, s))
