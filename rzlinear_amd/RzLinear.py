@@ -46,6 +46,13 @@ class RzLinear(nn.Module):
         block_size_k, block_size_n: hashed tile, powers of two in [16, 256]; one tile for
             forward, input-grad and weight-grad, which is what makes the three see the same W.
             The defaults are the reference launchers' defaults.
+        fuse_grad_accumulation: backward adds this layer's weight gradient straight into the
+            parameter's gradient buffer (``hashed_weight.main_grad`` if the parameter carries such
+            a [H] tensor — float32 master gradients — else ``hashed_weight.grad``) inside the
+            weight-grad kernels, and hands autograd no weight gradient.  Layers that share one
+            hashed_weight (python/rz_linear/RzLinear.py:54-58) then cost no extra pass over H per
+            layer and no zero-fill.  Like every fused accumulation it bypasses gradient hooks on
+            the parameter and higher-order differentiation through it.
     """
 
     P = 45007   # prime of the hash
@@ -54,13 +61,15 @@ class RzLinear(nn.Module):
     def __init__(self, input_dim: int, output_dim: int, chunk_size: int = 1,
                  hashed_weight: nn.Parameter = None, tiled=True, seed: int = 1024, bias: bool = True,
                  dtype: torch.dtype = torch.float32, compress_ratio: float = 0.0625,
-                 init_factor: float = 1.0, block_size_k: int = 32, block_size_n: int = 64) -> None:
+                 init_factor: float = 1.0, block_size_k: int = 32, block_size_n: int = 64,
+                 fuse_grad_accumulation: bool = False) -> None:
         super().__init__()
         assert input_dim < _INT32_SAFE_DIM and output_dim < _INT32_SAFE_DIM
 
         # geometry and hashing
         self._input_dim, self._output_dim = input_dim, output_dim
         self._block_size_k, self._block_size_n = block_size_k, block_size_n
+        self._fuse_grad_accumulation = fuse_grad_accumulation
         self._chunk_size = chunk_size
         self._seed = seed
         self._random_numbers = self._generate_random_numbers(seed)   # plain attribute: stays on the CPU
@@ -93,5 +102,5 @@ class RzLinear(nn.Module):
         bias = self._bias if isinstance(self._bias, torch.Tensor) else None
         out = RzLinearFunction.apply(rows, self._hashed_weight, self._random_numbers, self._output_dim,
                                      self._chunk_size, self._init_factor, self._block_size_k,
-                                     self._block_size_n, bias)
+                                     self._block_size_n, bias, self._fuse_grad_accumulation)
         return out if x.dim() == 2 else out.view(*lead, out.shape[-1])

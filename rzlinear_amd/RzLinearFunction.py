@@ -39,16 +39,18 @@ class RzLinearFunction(torch.autograd.Function):
     """output = (input @ W_hashed) * init_factor (+ bias).
 
     forward(input[M, K], hashed_weight[H], random_numbers[8] (CPU), output_dim, chunk_size,
-            init_factor, block_size_k=None, block_size_n=None, bias=None) -> [M, output_dim]
+            init_factor, block_size_k=None, block_size_n=None, bias=None,
+            fuse_grad_accumulation=False) -> [M, output_dim]
 
     The first six arguments are the reference's; chunk_size is carried and unused, as there.
-    The optional ones select the hashed tile (default: ``controls``) and fuse the layer's bias
-    into the forward kernel.
+    The optional ones select the hashed tile (default: ``controls``), fuse the layer's bias into
+    the forward kernel, and make backward add the weight gradient into the parameter's own
+    gradient buffer instead of returning it (see RzLinear).
     """
 
     @staticmethod
     def forward(ctx, input, hashed_weight, random_numbers, output_dim, chunk_size, init_factor,
-                block_size_k=None, block_size_n=None, bias=None):
+                block_size_k=None, block_size_n=None, bias=None, fuse_grad_accumulation=False):
         consts = _hash_args(random_numbers)
         tile = (int(controls['block_size_k'] if block_size_k is None else block_size_k),
                 int(controls['block_size_n'] if block_size_n is None else block_size_n))
@@ -61,6 +63,7 @@ class RzLinearFunction(torch.autograd.Function):
         ctx.output_dim, ctx.chunk_size, ctx.init_factor = output_dim, chunk_size, init_factor
         ctx.tile = tile
         ctx.has_bias = bias is not None
+        ctx.fuse_grad_accumulation = bool(fuse_grad_accumulation)
         return output
 
     @staticmethod
@@ -80,7 +83,22 @@ class RzLinearFunction(torch.autograd.Function):
         if need_input:      # enqueued first, like the reference's rz_linear_backward_tl
             input_grad = rz_linear_backward_input_grad_tl(grad, hashed_weight.data, ctx.init_factor,
                                                           M, K, N, H, *consts, **kwargs)
-        if need_weight and need_bias:   # one pass over grad yields both
+        if need_weight and ctx.fuse_grad_accumulation:
+            # Add into the parameter's gradient buffer inside the kernels.  The first layer to
+            # reach a parameter without a gradient overwrites a fresh buffer (no zero-fill), the
+            # others accumulate; autograd gets no weight gradient and so adds nothing itself.
+            target = getattr(hashed_weight, 'main_grad', None)
+            accumulate = True
+            if target is None:
+                if hashed_weight.grad is None:
+                    hashed_weight.grad = torch.empty_like(hashed_weight)
+                    accumulate = False
+                target = hashed_weight.grad
+            launcher = rz_linear_backward_weight_bias_grad_tl if need_bias else rz_linear_backward_weight_grad_tl
+            result = launcher(input, grad, ctx.init_factor, M, K, N, H, *consts, out=target, accumulate=accumulate,
+                              **kwargs)
+            bias_grad = result[1] if need_bias else None
+        elif need_weight and need_bias:   # one pass over grad yields both
             weight_grad, bias_grad = rz_linear_backward_weight_bias_grad_tl(input, grad, ctx.init_factor,
                                                                             M, K, N, H, *consts, **kwargs)
         elif need_weight:
@@ -88,4 +106,4 @@ class RzLinearFunction(torch.autograd.Function):
                                                             M, K, N, H, *consts, **kwargs)
         elif need_bias:
             bias_grad = grad.sum(dim=0)
-        return input_grad, weight_grad, None, None, None, None, None, None, bias_grad
+        return input_grad, weight_grad, None, None, None, None, None, None, bias_grad, None

@@ -53,6 +53,10 @@ def weight_grad_hashed(input, output_grad, init_factor, M, K, N, H, R, BLOCK_SIZ
         if accumulate:
             flags |= _lib.WG_ACCUMULATE
     bias_grad = torch.empty((N,), device=output_grad.device, dtype=output_grad.dtype) if with_bias_grad else None
+    if M == 0:   # an empty batch contributes a zero gradient (the reference returns its zeros(H))
+        if not accumulate:
+            out.zero_()
+        return out, (bias_grad.zero_() if with_bias_grad else None)
     tuning = _lib.current_tuning()
     need = lib.rz_weight_grad_hashed_workspace_bytes(M, K, N, H, BLOCK_SIZE_K, BLOCK_SIZE_N, code, flags,
                                                      int(with_bias_grad), tuning)
@@ -129,6 +133,8 @@ def input_grad_hashed(output_grad, hashed_weight, init_factor, M, K, N, H, R, BK
     stream = _lib.require_gpu(output_grad, hashed_weight)
     if hashed_weight.dtype != output_grad.dtype:
         raise TypeError("output_grad is %s but hashed_weight is %s" % (output_grad.dtype, hashed_weight.dtype))
+    if M == 0:
+        return torch.empty((0, K), device=output_grad.device, dtype=output_grad.dtype)
     dy, lddy = _lib.rows(output_grad)
     hw = hashed_weight.contiguous()
     input_grad = torch.empty((M, K), device=output_grad.device, dtype=output_grad.dtype)

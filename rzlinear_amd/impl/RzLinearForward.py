@@ -51,6 +51,8 @@ def forward_hashed(input, hashed_weight, bias, init_factor, M, K, N, H, R, BK, B
         if bias.dtype != input.dtype or bias.numel() != N:
             raise TypeError("bias must be a [%d] tensor of %s" % (N, input.dtype))
         bias = bias.contiguous()
+    if M == 0:   # an empty batch: nothing to launch, as the reference returns its empty zeros((0, N))
+        return torch.empty((0, N), device=input.device, dtype=input.dtype)
     x, ldx = _lib.rows(input)
     hw = hashed_weight.contiguous()
     output = torch.empty((M, N), device=input.device, dtype=input.dtype)

@@ -258,6 +258,89 @@ def test_function_apply_with_the_reference_six_arguments(oracle):
     assert rel_err(x2.grad.cpu().numpy(), 2 * oracle.input_grad(dy64, hw64, K, BK, BN, R1024, 1.0)) <= 1e-4
 
 
+@pytest.mark.parametrize("master", [False, True], ids=["grad", "main_grad_fp32"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=lambda d: str(d).split(".")[-1])
+def test_layers_sharing_a_parameter_accumulate_inside_the_kernels(oracle, dtype, master):
+    """Three RzLinear layers over ONE hashed_weight (python/rz_linear/RzLinear.py:54-58) with
+    fuse_grad_accumulation: backward adds every layer's weight gradient into the parameter's
+    gradient buffer inside the weight-grad kernels (no tensor per layer, no add over H by
+    autograd).  Against the sum of the oracle's three gradients, and against the same network
+    without the option."""
+    import torch.nn as nn
+    from rzlinear_amd import RzLinear
+    dims = [(96, 160, 64, 64), (160, 128, 32, 64), (128, 72, 64, 32)]      # (K, N, BK, BN) per layer
+    H, M = 30000, 200
+    seeds = [3, 4, 5]
+    g = torch.Generator().manual_seed(99)
+    hw0 = ((torch.rand(H, generator=g) * 2 - 1) / 10).to(dtype)
+    x0 = torch.randn((M, dims[0][0]), generator=g).to(dtype)
+    dy0 = torch.randn((M, dims[-1][1]), generator=g).to(dtype)
+    _say("shared parameter", dtype, "main_grad" if master else "grad")
+
+    def run(fuse):
+        hw = nn.Parameter(hw0.clone().cuda())
+        if fuse and master:
+            hw.main_grad = torch.zeros(H, dtype=torch.float32, device="cuda")
+        layers = [RzLinear(K, N, hashed_weight=hw, seed=sd, bias=False, dtype=dtype, init_factor=0.5,
+                           block_size_k=BK, block_size_n=BN, fuse_grad_accumulation=fuse)
+                  for (K, N, BK, BN), sd in zip(dims, seeds)]
+        x = x0.clone().cuda().requires_grad_(True)
+        acts, h = [x], x
+        for layer in layers:
+            h = layer(h)
+            acts.append(h)
+        h.backward(dy0.cuda())
+        torch.cuda.synchronize()
+        grad = hw.main_grad if (fuse and master) else hw.grad
+        return layers, [a.detach() for a in acts], x.grad, grad
+
+    layers, acts, dx_fused, grad_fused = run(True)
+    _, _, dx_plain, grad_plain = run(False)
+    # oracle: chain the per-layer gradients through the recorded activations
+    hw64 = hw0.double().numpy()
+    up = dy0.double().numpy()
+    want = np.zeros(H)
+    for layer, (K, N, BK, BN), a in reversed(list(zip(layers, dims, acts[:-1]))):
+        R = layer._random_numbers.tolist()
+        want += oracle.weight_grad(a.double().cpu().numpy(), up, H, BK, BN, R, 0.5)
+        up = oracle.input_grad(up, hw64, K, BK, BN, R, 0.5)
+        up = torch.from_numpy(up).to(dtype).double().numpy()      # the kernels round dX to the layer dtype
+    tol = TOL[dtype] * 2                                          # three layers' rounding on the way down
+    assert grad_fused.dtype == (torch.float32 if master else dtype)
+    assert rel_err(grad_fused.float().cpu().numpy(), want) <= tol
+    assert rel_err(grad_plain.float().cpu().numpy(), want) <= tol
+    assert rel_err(grad_fused.float().cpu().numpy(), grad_plain.float().cpu().numpy().astype(np.float64)) <= tol
+    assert torch.equal(dx_fused, dx_plain)                        # the input gradient does not depend on the option
+    # a second backward keeps adding into the same buffer
+    before = grad_fused.clone()
+    h = acts[0].clone().requires_grad_(True)
+    out = h
+    for layer in layers:
+        out = layer(out)
+    out.backward(dy0.cuda())
+    torch.cuda.synchronize()
+    now = layers[0]._hashed_weight.main_grad if master else layers[0]._hashed_weight.grad
+    assert rel_err(now.float().cpu().numpy(), 2 * before.float().cpu().numpy().astype(np.float64)) <= tol
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=lambda d: str(d).split(".")[-1])
+def test_empty_batch(dtype):
+    """M = 0: the reference's launchers return an empty output / input gradient and a zero
+    weight gradient (torch.zeros((0, N)), torch.zeros(H)); so do these, without a launch."""
+    from rzlinear_amd import RzLinear
+    layer = RzLinear(64, 96, dtype=dtype, compress_ratio=0.5, block_size_k=32, block_size_n=32).cuda()
+    x = torch.zeros((0, 64), dtype=dtype, device="cuda", requires_grad=True)
+    y = layer(x)
+    assert y.shape == (0, 96) and y.dtype == dtype
+    y.sum().backward()
+    torch.cuda.synchronize()
+    assert x.grad.shape == (0, 64)
+    assert layer._hashed_weight.grad.shape == layer._hashed_weight.shape
+    assert float(layer._hashed_weight.grad.abs().max()) == 0.0 and float(layer._bias.grad.abs().max()) == 0.0
+    y3 = layer(torch.zeros((2, 0, 64), dtype=dtype, device="cuda"))
+    assert y3.shape == (2, 0, 96)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=lambda d: str(d).split(".")[-1])
 @pytest.mark.parametrize("shape", [(32, 2048, 1024, 70000, 32, 64), (100, 4096, 300, 20000, 64, 64),
                                    (7, 2100, 520, 9000, 16, 32)], ids=lambda s: "x".join(map(str, s)))

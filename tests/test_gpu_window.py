@@ -84,6 +84,25 @@ def test_windowed_accumulate_and_fp32_buffer(oracle, tuned, dtype):
         assert rel_err(buf.float().cpu().numpy(), ref) <= TOL[dtype]
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16], ids=_dt_id)
+def test_bias_gradient_beside_the_window_kernel(oracle, tuned, dtype):
+    """A layer with a bias asks for dbias in the same call; the window kernel does not stage dY by
+    tile columns, so the column sums come from a pass of their own and the window path is kept."""
+    from rzlinear_amd import _lib
+    from rzlinear_amd.impl.RzLinearBackward import rz_linear_backward_weight_bias_grad_tl
+    tuned(window=1)
+    M, K, N, H, BK, BN = 45, 384, 520, 200000, 64, 64
+    code = _lib.dtype_code(torch.empty(0, dtype=dtype))
+    assert _lib.plan_query(2, M, K, N, H, BK, BN, code, 0, True)["mode"] == "window"
+    _say("window + dbias", dtype)
+    (x, _, dy), (x64, _, dy64) = make_inputs(M, K, N, H, dtype, seed=35)
+    dhw, dbias = rz_linear_backward_weight_bias_grad_tl(x, dy, 0.5, M, K, N, H, *rargs(R1024), BLOCK_SIZE_K=BK,
+                                                        BLOCK_SIZE_N=BN)
+    torch.cuda.synchronize()
+    assert rel_err(dhw.float().cpu().numpy(), oracle.weight_grad(x64, dy64, H, BK, BN, R1024, 0.5)) <= TOL[dtype]
+    assert rel_err(dbias.float().cpu().numpy(), dy64.sum(axis=0)) <= TOL[dtype]
+
+
 def test_library_picks_the_window_path_for_skinny_batches(oracle):
     """M = 32 against K = N = 4096 with a 2^20-element hashed_weight: no tuning override."""
     from rzlinear_amd.impl.RzLinearBackward import rz_linear_backward_weight_grad_tl
