@@ -79,7 +79,8 @@ typedef struct rz_tuning {
   int window;     /* weight-grad: 0 = automatic, 1 = dHW by windows whenever possible, -1 = never */
   int split;      /* forward / input-grad: 0 = automatic, -1 = never split the contraction */
   int clamp;      /* ragged 16-bit shapes: 0 = automatic, -1 = always the bounds-checked kernels */
-  int resident;   /* forward / input-grad: 0 = automatic, -1 = never keep hashed_weight in LDS */
+  int fold;       /* weight-grad with a hashed_weight too large for LDS: 0 = automatic, 1 = X^T.dY stored
+                     tile by tile and folded into dHW by a second kernel whenever possible, -1 = never */
   int reserved;   /* must be 0 */
 } rz_tuning;
 
@@ -258,8 +259,9 @@ int rz_weight_grad_hashed(const void* X, const void* dY, void* dHW, void* dbias,
  * Fills out[8] = { C-tile edge, slices, contracted elements per slice, contracted elements per
  * kernel step, mode, workgroups, 0, 0 } with mode 0 = plain store, 1 = split contraction with
  * fp32 partial planes, 2 = weight-grad through LDS images of dHW, 3 = weight-grad by global
- * atomics, 4 = weight-grad by windows of dHW, 5 = weight-grad through LDS images of segments of
- * dHW.  For tests of the planning logic and for tuning; no counterpart in the reference.
+ * atomics, 4 = weight-grad by windows of dHW, 5 = weight-grad stored tile by tile and folded
+ * into dHW by a second kernel.  For tests of the planning logic and for tuning; no counterpart in the
+ * reference.
  */
 int rz_plan_query(int op, int M, int K, int N, int H, int BK, int BN, int dtype, unsigned flags,
                   int with_dbias, const rz_tuning* tuning, int32_t out[8]);

@@ -31,7 +31,7 @@ class Tuning(ctypes.Structure):
     automatic).  Only tests and benchmarks set any of it."""
     _fields_ = [("tile", ctypes.c_int), ("stages", ctypes.c_int), ("lds_image", ctypes.c_int),
                 ("window", ctypes.c_int), ("split", ctypes.c_int), ("clamp", ctypes.c_int),
-                ("resident", ctypes.c_int), ("reserved", ctypes.c_int)]
+                ("fold", ctypes.c_int), ("reserved", ctypes.c_int)]
 
 
 # What the launchers of this package pass as `tuning` (None = automatic).  The C library keeps no
@@ -206,7 +206,7 @@ def tile_offsets(K, N, H, BLOCK_SIZE_K, BLOCK_SIZE_N, random_numbers, hash_level
     return out
 
 
-PLAN_MODES = {0: "store", 1: "split", 2: "lds_image", 3: "atomics", 4: "window", 5: "segment_images"}
+PLAN_MODES = {0: "store", 1: "split", 2: "lds_image", 3: "atomics", 4: "window", 5: "fold"}
 
 
 def plan_query(op, M, K, N, H, BK, BN, dtype_code_, flags=0, with_dbias=False):

@@ -6,6 +6,7 @@
 #include <atomic>
 
 #include "rz_common.h"
+#include "rz_fold.h"
 #include "rz_launch.h"
 #include "rz_window.h"
 
@@ -281,6 +282,32 @@ static void launch_reduce_partials(int out_dtype, const float* part, void* out, 
     hipLaunchKernelGGL((reduce_partials_kernel<f16_t, ACC>), grid, block, 0, s, part, (f16_t*)out, H, pitch, nparts);
 }
 
+// Enqueues the fold kernel for tiles of `loads` * 1024 elements (smaller tiles: loads = 1).
+static hipError_t launch_fold(const FoldParams& fp, int loads, hipStream_t s) {
+  static std::atomic<uint64_t> raised[5];
+  const size_t lds = fold_lds_bytes(fp.window);
+  if ((fp.partial == nullptr && (fp.shares != 1 || fp.out == nullptr)) || fp.window <= 0 || fp.window % kFoldThreads != 0 || fp.window > kFoldWindowMax || fp.slices > kFoldList ||
+      (long long)fp.windows * fp.window < fp.H)
+    return hipErrorInvalidValue;
+  const dim3 grid((unsigned)(fp.windows * fp.shares)), block(kFoldThreads);
+  auto go = [&](auto kernel, int slot) -> hipError_t {
+    if (lds > 64 * 1024) {
+      hipError_t e = raise_lds_limit(reinterpret_cast<const void*>(kernel), raised[slot]);
+      if (e != hipSuccess) return e;
+    }
+    hipLaunchKernelGGL(kernel, grid, block, lds, s, fp);
+    return hipGetLastError();
+  };
+  switch (loads) {
+    case 1: return go(fold_tiles_kernel<1>, 0);
+    case 2: return go(fold_tiles_kernel<2>, 1);
+    case 4: return go(fold_tiles_kernel<4>, 2);
+    case 8: return go(fold_tiles_kernel<8>, 3);
+    case 16: return go(fold_tiles_kernel<16>, 4);
+    default: return hipErrorInvalidValue;
+  }
+}
+
 template <bool ACC>
 static void launch_convert(int out_dtype, const float* src, void* dst, int n, hipStream_t s) {
   const dim3 grid((n + 255) / 256), block(256);
@@ -306,16 +333,16 @@ static void launch_reduce_colsum(int out_dtype, const float* part, void* out, in
 static inline size_t round256(size_t b) { return (b + 255) & ~(size_t)255; }
 
 // Workspace layout of a weight-grad call: [main][column sums].  main = the partial images (LDS
-// image mode), the table of tile offsets (window kernel) or, for the atomic scatter into a
-// 16-bit dHW, its fp32 image.
+// image mode), the tile-by-tile X^T.dY followed by the fold kernel's images, the table of tile
+// offsets (window kernel) or, for the atomic scatter into a 16-bit dHW, its fp32 image.
 struct WeightGradWorkspace {
   size_t main_bytes, total_bytes;
 };
 static WeightGradWorkspace weight_grad_workspace(const WeightGradPlan& plan, const WindowPlan& window, int H,
                                                  bool dhw_f32, bool with_dbias) {
   WeightGradWorkspace w;
-  if (plan.image_pitch > 0) w.main_bytes = plan.workspace_bytes;
-  else if (window.use) w.main_bytes = round256((size_t)window.tiles * sizeof(int32_t));  // tile offsets
+  if (window.use) w.main_bytes = round256((size_t)window.tiles * sizeof(int32_t));  // tile offsets
+  else if (plan.image_pitch > 0 || plan.fold.use) w.main_bytes = plan.workspace_bytes;
   else w.main_bytes = dhw_f32 ? 0 : round256((size_t)H * sizeof(float));
   // (the window kernel does not stage dY by tile columns: its bias gradient is a pass of its own)
   w.total_bytes = w.main_bytes + (with_dbias && !window.use ? plan.colsum_bytes : 0);
@@ -340,9 +367,9 @@ static int weight_grad_impl(const void* X, const void* dY, void* dHW, void* dbia
   const bool accumulate = (flags & RZ_WG_ACCUMULATE) != 0;
   const int dhw_dtype = (flags & RZ_WG_DHW_F32) ? RZ_F32 : dtype;
   const int dbias_dtype = (flags & RZ_WG_DBIAS_F32) ? RZ_F32 : dtype;
-  const WeightGradPlan plan = plan_weight_grad(M, K, N, H, dtype_bytes(dtype), tuning);
+  const WeightGradPlan plan = plan_weight_grad(M, K, N, H, BK, BN, dtype_bytes(dtype), tuning);
   WindowPlan wp = {};
-  if (plan.image_pitch == 0) wp = plan_window(M, K, N, H, BK, BN, dtype_bytes(dtype), tuning);
+  if (!plan.lds_image()) wp = plan_window(M, K, N, H, BK, BN, dtype_bytes(dtype), tuning, plan);
   const WeightGradWorkspace ws = weight_grad_workspace(plan, wp, H, dhw_dtype == RZ_F32, dbias != nullptr);
   if (ws.total_bytes > 0 && (workspace == nullptr || workspace_bytes < ws.total_bytes)) return RZ_ERR_WORKSPACE;
   hipStream_t s = (hipStream_t)stream;
@@ -355,7 +382,7 @@ static int weight_grad_impl(const void* X, const void* dY, void* dHW, void* dbia
   p.ldb = lddy;
   p.scale = init_factor;
   if (dbias != nullptr && !wp.use) p.colsum = reinterpret_cast<float*>(static_cast<char*>(workspace) + ws.main_bytes);
-  if (plan.image_pitch == 0 && wp.use) {
+  if (wp.use) {
     // large hashed_weight, short contraction: windows of dHW instead of K*N atomics.  The
     // tile offsets are hashed once into the workspace; every workgroup scans them.
     {
@@ -386,7 +413,42 @@ static int weight_grad_impl(const void* X, const void* dY, void* dHW, void* dbia
       return RZ_OK;
     }
   }
-  if (plan.image_pitch > 0) {
+  if (plan.fold.use) {
+    // no scatter in the contraction: X^T.dY goes to the workspace tile by tile, the fold kernel's
+    // workgroups each add up the tiles that land in their window of hashed_weight (per share of
+    // the tiles), and the shares' images are added up (no atomics, fixed summation order)
+    const FoldPlan& f = plan.fold;
+    p.scatter = nullptr;
+    p.tiles_out = (float*)workspace;
+    p.out_tiles_k = (K + BK - 1) / BK;
+    p.out_tiles_n = (N + BN - 1) / BN;
+    if (launch_gemm(dtype, kWeightGrad, p, &plan, nullptr, tuning, s) != hipSuccess) return RZ_ERR_LAUNCH;
+    FoldParams fp;
+    fp.tiles = p.tiles_out;
+    int32_t* offsets = (int32_t*)((char*)workspace + f.tiles_bytes + f.partial_bytes);
+    hipLaunchKernelGGL(tile_offsets_kernel, dim3((p.out_tiles_k * p.out_tiles_n + 255) / 256), dim3(256), 0, s, offsets,
+                       p.out_tiles_k, p.out_tiles_n, p.h);
+    if (hipGetLastError() != hipSuccess) return RZ_ERR_LAUNCH;
+    fp.offsets = offsets;
+    fp.partial = f.shares > 1 ? (float*)((char*)workspace + f.tiles_bytes) : nullptr;
+    fp.out = dHW;
+    fp.out_dtype = dhw_dtype;
+    fp.accumulate = accumulate ? 1 : 0;
+    fp.h = p.h;
+    fp.H = H;
+    fp.pitch = (H + 3) & ~3;
+    fp.tiles_k = p.out_tiles_k;
+    fp.tiles_n = p.out_tiles_n;
+    fp.slices = plan.splits;
+    fp.window = f.window;
+    fp.windows = f.windows;
+    fp.shares = f.shares;
+    if (launch_fold(fp, f.loads, s) != hipSuccess) return RZ_ERR_LAUNCH;
+    if (f.shares > 1) {
+      if (accumulate) launch_reduce_partials<true>(dhw_dtype, fp.partial, dHW, H, fp.pitch, f.shares, s);
+      else launch_reduce_partials<false>(dhw_dtype, fp.partial, dHW, H, fp.pitch, f.shares, s);
+    }
+  } else if (plan.image_pitch > 0) {
     // every workgroup sums its tiles into an LDS image of dHW and stores it as a partial image;
     // the partial images are then added up (no global atomics, fixed summation order)
     p.scatter = (float*)workspace;
@@ -640,10 +702,11 @@ RZ_API size_t rz_weight_grad_hashed_workspace_bytes(int M, int K, int N, int H, 
   const int eb = dtype_bytes(dtype);
   const rz_tuning t = tuning_or_default(tuning);
   if (eb == 0 || M < 1 || K < 1 || N < 1 || H < 1 || !tuning_valid(t)) return 0;
-  const WeightGradPlan plan = plan_weight_grad(M, K, N, H, eb, t);
+  if (check_tile(BK, BN) != RZ_OK) return 0;
+  const WeightGradPlan plan = plan_weight_grad(M, K, N, H, BK, BN, eb, t);
   const bool dhw_f32 = (flags & RZ_WG_DHW_F32) != 0 || dtype == RZ_F32;
   WindowPlan wp = {};
-  if (plan.image_pitch == 0 && check_tile(BK, BN) == RZ_OK) wp = plan_window(M, K, N, H, BK, BN, eb, t);
+  if (!plan.lds_image()) wp = plan_window(M, K, N, H, BK, BN, eb, t, plan);
   return weight_grad_workspace(plan, wp, H, dhw_f32, with_dbias != 0).total_bytes;
 }
 
@@ -697,16 +760,16 @@ RZ_API int rz_plan_query(int op, int M, int K, int N, int H, int BK, int BN, int
   if (st != RZ_OK) return st;
   for (int i = 0; i < 8; i++) out[i] = 0;
   if (op == kWeightGrad) {
-    const WeightGradPlan plan = plan_weight_grad(M, K, N, H, eb, t);
+    const WeightGradPlan plan = plan_weight_grad(M, K, N, H, BK, BN, eb, t);
     WindowPlan wp = {};
-    if (plan.image_pitch == 0) wp = plan_window(M, K, N, H, BK, BN, eb, t);
+    if (!plan.lds_image()) wp = plan_window(M, K, N, H, BK, BN, eb, t, plan);
     if (wp.use) {
       out[0] = 0; out[1] = 1; out[2] = M; out[3] = 32; out[4] = 4; out[5] = wp.windows;
       return RZ_OK;
     }
     const KernelForm f = kernel_form(op, K, N, M, plan.r_chunk, plan.tile, plan.workgroups, eb, t);
     out[0] = plan.tile; out[1] = plan.splits; out[2] = plan.r_chunk; out[3] = f.step;
-    out[4] = plan.image_pitch > 0 ? 2 : 3;
+    out[4] = plan.fold.use ? 5 : plan.image_pitch > 0 ? 2 : 3;
     out[5] = (int32_t)plan.workgroups;
     return RZ_OK;
   }

@@ -104,6 +104,11 @@ struct GemmParams {
   float* scatter;     // weight-grad target: fp32 image of dHW (direct atomics), or the
                       // per-workgroup partial images [workgroups][image_pitch] (LDS mode)
   int image_pitch;    // > 0 selects the LDS mode: floats per partial image (H rounded up to 4)
+  float* tiles_out;   // weight-grad, non-null: no scatter at all; the C tile (scaled X^T.dY) is stored
+                      // hashed tile by hashed tile, tile (tk, tn) of slice s as BK*BN contiguous floats
+                      // at ((s * tiles_k + tk) * tiles_n + tn) * BK*BN (zeros beyond K x N), and a
+                      // second kernel folds the tiles into dHW
+  int out_tiles_k, out_tiles_n;   // ... its tile grid: ceil(K / BK) x ceil(N / BN)
   float* colsum;      // weight-grad that also yields the bias gradient: partial column sums of B
                       // (dY), one row per (slice, tile row): [slices * tiles_i][colsum_pitch]
   int colsum_pitch;   // floats per row of colsum (J rounded up to the tile)

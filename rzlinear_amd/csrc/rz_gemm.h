@@ -177,8 +177,7 @@ struct GemmKernel {
   static constexpr int kOffSlots = 32;    // two banks of kOffBank steps
   static constexpr int kOffBank = 16;
   static constexpr int kOffWindow = (TR / 16) * (TJ / 16);
-  static constexpr int kOffEntries =
-      (OP == kWeightGrad) ? (TI / 16) * (TJ / 16) : kOffSlots * kOffWindow;
+  static constexpr int kOffEntries = (OP == kWeightGrad) ? (TI / 16) * (TJ / 16) : kOffSlots * kOffWindow;
 
   struct Smem {
     alignas(16) T a[NSTAGE][LA::kElems];
@@ -264,8 +263,13 @@ struct GemmKernel {
     return v;
   }
 
-  static __device__ void run(const GemmParams& p, Smem& sm) {
-    const int tid = threadIdx.x;
+  static __device__ __forceinline__ void run(const GemmParams& p, Smem& sm) {
+    run_item(p, sm, threadIdx.x, blockIdx.x, blockIdx.y, gridDim.x);
+  }
+
+  // One C tile (workgroup id `bx` of `gx`, as the hardware deals them to the XCDs) and slice `by`
+  // of the contracted dimension.
+  static __device__ __forceinline__ void run_item(const GemmParams& p, Smem& sm, const int tid, int bx, int by, int gx) {
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // (uniform: lives in a scalar register)
     const int wave_i = wave / WJ, wave_j = wave % WJ;
@@ -279,9 +283,9 @@ struct GemmKernel {
     // Workgroup ids are dealt round-robin to the 8 XCDs; renumber so that each XCD (one L2)
     // gets a contiguous run of tiles, then walk tiles with J fastest (forward/input-grad
     // share the streamed A panel) or in square-ish groups (weight-grad streams both).
-    int id = blockIdx.x;
+    int id = bx;
     {
-      const int nwg = gridDim.x, per = nwg >> 3, rem = nwg & 7, x = id & 7, q = id >> 3;
+      const int nwg = gx, per = nwg >> 3, rem = nwg & 7, x = id & 7, q = id >> 3;
       id = x * per + (x < rem ? x : rem) + q;
     }
     int ti, tj;
@@ -297,7 +301,7 @@ struct GemmKernel {
       tj = id % p.tiles_j;
     }
     const int i0 = ti * TI, j0 = tj * TJ;
-    const int r_begin = blockIdx.y * p.r_chunk;
+    const int r_begin = by * p.r_chunk;
     const int r_end = (r_begin + p.r_chunk) < p.R ? (r_begin + p.r_chunk) : p.R;
     const int steps = (r_end - r_begin + TR - 1) / TR;
 
@@ -593,6 +597,13 @@ struct GemmKernel {
         }
       }
     }
+    // a uniform pointer, said to be one (two scalar registers): the base operand of the loads above
+    auto uniform_ptr = [&](const T* ptr) -> const T* {
+      const uint64_t v = (uint64_t)(uintptr_t)ptr;
+      const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
+      const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+      return (const T*)(uintptr_t)(((uint64_t)hi << 32) | lo);
+    };
     // all tiles of R step `step` -> LDS stage `st`
     auto direct_issue = [&](int step, int st) {
       const int r0 = r_begin + step * TR;
@@ -600,23 +611,24 @@ struct GemmKernel {
         direct_issue_plain_slow(step, st);
       } else {
         // first element of the A tile of this step (uniform)
-        const T* a_base = (A_LAYOUT == kRContig) ? gA + (int64_t)i0 * p.lda + r0 : gA + (int64_t)r0 * p.lda + i0;
+        const T* a_base = uniform_ptr((A_LAYOUT == kRContig) ? gA + (int64_t)i0 * p.lda + r0 : gA + (int64_t)r0 * p.lda + i0);
 #pragma unroll
         for (int q = 0; q < LA::kPieces; q++) direct_load_so(a_base, a_voff[q], sm.a[st], q, LA::kPieces);
         if constexpr (OP == kWeightGrad) {
-          const T* b_base = gB + (int64_t)r0 * p.ldb + j0;
+          const T* b_base = uniform_ptr(gB + (int64_t)r0 * p.ldb + j0);
 #pragma unroll
           for (int q = 0; q < LB::kPieces; q++) direct_load_so(b_base, b_voff[q], sm.b[st], q, LB::kPieces);
         }
       }
       if constexpr (OP != kWeightGrad) {
         const int* tab = sm.off + (step & (kOffSlots - 1)) * kOffWindow;
+        const T* hw_base = uniform_ptr(gHW);
         uint32_t off[LB::kPieces];
 #pragma unroll
         for (int q = 0; q < LB::kPieces; q++) off[q] = (uint32_t)tab[b_tab[q]];   // all lookups first, then the loads
 #pragma unroll
         for (int q = 0; q < LB::kPieces; q++)
-          direct_load_so(gHW, off[q] * (uint32_t)sizeof(T) + b_voff[q], sm.b[st], q, LB::kPieces);
+          direct_load_so(hw_base, off[q] * (uint32_t)sizeof(T) + b_voff[q], sm.b[st], q, LB::kPieces);
       }
     };
     // CLAMP, last R step with fewer than TR elements of R: once every wavefront's loads of that
@@ -833,7 +845,7 @@ struct GemmKernel {
         for (int c = tid; c < TJ; c += kThreads) {
           float s = 0.f;
           for (int g = 0; g < kGroups; g++) s += image[g * TJ + c];
-          p.colsum[((size_t)blockIdx.y * p.tiles_i + ti) * (size_t)p.colsum_pitch + j0 + c] = s;
+          p.colsum[((size_t)by * p.tiles_i + ti) * (size_t)p.colsum_pitch + j0 + c] = s;
         }
         __syncthreads();
       }
@@ -845,9 +857,41 @@ struct GemmKernel {
       // than the operand stages), else in its usual place
       int* etab = image_mode ? reinterpret_cast<int*>(image + p.image_pitch) : sm.off;
       const OffWindow w = off_window(p.h, i0, TI, j0, TJ);
-      for (int t = tid; t < w.count; t += kThreads)
-        etab[t] = (int)tile_offset(p.h, (uint32_t)(w.tk0 + t / w.ntn), (uint32_t)(w.tn0 + t % w.ntn));
+      const bool tiled = p.tiles_out != nullptr;
+      for (int t = tid; t < w.count; t += kThreads) {
+        const int tk = w.tk0 + t / w.ntn, tn = w.tn0 + t % w.ntn;
+        if (tiled)   // where the tile starts in the tile-by-tile output (-1: the C tile reaches beyond the grid)
+          etab[t] = (tk < p.out_tiles_k && tn < p.out_tiles_n)
+                        ? ((by * p.out_tiles_k + tk) * p.out_tiles_n + tn) << (p.h.bk_shift + p.h.bn_shift)
+                        : -1;
+        else
+          etab[t] = (int)tile_offset(p.h, (uint32_t)tk, (uint32_t)tn);
+      }
       __syncthreads();
+      // No scatter: the accumulators are stored plainly, hashed tile by hashed tile (whole tiles:
+      // zeros where a tile reaches beyond K x N); the fold kernel adds the tiles into dHW.
+      auto store_tiles = [&]() {
+#pragma unroll
+        for (int a = 0; a < MI; a++)
+#pragma unroll
+          for (int b = 0; b < MJ; b++) {
+            const int n = j0 + blk_j(b) + (lane & 31);
+            int base[4];
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+              const int k = i0 + blk_i(a) + g * 8 + (lane >> 5) * 4;
+              const int start = etab[((k >> p.h.bk_shift) - w.tk0) * w.ntn + ((n >> p.h.bn_shift) - w.tn0)];
+              base[g] = start < 0 ? -1 : start + (k & (p.h.BK - 1)) * p.h.BN + (n & (p.h.BN - 1));
+            }
+#pragma unroll
+            for (int e = 0; e < 16; e++) {
+              const int k = i0 + blk_i(a) + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
+              const bool inside = FULL || (k < p.I && n < p.J);
+              if (FULL || base[e >> 2] >= 0)
+                p.tiles_out[(uint32_t)(base[e >> 2] + (e & 3) * p.h.BN)] = inside ? acc[a][b][e] * p.scale : 0.f;
+            }
+          }
+      };
       // Scatter-add of the accumulators.  The four rows e&3 of a row group (e>>2) are adjacent
       // rows of one hashed tile (tiles are at least 16 rows), so one table lookup per row
       // group gives all four addresses; the lookups of a 32x32 block are issued together and
@@ -876,7 +920,9 @@ struct GemmKernel {
             }
           }
       };
-      if (image_mode) {
+      if (tiled) {
+        store_tiles();
+      } else if (image_mode) {
         // Tiles of one workgroup overlap in hashed_weight: sum them in an LDS image of dHW
         // first, then store the image as this workgroup's partial result.
         if (p.h.bk_shift >= 5 && p.h.bn_shift >= 5) {
@@ -923,7 +969,7 @@ struct GemmKernel {
           scatter(image);
           __syncthreads();
         }
-        float* dst = p.scatter + ((size_t)blockIdx.y * gridDim.x + blockIdx.x) * (size_t)p.image_pitch;
+        float* dst = p.scatter + ((size_t)by * gx + bx) * (size_t)p.image_pitch;
         for (int i = tid * 4; i < p.image_pitch; i += kThreads * 4)
           *reinterpret_cast<float4*>(dst + i) = *reinterpret_cast<const float4*>(image + i);
       } else {
@@ -931,9 +977,9 @@ struct GemmKernel {
       }
     } else {
       if (p.partial != nullptr) {
-        // R is split over blockIdx.y (few C tiles, long R): this slice's scaled fp32 partial
+        // R is split over the slices `by` (few C tiles, long R): this slice's scaled fp32 partial
         // result goes to its own [I][J] plane; a second kernel adds the planes up
-        float* __restrict__ gP = p.partial + (size_t)blockIdx.y * (size_t)p.I * (size_t)p.J;
+        float* __restrict__ gP = p.partial + (size_t)by * (size_t)p.I * (size_t)p.J;
 #pragma unroll
         for (int a = 0; a < MI; a++) {
 #pragma unroll

@@ -9,19 +9,6 @@
 
 namespace rz {
 
-// Kernels that use more than the default 64 KB of LDS need their limit raised once per kernel
-// and device; `done` is that kernel's bit set of devices already served.
-static inline hipError_t raise_lds_limit(const void* kernel, std::atomic<uint64_t>& done) {
-  int dev = 0;
-  hipError_t e = hipGetDevice(&dev);
-  if (e != hipSuccess) return e;
-  const uint64_t bit = 1ull << (dev & 63);
-  if (done.load(std::memory_order_acquire) & bit) return hipSuccess;
-  e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-  if (e == hipSuccess) done.fetch_or(bit, std::memory_order_release);
-  return e;
-}
-
 template <typename T, int OP, int TI, int TJ, int WI, int WJ, int NSTAGE, bool FULL, bool COLSUM, bool CLAMP = false>
 static hipError_t launch_one(GemmParams p, const WeightGradPlan* plan, const SplitPlan* split,
                              hipStream_t stream) {
@@ -39,6 +26,10 @@ static hipError_t launch_one(GemmParams p, const WeightGradPlan* plan, const Spl
     p.r_chunk = plan->r_chunk;
     p.image_pitch = plan->image_pitch;
     if ((size_t)p.image_pitch * sizeof(float) > kMaxImageBytes) return hipErrorInvalidValue;
+    // exactly one target: the tile-by-tile output, or an image (LDS mode: partial images) to scatter into
+    if (plan->fold.use != (p.tiles_out != nullptr) || (p.tiles_out == nullptr) == (p.scatter == nullptr))
+      return hipErrorInvalidValue;
+    if (plan->fold.use && p.image_pitch > 0) return hipErrorInvalidValue;
     if (COLSUM) {
       if (p.colsum == nullptr || plan->colsum_pitch != p.tiles_j * TJ ||
           plan->colsum_rows != plan->splits * p.tiles_i)
@@ -123,7 +114,7 @@ static hipError_t launch_gemm_t(int op, GemmParams p, const WeightGradPlan* plan
   const bool cut = !wg && split != nullptr && split->splits > 1;
   const int tile = wg ? plan->tile : (split != nullptr ? split->tile : pick_tile(p.I, p.J, (int)sizeof(T), tuning));
   const int chunk = wg ? plan->r_chunk : (cut ? split->r_chunk : p.R);
-  const long long workgroups = tile_count(p.I, p.J, tile) * (wg ? plan->splits : 1);
+  const long long workgroups = wg ? plan->workgroups : tile_count(p.I, p.J, tile);
   const KernelForm form = kernel_form(op, p.I, p.J, p.R, chunk, tile, workgroups, (int)sizeof(T), tuning);
   switch (form.tile * 100 + form.waves * 10 + form.stages) {
     case 25682: return launch_op<T, 256, 2, 4, 2>(op, p, plan, split, form, stream);

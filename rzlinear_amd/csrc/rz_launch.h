@@ -1,6 +1,8 @@
 // Host-side launch of the contraction kernels; one translation unit per element type.
 #pragma once
 
+#include <atomic>
+
 #include "../../include/rzlinear.h"
 #include "rz_common.h"
 
@@ -17,7 +19,20 @@ static inline bool tuning_valid(const rz_tuning& t) {
   return (t.tile == 0 || t.tile == 64 || t.tile == 128 || t.tile == 256) && (t.stages == 0 || t.stages == 1) &&
          (t.lds_image == 0 || t.lds_image == -1) && (t.window >= -1 && t.window <= 1) &&
          (t.split == 0 || t.split == -1) && (t.clamp == 0 || t.clamp == -1) &&
-         (t.resident == 0 || t.resident == -1) && t.reserved == 0;
+         (t.fold >= -1 && t.fold <= 1) && t.reserved == 0;
+}
+
+// Kernels that use more than the default 64 KB of LDS need their limit raised once per kernel
+// and device; `done` is that kernel's bit set of devices already served.
+static inline hipError_t raise_lds_limit(const void* kernel, std::atomic<uint64_t>& done) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  const uint64_t bit = 1ull << (dev & 63);
+  if (done.load(std::memory_order_acquire) & bit) return hipSuccess;
+  e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+  if (e == hipSuccess) done.fetch_or(bit, std::memory_order_release);
+  return e;
 }
 
 static constexpr int kComputeUnits = 256;
@@ -79,6 +94,45 @@ static inline int pick_tile(int I, int J, int elem_bytes, const rz_tuning& tunin
   return best;
 }
 
+// Weight-grad without any scatter in the contraction kernel: X^T.dY is stored tile by tile and a
+// second kernel, whose workgroups own windows of hashed_weight, folds the tiles into dHW.
+struct FoldPlan {
+  int use;
+  int window, windows;   // floats per window (a multiple of 1024, at most 32768) and their number
+  int shares;            // workgroups per window, each with an equal part of the window's tiles and an image of its own
+  int loads;             // per list entry and thread: BK*BN / 1024, at least 1
+  size_t tiles_bytes;    // the tile-by-tile X^T.dY: slices * tiles * BK*BN floats
+  size_t partial_bytes;  // shares images of dHW (none with a single share: the fold kernel writes dHW)
+  size_t offsets_bytes;  // where every tile starts in hashed_weight, one int32 per tile
+};
+
+static inline FoldPlan plan_fold(int K, int N, int H, int BK, int BN, int slices) {
+  FoldPlan f = {};
+  const long long E = (long long)BK * BN;
+  const long long tiles = (long long)((K + BK - 1) / BK) * ((N + BN - 1) / BN);
+  // (element indices of the buffer are 32-bit in the kernels; the fold lists slices entries per tile)
+  if (E > 16384 || slices > 64 || (long long)slices * tiles * E >= (1LL << 31)) return f;
+  const int kWindowMax = 32768, kThreads = 1024;
+  f.windows = (H + kWindowMax - 1) / kWindowMax;
+  // from half a window per compute unit on, the windows are cut so that whole rounds of workgroups
+  // come out, and every workgroup writes its window of dHW itself (no shares, no images)
+  if (f.windows * 2 >= kComputeUnits) f.windows = (f.windows + kComputeUnits - 1) / kComputeUnits * kComputeUnits;
+  f.window = (((H + f.windows - 1) / f.windows) + kThreads - 1) / kThreads * kThreads;
+  f.windows = (H + f.window - 1) / f.window;
+  // (a workgroup fills a compute unit: no more workgroups than compute units, or two would wait for a second round)
+  long long shares = f.windows * 2 >= kComputeUnits ? 1 : kComputeUnits / f.windows;
+  if (shares > slices * tiles / 8) shares = slices * tiles / 8;   // a share is worth a workgroup from some tiles on
+  if (shares < 1) shares = 1;
+  f.shares = (int)shares;
+  f.loads = E >= 1024 ? (int)(E / 1024) : 1;
+  f.tiles_bytes = ((size_t)slices * tiles * E * sizeof(float) + 255) & ~(size_t)255;
+  const size_t pitch = (size_t)((H + 3) & ~3);
+  f.partial_bytes = f.shares > 1 ? ((size_t)f.shares * pitch * sizeof(float) + 255) & ~(size_t)255 : 0;
+  f.offsets_bytes = ((size_t)tiles * sizeof(int32_t) + 255) & ~(size_t)255;
+  f.use = 1;
+  return f;
+}
+
 // How the weight-grad contraction C[K,N] = X^T.dY over M is cut into workgroups, and how the
 // finished tiles reach dHW.
 struct WeightGradPlan {
@@ -89,11 +143,14 @@ struct WeightGradPlan {
   int image_pitch;   // > 0: every workgroup first sums its tiles into an fp32 image of dHW held
                      // in LDS and stores it as one partial image; a second kernel adds the
                      // partial images up.  0: tiles go to dHW by global atomics.
+  FoldPlan fold;        // fold.use: no scatter in the contraction kernel at all (tile-by-tile output)
+  double fold_us;       // ... and roughly how long the whole weight-grad then takes, in microseconds
   size_t workspace_bytes;   // partial images, or the fp32 image for the atomics (16-bit dHW)
   // bias gradient computed in the same pass: partial column sums of dY, one row per
   // (slice, tile row), stored behind the first `workspace_bytes` of the workspace
   int colsum_rows, colsum_pitch;
   size_t colsum_bytes;
+  bool lds_image() const { return image_pitch > 0; }
 };
 
 // LDS bytes of a compute unit that an fp32 image of dHW may take (the rest holds the small
@@ -104,7 +161,8 @@ static inline long long tile_cover(int K, int N, int t) {
   return (long long)((K + t - 1) / t) * ((N + t - 1) / t) * t * t;
 }
 
-static inline WeightGradPlan plan_weight_grad(int M, int K, int N, int H, int elem_bytes, const rz_tuning& t) {
+static inline WeightGradPlan plan_weight_grad(int M, int K, int N, int H, int BK, int BN, int elem_bytes,
+                                              const rz_tuning& t) {
   WeightGradPlan pl;
   const int pitch = (H + 3) & ~3;
   const bool image = t.lds_image != -1 && (size_t)pitch * sizeof(float) <= kMaxImageBytes;
@@ -141,8 +199,33 @@ static inline WeightGradPlan plan_weight_grad(int M, int K, int N, int H, int el
   pl.r_chunk = steps_per * TR;
   pl.workgroups = tiles * pl.splits;
   pl.image_pitch = image ? pitch : 0;
+  pl.fold = FoldPlan{};
+  pl.fold_us = 0.0;
+  if (!image && t.fold != -1) {
+    const FoldPlan f = plan_fold(K, N, H, BK, BN, pl.splits);
+    if (f.use) {
+      // what the two ways cost beyond the contraction itself, in microseconds: the part of the
+      // K*N global atomics per slice that the contraction does not hide (about 2.8 ps each,
+      // measured), against reading the tiles back (their stores overlap the contraction, unless
+      // it is shorter than they are), writing and reading the images, and two more launches
+      const double elems = (double)pl.splits * (double)K * (double)N;
+      const double product_us = 2.0 * (double)M * K * N / (elem_bytes == 4 ? 110e6 : 900e6);
+      const double store_us = elems * 4.0 / 4.0e6;
+      const double atomics_us = elems * 2.8e-6;
+      // (a workgroup of the fold kernel reads some 15 GB/s: few workgroups cannot use the memory system)
+      const double read_bytes = elems * 4.0 * (1.0 + (double)BK * BN / f.window);
+      const double all_us = (read_bytes + 2.0 * (double)f.partial_bytes) / 4.5e6;
+      const double one_us = read_bytes / ((double)f.windows * f.shares) / 15e3;
+      const double fold_us = (store_us > product_us ? store_us - product_us : 0.0) + (all_us > one_us ? all_us : one_us) + 10.0;
+      if (t.fold == 1 || fold_us < atomics_us) {
+        pl.fold = f;
+        pl.fold_us = product_us + fold_us;
+      }
+    }
+  }
   size_t ws = 0;
-  if (pl.image_pitch > 0) ws = (size_t)pl.workgroups * pl.image_pitch * sizeof(float);
+  if (pl.fold.use) ws = pl.fold.tiles_bytes + pl.fold.partial_bytes + pl.fold.offsets_bytes;
+  else if (pl.image_pitch > 0) ws = (size_t)pl.workgroups * pl.image_pitch * sizeof(float);
   else if (elem_bytes == 2) ws = (size_t)H * sizeof(float);   // fp32 image for the atomics
   pl.workspace_bytes = (ws + 255) & ~(size_t)255;
   pl.colsum_rows = pl.splits * ((K + pl.tile - 1) / pl.tile);
@@ -164,7 +247,8 @@ static constexpr int kWindowFloats = 25600;   // LDS floats a workgroup can hold
 
 static inline bool window_tile_supported(int BK, int BN) { return BN == 64 && (BK == 64 || BK == 32); }
 
-static inline WindowPlan plan_window(int M, int K, int N, int H, int BK, int BN, int elem_bytes, const rz_tuning& t) {
+static inline WindowPlan plan_window(int M, int K, int N, int H, int BK, int BN, int elem_bytes, const rz_tuning& t,
+                                     const WeightGradPlan& other) {
   WindowPlan pl = {false, 0, 0, 0};
   if (t.window == -1 || !window_tile_supported(BK, BN)) return pl;
   const long long tiles = (long long)((K + BK - 1) / BK) * ((N + BN - 1) / BN);
@@ -186,8 +270,10 @@ static inline WindowPlan plan_window(int M, int K, int N, int H, int BK, int BN,
   const double per_wg = (double)tiles * ((double)w + (double)BK * BN) / (double)H;
   const double wg_rounds = (double)((pl.windows + kComputeUnits - 1) / kComputeUnits);
   const double t_window = wg_rounds * per_wg * (elem_bytes == 4 ? 0.7 + 1.0 * chunks : 0.32 + 0.23 * chunks) + 28.0;
+  // ... against what the contraction kernel's plan would take: the fold, or the atomic scatter
   const double t_scatter = 0.9 * (double)K * N / 184e3 + 2.0 * M * (double)K * N / 800e6;
-  pl.use = t.window == 1 || t_window * 1.2 < t_scatter;
+  const double t_other = other.fold.use ? other.fold_us : t_scatter;
+  pl.use = t.window == 1 || t_window * 1.1 < t_other;
   return pl;
 }
 

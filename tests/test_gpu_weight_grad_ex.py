@@ -118,3 +118,59 @@ def test_ex_argument_checks():
     with pytest.raises(TypeError):
         rz_linear_backward_weight_grad_tl(x, dy, 1.0, M, K, N, H, *rargs(R1024), BLOCK_SIZE_K=64,
                                           BLOCK_SIZE_N=64, out=torch.zeros((H,), device="cuda", dtype=torch.float16))
+
+
+FOLD_CASES = [
+    # (M, K, N, H, BK, BN, forced C tile)
+    (40, 4096, 8192, 200000, 64, 64, 256),     # seven windows of hashed_weight, 36 shares of the 8192 tiles
+    (48, 4096, 4096, 70000, 64, 64, 128),
+    (64, 2048, 4096, 70000, 32, 64, 0),        # the reference's default hashed tile: two loads per tile and thread
+    (300, 200, 330, 90000, 32, 64, 128),       # ragged in M, K and N: whole tiles are stored, zeros beyond K x N
+    (520, 264, 328, 90000, 64, 32, 256),       # the C tile reaches beyond the grid of hashed tiles
+    (2100, 512, 384, 50000, 128, 64, 128),     # M cut into slices: a list entry per (tile, slice); eight loads
+    (200, 256, 512, 40000, 16, 64, 64),        # 16-row hashed tiles, 64 C tile
+    (130, 300, 200, 37000, 16, 16, 0),         # tiles smaller than the workgroup: 256 of 1024 threads have an element
+    (96, 512, 768, 60000, 128, 128, 256),      # sixteen loads per tile and thread
+    (70, 1024, 1024, 1 << 20, 32, 32, 0),      # 32 windows; one load per tile and thread
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16], ids=_dt_id)
+@pytest.mark.parametrize("shape", FOLD_CASES, ids=_shape_id)
+def test_tiles_stored_plainly_and_folded_into_the_gradient(oracle, tuned, shape, dtype):
+    """hashed_weight too large for an LDS image: the contraction kernel stores X^T.dY tile by tile
+    and scatters nothing; the fold kernel's workgroups own windows of hashed_weight and add up the
+    tiles that land there.  No atomics, a fixed order of additions: the same bits on every call.
+    With the bias gradient, and accumulating into an existing buffer."""
+    from rzlinear_amd import _lib
+    from rzlinear_amd.impl.RzLinearBackward import (rz_linear_backward_weight_bias_grad_tl,
+                                                    rz_linear_backward_weight_grad_tl)
+    M, K, N, H, BK, BN, tile = shape
+    tuned(fold=1, window=-1, tile=tile)
+    code = _lib.dtype_code(torch.empty(0, dtype=dtype))
+    plan = _lib.plan_query(2, M, K, N, H, BK, BN, code)
+    _say("fold", shape, dtype, plan)
+    assert plan["mode"] == "fold", plan
+    (x, _, dy), (x64, _, dy64) = make_inputs(M, K, N, H, dtype, seed=67)
+    kw = dict(BLOCK_SIZE_K=BK, BLOCK_SIZE_N=BN)
+    ref = oracle.weight_grad(x64, dy64, H, BK, BN, R1024, 0.5)
+    a = rz_linear_backward_weight_grad_tl(x, dy, 0.5, M, K, N, H, *rargs(R1024), **kw)
+    b, dbias = rz_linear_backward_weight_bias_grad_tl(x, dy, 0.5, M, K, N, H, *rargs(R1024), **kw)
+    torch.cuda.synchronize()
+    f = lambda t: t.float().cpu().numpy()
+    assert rel_err(f(a), ref) <= TOL[dtype]
+    assert (f(a)[ref == 0] == 0).all()                 # slots that no tile covers are exactly zero
+    assert rel_err(f(dbias), dy64.sum(axis=0)) <= TOL[dtype]
+    assert torch.equal(a, b)
+    assert torch.equal(a, rz_linear_backward_weight_grad_tl(x, dy, 0.5, M, K, N, H, *rargs(R1024), **kw))
+    start = torch.linspace(-1, 1, H).cuda()
+    buf = start.clone()
+    rz_linear_backward_weight_grad_tl(x, dy, 0.5, M, K, N, H, *rargs(R1024), out=buf, accumulate=True, **kw)
+    torch.cuda.synchronize()
+    assert rel_err(buf.cpu().numpy(), start.double().cpu().numpy() + ref) <= TOL[dtype]
+    # and the atomic scatter agrees
+    tuned(fold=-1, window=-1, tile=tile)
+    assert _lib.plan_query(2, M, K, N, H, BK, BN, code)["mode"] == "atomics"
+    c = rz_linear_backward_weight_grad_tl(x, dy, 0.5, M, K, N, H, *rargs(R1024), **kw)
+    torch.cuda.synchronize()
+    assert rel_err(f(c), ref) <= TOL[dtype]
