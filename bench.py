@@ -62,11 +62,26 @@ PEAK = {"bf16": 2500.0, "fp16": 2500.0, "fp32": 157.3}
 # figures are read off the committed summary named here; they describe the kernels of that
 # summary and are dropped (null) for a workload that has none.
 TRAFFIC = {
+    # HBM bytes per launch of the contraction kernel of each leg: FETCH_SIZE * 2.0 + WRITE_SIZE * 1.0 KiB
+    # (factors from the copy calibration in the same profile)
     ("square4096", "bf16"): {
         "profile": "profiles/rz_gemm_bf16_square4096.txt",
-        "bytes": {"forward": int((16672.7 * 2.0 + 32768.0) * 1024),       # algorithmic: 64.03 MiB
-                  "input_grad": int((16672.7 * 2.0 + 32768.0) * 1024),
-                  "weight_grad": int((98457.7 * 2.0 + 16785.8) * 1024)},  # X, dY re-read by 3 XCD groups; + partial images
+        "bytes": {"forward": int((16682.2 * 2.0 + 32768.0) * 1024),       # algorithmic: 64.03 MiB
+                  "input_grad": int((16684.0 * 2.0 + 32768.0) * 1024),
+                  "weight_grad": int((98463.2 * 2.0 + 16784.5) * 1024)},  # X, dY re-read by the XCDs' tile groups; + partial images
+    },
+    ("square4096", "fp32"): {
+        "profile": "profiles/rz_gemm_fp32_square4096.txt",
+        "bytes": {"forward": int((34692.2 * 2.0 + 68352.0) * 1024),       # algorithmic: 128.06 MiB
+                  "input_grad": int((33275.6 * 2.0 + 65536.0) * 1024),
+                  "weight_grad": int((196817.3 * 2.0 + 16784.0) * 1024)},
+    },
+    ("ffn", "bf16"): {
+        "profile": "profiles/rz_gemm_fold_bf16_ffn.txt",
+        "bytes": {"forward": int((71090.8 * 2.0 + 262144.0) * 1024),      # algorithmic: 320.1 MiB
+                  "input_grad": int((132349.0 * 2.0 + 65536.0) * 1024),
+                  # contraction (X, dY re-read by the XCDs' tile groups; X^T.dY written tile by tile: 256 MiB)
+                  "weight_grad": int((786642.5 * 2.0 + 262144.0) * 1024)},
     },
 }
 

@@ -299,7 +299,9 @@ static inline SplitPlan plan_split(int I, int J, int R, int elem_bytes, const rz
   const int min_steps = ((tiles * 2 < kComputeUnits) ? 8 : 16) / ((elem_bytes == 4 ? 2 : 1) * (TR * elem_bytes / 128));
   if (want > r_steps / min_steps) want = r_steps / min_steps;
   if (want > 16) want = 16;
-  if (tiles * 2 >= (long long)kComputeUnits * slots || want < 2 || t.split == -1)
+  // (measured, fp32 1024^3: with a workgroup on every compute unit already, cutting the
+  //  contraction in four plus the pass that adds the slices takes longer than not cutting it)
+  if (tiles >= kComputeUnits || want < 2 || t.split == -1)
     want = 1;
   const int steps_per = (int)((r_steps + want - 1) / want);
   pl.splits = (r_steps + steps_per - 1) / steps_per;
