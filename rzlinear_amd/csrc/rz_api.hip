@@ -245,6 +245,7 @@ static hipError_t reduce_slices_dtype(int dtype, const float* part, void* C, con
 static int run_plain_op(int op, int dtype, GemmParams p, const void* bias, void* workspace,
                         size_t workspace_bytes, bool may_split, const rz_tuning& tuning, hipStream_t s) {
   if (may_split) {
+    // tile and slices are chosen together
     const SplitPlan sp = plan_split(p.I, p.J, p.R, dtype_bytes(dtype), tuning);
     if (sp.splits > 1) {
       if (workspace == nullptr || workspace_bytes < sp.workspace_bytes) return RZ_ERR_WORKSPACE;
@@ -254,6 +255,8 @@ static int run_plain_op(int op, int dtype, GemmParams p, const void* bias, void*
       return reduce_slices_dtype(dtype, p.partial, p.C, bias, p.I, p.J, p.ldc, sp.splits, s) == hipSuccess
                  ? RZ_OK : RZ_ERR_LAUNCH;
     }
+    p.bias = bias;
+    return launch_gemm(dtype, op, p, nullptr, &sp, tuning, s) == hipSuccess ? RZ_OK : RZ_ERR_LAUNCH;
   }
   p.bias = bias;
   return launch_gemm(dtype, op, p, nullptr, nullptr, tuning, s) == hipSuccess ? RZ_OK : RZ_ERR_LAUNCH;
@@ -778,7 +781,7 @@ RZ_API int rz_plan_query(int op, int M, int K, int N, int H, int BK, int BN, int
   const SplitPlan sp = plan_split(I, J, R, eb, t);
   const bool cut = sp.splits > 1;
   const int chunk = cut ? sp.r_chunk : R;
-  const KernelForm f = kernel_form(op, I, J, R, chunk, sp.tile, tile_count(I, J, sp.tile), eb, t);
+  const KernelForm f = kernel_form(op, I, J, R, chunk, sp.tile, tile_count(I, J, sp.tile) * sp.splits, eb, t);
   out[0] = sp.tile; out[1] = sp.splits; out[2] = chunk; out[3] = f.step; out[4] = cut ? 1 : 0;
   out[5] = (int32_t)(tile_count(I, J, sp.tile) * sp.splits);
   return RZ_OK;

@@ -114,7 +114,7 @@ static hipError_t launch_gemm_t(int op, GemmParams p, const WeightGradPlan* plan
   const bool cut = !wg && split != nullptr && split->splits > 1;
   const int tile = wg ? plan->tile : (split != nullptr ? split->tile : pick_tile(p.I, p.J, (int)sizeof(T), tuning));
   const int chunk = wg ? plan->r_chunk : (cut ? split->r_chunk : p.R);
-  const long long workgroups = wg ? plan->workgroups : tile_count(p.I, p.J, tile);
+  const long long workgroups = wg ? plan->workgroups : tile_count(p.I, p.J, tile) * (cut ? split->splits : 1);
   const KernelForm form = kernel_form(op, p.I, p.J, p.R, chunk, tile, workgroups, (int)sizeof(T), tuning);
   switch (form.tile * 100 + form.waves * 10 + form.stages) {
     case 25682: return launch_op<T, 256, 2, 4, 2>(op, p, plan, split, form, stream);

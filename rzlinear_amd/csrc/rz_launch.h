@@ -286,28 +286,58 @@ struct SplitPlan {
   size_t workspace_bytes;
 };
 
+// Relative throughput of `wgs` workgroups of tile t (see tile_score_full, which this restates for
+// a workgroup count that includes the slices of a cut contraction).
+static inline double tile_rate(double wgs, int t, int elem_bytes) {
+  const double per_cu = wgs / kComputeUnits;
+  const bool f32 = elem_bytes == 4;
+  const int slots = (t == 256) ? 1 : (t == 128 ? 2 : 4);
+  const double lo = (t == 256) ? 1.0 : (t == 128 ? (f32 ? 0.86 : 0.51) : (f32 ? 0.60 : 0.16));
+  const double hi = (t == 256) ? 1.0 : (t == 128 ? (f32 ? 0.90 : 0.75) : (f32 ? 0.80 : 0.33));
+  if (per_cu <= 1.0) return lo * per_cu;
+  const double cap = (double)kComputeUnits * slots;
+  const double rounds = (double)((long long)((wgs + cap - 1) / cap));
+  const double util = wgs / (rounds * cap);
+  const double fill = per_cu >= slots ? 1.0 : (per_cu - 1.0) / (slots - 1.0);
+  const double e = lo + (hi - lo) * fill;
+  return per_cu >= slots ? e * util : e;
+}
+
+// Tile and number of slices together: the pair with the least estimated time.  A slice pays the
+// fill and drain of its pipeline (about three steps), the cut pays the fp32 partial planes
+// (written, read back) and the launch of the kernel that adds them.
 static inline SplitPlan plan_split(int I, int J, int R, int elem_bytes, const rz_tuning& t) {
-  SplitPlan pl;
-  pl.tile = pick_tile(I, J, elem_bytes, t);
-  const int TR = slice_unit(pl.tile, elem_bytes);
-  const long long tiles = tile_count(I, J, pl.tile);
-  const int r_steps = (R + TR - 1) / TR;
-  const int slots = (pl.tile == 256) ? 1 : (pl.tile == 128 ? 2 : 4);
-  long long want = ((long long)kComputeUnits * slots + tiles - 1) / tiles;   // fill every CU slot
-  // a slice should run at least 16 steps (8 when most compute units would otherwise sit idle);
-  // an fp32 step is several times longer than a 16-bit one, so half as many will do
-  const int min_steps = ((tiles * 2 < kComputeUnits) ? 8 : 16) / ((elem_bytes == 4 ? 2 : 1) * (TR * elem_bytes / 128));
-  if (want > r_steps / min_steps) want = r_steps / min_steps;
-  if (want > 16) want = 16;
-  // (measured, fp32 1024^3: with a workgroup on every compute unit already, cutting the
-  //  contraction in four plus the pass that adds the slices takes longer than not cutting it)
-  if (tiles >= kComputeUnits || want < 2 || t.split == -1)
-    want = 1;
-  const int steps_per = (int)((r_steps + want - 1) / want);
-  pl.splits = (r_steps + steps_per - 1) / steps_per;
-  pl.r_chunk = steps_per * TR;
-  pl.workspace_bytes = pl.splits > 1 ? (size_t)pl.splits * (size_t)I * (size_t)J * sizeof(float) : 0;
-  return pl;
+  SplitPlan best = {};
+  double best_us = 0.0;
+  const double peak = elem_bytes == 4 ? 137e6 : 1150e6;   // flop per microsecond of the 256 tile on a full chip
+  const int tiles_of[3] = {256, 128, 64};
+  for (int tile : tiles_of) {
+    if (t.tile && tile != t.tile) continue;
+    const int TR = slice_unit(tile, elem_bytes);
+    const long long tiles = tile_count(I, J, tile);
+    const int r_steps = (R + TR - 1) / TR;
+    const double useful = (double)I * (double)J / ((double)tiles * tile * tile);
+    for (int want = 1; want <= 16; want++) {
+      if (want > 1 && t.split == -1) break;
+      const int steps_per = (r_steps + want - 1) / want;
+      const int slices = (r_steps + steps_per - 1) / steps_per;
+      if (slices != want) continue;                           // (the same cut as a smaller `want`)
+      if (slices > 1 && steps_per * (TR * elem_bytes / 128) < 4) break;   // slices of a few steps are all fill and drain
+      const double steps = (double)steps_per * (TR * elem_bytes / 128);
+      const double rate = peak * tile_rate((double)tiles * slices, tile, elem_bytes) * useful * steps / (steps + 2.0);
+      double us = 2.0 * (double)I * (double)J * (double)R / rate + 4.0;
+      if (slices > 1) us += (2.0 * slices * (double)I * J * 4.0 + (double)I * J * elem_bytes) / 4.0e6 + 4.0;
+      // (near ties go to the larger tile and the fewer slices, which come first)
+      if (best.tile == 0 || us < best_us * 0.97) {
+        best.tile = tile;
+        best.splits = slices;
+        best.r_chunk = steps_per * TR;
+        best_us = us;
+      }
+    }
+  }
+  best.workspace_bytes = best.splits > 1 ? (size_t)best.splits * (size_t)I * (size_t)J * sizeof(float) : 0;
+  return best;
 }
 
 // Which instantiation of the contraction kernel runs a launch: C tile, wavefronts, LDS stages,
