@@ -158,10 +158,13 @@ int rz_input_grad_ws(const void* dY, const void* HW, void* dX, void* workspace,
  * Bytes of device workspace rz_weight_grad needs for this problem (0 when none).
  * When hashed_weight is small enough for an fp32 image of dHW to fit the LDS of a compute
  * unit, every workgroup stores one partial image ([workgroups][H rounded up to 4] floats) that
- * a second kernel adds up; otherwise the 16-bit types need an fp32 image of dHW (H floats)
- * for the atomic adds and fp32 needs nothing — unless M is small against K*N, when dHW is
- * computed in windows (no atomics) and the workspace holds one int32 offset per W tile.
- * The size depends on M: ask again when the batch size changes.
+ * a second kernel adds up.  Otherwise one of three: with many W tiles per element of dHW the
+ * contraction stores X^T.dY tile by tile (4 * ceil(K/BK)*BK * ceil(N/BN)*BN bytes per slice of M)
+ * and a second kernel folds the tiles into dHW (plus a few images of dHW and one int32 offset
+ * per W tile); with M small against K*N, dHW is computed in windows and the workspace holds
+ * only the offsets; with few tiles the 16-bit types need an fp32 image of dHW (H floats) for
+ * atomic adds and fp32 needs nothing.  The size depends on M: ask again when the batch size
+ * changes.
  */
 size_t rz_weight_grad_workspace_bytes(int M, int K, int N, int H, int BK, int BN, int dtype);
 
@@ -170,9 +173,11 @@ size_t rz_weight_grad_workspace_bytes(int M, int K, int N, int H, int BK, int BN
  * off(tk,tn); dHW is zeroed and fully overwritten by the call (element type `dtype`).
  * Replaces rz_linear_backward_weight_grad_tl                          impl/RzLinearBackward.py:23-97
  * (kernel rz_linear_backward_weight_grad_core                         impl/RzLinearBackward.py:291-371).
- * Accumulation and the scatter are done in fp32 for every dtype.  With the LDS-image path
- * the only unordered sums are the LDS adds inside one workgroup; with global atomics the
- * summation order across tiles is not fixed, as in the reference.
+ * Accumulation and the scatter are done in fp32 for every dtype.  The LDS-image, fold and
+ * window paths add in a fixed order (plain read-add-write in LDS, ordered by barriers, by list
+ * order or by flags; partial images are added in index order): the same inputs give the same
+ * bits on every call.  Only the global-atomic path (few W tiles and a hashed_weight too large
+ * for LDS) leaves the summation order across tiles open, as the reference does.
  */
 int rz_weight_grad(const void* X, const void* dY, void* dHW, void* workspace,
                    size_t workspace_bytes, int M, int K, int N, int H, int BK, int BN,
