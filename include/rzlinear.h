@@ -190,9 +190,10 @@ int rz_weight_grad(const void* X, const void* dY, void* dHW, void* workspace,
  * a 32 MiB device array that is part of the library (every GPU that loads the library holds its
  * own copy until the process ends).  No counterpart in the reference; it is for callers that
  * cannot allocate: code under HIP graph capture, tight serving loops, harnesses that forbid
- * hipMalloc.  Same arguments, results and status codes as rz_weight_grad otherwise; a problem
- * whose rz_weight_grad_workspace_bytes exceeds 32 MiB is refused with RZ_ERR_SCRATCH_LIMIT (at
- * M = N = K = 4096, H = 16778 the need is 17 MB).  The first call on a device looks the array's
+ * hipMalloc.  Same arguments, results and status codes as rz_weight_grad otherwise.  A problem
+ * for which rz_weight_grad would store X^T.dY tile by tile in more than 32 MiB takes the scatter
+ * kernel with global atomics instead; a problem that needs more than 32 MiB even so is refused
+ * with RZ_ERR_SCRATCH_LIMIT (at M = N = K = 4096, H = 16778 the need is 17 MB).  The first call on a device looks the array's
  * address up (make that call outside a graph capture).  All calls on one GPU share the one array:
  * calls that overlap in time on the same GPU — different streams, or different host threads —
  * race on it and must be serialised by the caller; calls on one stream are ordered and safe.

@@ -689,15 +689,22 @@ RZ_API int rz_weight_grad(const void* X, const void* dY, void* dHW, void* worksp
 RZ_API int rz_weight_grad_static(const void* X, const void* dY, void* dHW, int M, int K, int N, int H, int BK,
                                  int BN, const int32_t R[8], float init_factor, int64_t ldx, int64_t lddy,
                                  int dtype, void* stream) {
-  // the same plan, kernels and checks as rz_weight_grad; only the workspace differs
-  if (dtype_bytes(dtype) != 0 && M >= 1 && K >= 1 && N >= 1 && H >= 1 &&
-      rz_weight_grad_workspace_bytes(M, K, N, H, BK, BN, dtype) > kScratchBytes)
-    return RZ_ERR_SCRATCH_LIMIT;
+  // the same kernels and checks as rz_weight_grad; only the workspace differs.  The plan is the
+  // same too, except that the fold (whose tile-by-tile buffer takes 4*K*N bytes and more) gives
+  // way to the scatter kernel when it does not fit the scratch array.
+  rz_tuning tuning = {};
+  if (dtype_bytes(dtype) != 0 && M >= 1 && K >= 1 && N >= 1 && H >= 1) {
+    if (rz_weight_grad_hashed_workspace_bytes(M, K, N, H, BK, BN, dtype, 0u, 0, &tuning) > kScratchBytes) {
+      tuning.fold = -1;
+      if (rz_weight_grad_hashed_workspace_bytes(M, K, N, H, BK, BN, dtype, 0u, 0, &tuning) > kScratchBytes)
+        return RZ_ERR_SCRATCH_LIMIT;
+    }
+  }
   int st = RZ_OK;
   void* ws = scratch_of_current_device(&st);
   if (ws == nullptr) return st;
   return weight_grad_impl(X, dY, dHW, nullptr, ws, kScratchBytes, M, K, N, H, BK, BN, R, init_factor, ldx, lddy,
-                          dtype, 0u, stream);
+                          dtype, 0u, stream, RZ_HASH_TWO_LEVEL, &tuning);
 }
 
 RZ_API size_t rz_weight_grad_hashed_workspace_bytes(int M, int K, int N, int H, int BK, int BN, int dtype,

@@ -75,6 +75,25 @@ def test_static_scratch_matches_the_workspace_entry_point(oracle, pair, dtype):
         assert_close(f(b), ref, dtype, "dHW (workspace)")
 
 
+def test_static_scratch_gives_up_the_fold_when_its_buffer_does_not_fit(oracle):
+    """rz_weight_grad stores X^T.dY tile by tile for this problem (4*K*N bytes and more); the
+    static entry point cannot, and takes the scatter kernel instead of refusing."""
+    from rzlinear_amd import _lib
+    lib = _lib.load()
+    M, K, N, H, BK, BN = 40, 4096, 8192, 200000, 64, 64
+    assert _lib.plan_query(2, M, K, N, H, BK, BN, _lib.RZ_BF16)["mode"] == "fold"
+    assert lib.rz_weight_grad_workspace_bytes(M, K, N, H, BK, BN, _lib.RZ_BF16) > SCRATCH_BYTES
+    _say("static scratch, fold does not fit", (M, K, N, H))
+    (x, _, dy), (x64, _, dy64) = make_inputs(M, K, N, H, torch.bfloat16, seed=71)
+    R = (ctypes.c_int32 * 8)(*R1024)
+    a = torch.full((H,), float("nan"), dtype=torch.bfloat16, device="cuda")
+    _lib.check(lib.rz_weight_grad_static(x.data_ptr(), dy.data_ptr(), a.data_ptr(), M, K, N, H, BK, BN, R, 0.5,
+                                         K, N, _lib.RZ_BF16, torch.cuda.current_stream().cuda_stream))
+    torch.cuda.synchronize()
+    assert_close(a.float().cpu().numpy(), oracle.weight_grad(x64, dy64, H, BK, BN, R1024, 0.5), torch.bfloat16,
+                 "dHW (static scratch, scatter instead of fold)")
+
+
 def test_static_scratch_refuses_what_does_not_fit():
     from rzlinear_amd import _lib
     lib = _lib.load()
