@@ -122,14 +122,19 @@ __device__ __forceinline__ u32x4_t mask_tail(u32x4_t v, int col, int col_lim) {
 // would start outside the operand is fetched from the nearest row / piece inside it (hashed
 // pieces need nothing: every tile index hashes to a valid slice).  What such a piece holds
 // only reaches rows or columns of C that the bounds-checked epilogue never stores.
+// WK (forward / input-grad): WK groups of WI x WJ wavefronts share a C tile; group g multiplies
+// the g-th part of every R step and the groups' accumulators are added through LDS at the end.
+// For a tile with one wavefront per SIMD (fp32, 64 x 64) this puts a second wavefront on every
+// SIMD, which fills the MFMA pipe while the first waits for its fragments.
 template <typename T, int OP, int TI, int TJ, int WI, int WJ, int NSTAGE, bool FULL, bool COLSUM = false,
-          bool CLAMP = false>
+          bool CLAMP = false, int WK = 1>
 struct GemmKernel {
+  static_assert(WK == 1 || (OP != kWeightGrad && NSTAGE == 2), "the R step is shared out only by the pipelined store kernels");
   static_assert(!(FULL && CLAMP), "complete tiles need no clamping");
   static_assert(!COLSUM || OP == kWeightGrad, "column sums belong to the weight-grad contraction");
   typedef ElemTraits<T> Tr;
   typedef typename Mfma<T>::Frag Frag;
-  static constexpr int kThreads = 64 * WI * WJ;
+  static constexpr int kThreads = 64 * WI * WJ * WK;
   static constexpr int VEC = Tr::kVec;
   static constexpr bool k16 = (Tr::kBytes == 2);
   // R step: 128 bytes of R — except the directly staged 128 tile with eight wavefronts, which
@@ -272,7 +277,8 @@ struct GemmKernel {
   static __device__ __forceinline__ void run_item(const GemmParams& p, Smem& sm, const int tid, int bx, int by, int gx) {
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // (uniform: lives in a scalar register)
-    const int wave_i = wave / WJ, wave_j = wave % WJ;
+    const int wave_k = wave / (WI * WJ);                 // which part of every R step
+    const int wave_i = (wave % (WI * WJ)) / WJ, wave_j = wave % WJ;
     // Offset in the C tile of a wavefront's 32x32 block (a, b).  Forward and input-grad give a
     // wavefront one contiguous WTI x WTJ sub-tile (whole cache lines per store).  Weight-grad
     // deals the blocks round-robin instead, so that the blocks of one hashed tile belong to
@@ -736,16 +742,17 @@ struct GemmKernel {
       // when stage s&1 has been read for the last time, the direct-to-LDS loads of step s+2
       // are issued into it; they have a whole step to land and are waited for just before the
       // barrier of step s+1.
-      constexpr int NKS = TR / KS;
-      static_assert(NKS >= 3, "pipeline needs at least three sub-steps per R step");
+      constexpr int NKS = TR / KS / WK;   // sub-steps of this wavefront's part of an R step
+      static_assert(NKS >= 3 && NKS * KS * WK == TR, "pipeline needs at least three sub-steps per R step");
+      const int ks0 = wave_k * NKS;
       Frag fa[2][MI], fb[2][MJ];
       auto frags = [&](int st, int ks, int buf) {
 #pragma unroll
         for (int a = 0; a < MI; a++)
-          fa[buf][a] = lds_frag<A_LAYOUT, LA>(sm.a[st], blk_i(a), ks, lane);
+          fa[buf][a] = lds_frag<A_LAYOUT, LA>(sm.a[st], blk_i(a), ks0 + ks, lane);
 #pragma unroll
         for (int b = 0; b < MJ; b++)
-          fb[buf][b] = lds_frag<B_LAYOUT, LB>(sm.b[st], blk_j(b), ks, lane);
+          fb[buf][b] = lds_frag<B_LAYOUT, LB>(sm.b[st], blk_j(b), ks0 + ks, lane);
       };
       auto mfmas = [&](int buf) {
 #pragma unroll
@@ -976,6 +983,34 @@ struct GemmKernel {
         scatter(p.scatter);
       }
     } else {
+      if constexpr (WK > 1) {
+        // add up the groups' accumulators: groups 1.. park theirs in the dead operand stages,
+        // group 0 adds them (fixed order) and stores the tile
+        float* park = reinterpret_cast<float*>(&sm);
+        static_assert(sizeof(float) * (WK - 1) * TI * TJ <= sizeof(Smem), "the accumulators must fit the stages");
+        __syncthreads();   // every wavefront is done reading the stages
+        const int slot = ((wave % (WI * WJ)) * MI * MJ) * 16 * 64 + lane;
+        if (wave_k > 0) {
+#pragma unroll
+          for (int a = 0; a < MI; a++)
+#pragma unroll
+            for (int b = 0; b < MJ; b++)
+#pragma unroll
+              for (int e = 0; e < 16; e++)
+                park[(wave_k - 1) * TI * TJ + slot + ((a * MJ + b) * 16 + e) * 64] = acc[a][b][e];
+        }
+        __syncthreads();
+        if (wave_k > 0) return;
+#pragma unroll
+        for (int g = 1; g < WK; g++)
+#pragma unroll
+          for (int a = 0; a < MI; a++)
+#pragma unroll
+            for (int b = 0; b < MJ; b++)
+#pragma unroll
+              for (int e = 0; e < 16; e++)
+                acc[a][b][e] += park[(g - 1) * TI * TJ + slot + ((a * MJ + b) * 16 + e) * 64];
+      }
       if (p.partial != nullptr) {
         // R is split over the slices `by` (few C tiles, long R): this slice's scaled fp32 partial
         // result goes to its own [I][J] plane; a second kernel adds the planes up
@@ -1023,9 +1058,9 @@ struct GemmKernel {
   }
 };
 
-template <typename T, int OP, int TI, int TJ, int WI, int WJ, int NSTAGE, bool FULL, bool COLSUM, bool CLAMP>
-__global__ __launch_bounds__(64 * WI * WJ) void rz_gemm_kernel(GemmParams p) {
-  typedef GemmKernel<T, OP, TI, TJ, WI, WJ, NSTAGE, FULL, COLSUM, CLAMP> K;
+template <typename T, int OP, int TI, int TJ, int WI, int WJ, int NSTAGE, bool FULL, bool COLSUM, bool CLAMP, int WK = 1>
+__global__ __launch_bounds__(64 * WI * WJ * WK) void rz_gemm_kernel(GemmParams p) {
+  typedef GemmKernel<T, OP, TI, TJ, WI, WJ, NSTAGE, FULL, COLSUM, CLAMP, WK> K;
   extern __shared__ __attribute__((aligned(16))) unsigned char rz_smem_raw[];
   K::run(p, *reinterpret_cast<typename K::Smem*>(rz_smem_raw));
 }

@@ -9,11 +9,12 @@
 
 namespace rz {
 
-template <typename T, int OP, int TI, int TJ, int WI, int WJ, int NSTAGE, bool FULL, bool COLSUM, bool CLAMP = false>
+template <typename T, int OP, int TI, int TJ, int WI, int WJ, int NSTAGE, bool FULL, bool COLSUM, bool CLAMP = false,
+          int WK = 1>
 static hipError_t launch_one(GemmParams p, const WeightGradPlan* plan, const SplitPlan* split,
                              hipStream_t stream) {
   static std::atomic<uint64_t> lds_limit_raised{0};
-  typedef GemmKernel<T, OP, TI, TJ, WI, WJ, NSTAGE, FULL, COLSUM, CLAMP> K;
+  typedef GemmKernel<T, OP, TI, TJ, WI, WJ, NSTAGE, FULL, COLSUM, CLAMP, WK> K;
   p.tiles_i = (p.I + TI - 1) / TI;
   p.tiles_j = (p.J + TJ - 1) / TJ;
   const long long tiles = (long long)p.tiles_i * p.tiles_j;
@@ -47,7 +48,7 @@ static hipError_t launch_one(GemmParams p, const WeightGradPlan* plan, const Spl
     p.r_chunk = r_steps * K::TR;
     p.partial = nullptr;
   }
-  auto kernel = rz_gemm_kernel<T, OP, TI, TJ, WI, WJ, NSTAGE, FULL, COLSUM, CLAMP>;
+  auto kernel = rz_gemm_kernel<T, OP, TI, TJ, WI, WJ, NSTAGE, FULL, COLSUM, CLAMP, WK>;
   size_t smem = sizeof(typename K::Smem);
   static_assert(sizeof(typename K::Smem) <= 160 * 1024, "tile does not fit the 160 KB LDS of a compute unit");
   if (OP == kWeightGrad && p.image_pitch > 0) {
@@ -67,14 +68,14 @@ static hipError_t launch_one(GemmParams p, const WeightGradPlan* plan, const Spl
 // FULL kernels carry no bounds checks: every tile and every R step must be complete.  Ragged
 // shapes: 16-bit tiles can still be staged directly, with edge pieces fetched from inside the
 // operands (CLAMP); everything else takes the bounds-checked kernel.
-template <typename T, int OP, int TILE, int WI, int WJ, int NSTAGE, bool COLSUM = false>
+template <typename T, int OP, int TILE, int WI, int WJ, int NSTAGE, bool COLSUM = false, int WK = 1>
 static hipError_t launch_tile(GemmParams p, const WeightGradPlan* plan, const SplitPlan* split,
                               const KernelForm& form, hipStream_t stream) {
   // (the form was derived on the host from the same rules that select the instantiation here:
   //  refuse to launch if the two ever disagree about the step length)
   if (form.full) {
     if (form.step != GemmKernel<T, OP, TILE, TILE, WI, WJ, NSTAGE, true>::TR) return hipErrorInvalidValue;
-    return launch_one<T, OP, TILE, TILE, WI, WJ, NSTAGE, true, COLSUM>(p, plan, split, stream);
+    return launch_one<T, OP, TILE, TILE, WI, WJ, NSTAGE, true, COLSUM, false, WK>(p, plan, split, stream);
   }
   if constexpr (sizeof(T) == 2 && NSTAGE == 2 && TILE >= 128) {
     if (form.clamp) {
@@ -83,19 +84,22 @@ static hipError_t launch_tile(GemmParams p, const WeightGradPlan* plan, const Sp
     }
   }
   if (form.clamp || form.step != GemmKernel<T, OP, TILE, TILE, WI, WJ, NSTAGE, false>::TR) return hipErrorInvalidValue;
-  return launch_one<T, OP, TILE, TILE, WI, WJ, NSTAGE, false, COLSUM>(p, plan, split, stream);
+  return launch_one<T, OP, TILE, TILE, WI, WJ, NSTAGE, false, COLSUM, false, WK>(p, plan, split, stream);
 }
 
-template <typename T, int TILE, int WI, int WJ, int NSTAGE>
+template <typename T, int TILE, int WI, int WJ, int NSTAGE, int WK = 1>
 static hipError_t launch_op(int op, GemmParams p, const WeightGradPlan* plan, const SplitPlan* split,
                             const KernelForm& form, hipStream_t stream) {
   switch (op) {
-    case kForward: return launch_tile<T, kForward, TILE, WI, WJ, NSTAGE>(p, plan, split, form, stream);
-    case kInputGrad: return launch_tile<T, kInputGrad, TILE, WI, WJ, NSTAGE>(p, plan, split, form, stream);
+    case kForward: return launch_tile<T, kForward, TILE, WI, WJ, NSTAGE, false, WK>(p, plan, split, form, stream);
+    case kInputGrad: return launch_tile<T, kInputGrad, TILE, WI, WJ, NSTAGE, false, WK>(p, plan, split, form, stream);
     case kWeightGrad:
-      // with a column-sum target the kernel also produces the bias gradient's partial sums
-      if (p.colsum != nullptr) return launch_tile<T, kWeightGrad, TILE, WI, WJ, NSTAGE, true>(p, plan, split, form, stream);
-      return launch_tile<T, kWeightGrad, TILE, WI, WJ, NSTAGE>(p, plan, split, form, stream);
+      if constexpr (WK == 1) {
+        // with a column-sum target the kernel also produces the bias gradient's partial sums
+        if (p.colsum != nullptr) return launch_tile<T, kWeightGrad, TILE, WI, WJ, NSTAGE, true>(p, plan, split, form, stream);
+        return launch_tile<T, kWeightGrad, TILE, WI, WJ, NSTAGE>(p, plan, split, form, stream);
+      }
+      return hipErrorInvalidValue;
     default: return hipErrorInvalidValue;
   }
 }
@@ -106,7 +110,8 @@ static hipError_t launch_op(int op, GemmParams p, const WeightGradPlan* plan, co
 //        eight of 64 x 32 when there is about one workgroup per compute unit; tuning.stages = 1
 //        selects a single-stage form that leans on several workgroups per compute unit
 //        instead of a pipeline (tuning aid)
-//    64:  64 x  64, four wavefronts of 32 x 32, for problems with few tiles
+//    64:  64 x  64, four wavefronts of 32 x 32, for problems with few tiles; fp32 forward /
+//        input-grad: eight, in two groups that share every R step between them
 template <typename T>
 static hipError_t launch_gemm_t(int op, GemmParams p, const WeightGradPlan* plan, const SplitPlan* split,
                                 const rz_tuning& tuning, hipStream_t stream) {
@@ -119,6 +124,9 @@ static hipError_t launch_gemm_t(int op, GemmParams p, const WeightGradPlan* plan
   switch (form.tile * 100 + form.waves * 10 + form.stages) {
     case 25682: return launch_op<T, 256, 2, 4, 2>(op, p, plan, split, form, stream);
     case 6442: return launch_op<T, 64, 2, 2, 2>(op, p, plan, split, form, stream);
+    case 6482:   // fp32 forward / input-grad: two groups of four wavefronts share every R step
+      if constexpr (sizeof(T) == 4) return launch_op<T, 64, 2, 2, 2, 2>(op, p, plan, split, form, stream);
+      return hipErrorInvalidValue;
     case 12841: return launch_op<T, 128, 2, 2, 1>(op, p, plan, split, form, stream);
     case 12882: return launch_op<T, 128, 2, 4, 2>(op, p, plan, split, form, stream);
     case 12842: return launch_op<T, 128, 2, 2, 2>(op, p, plan, split, form, stream);

@@ -359,7 +359,11 @@ static inline KernelForm kernel_form(int op, int I, int J, int R, int chunk, int
   // 128 tile: with about one workgroup per compute unit, eight wavefronts (two per SIMD, 64 x 32
   // each) hide latency better than four of 64 x 64; with more workgroups resident the
   // four-wavefront form does less LDS traffic per flop
-  f.waves = tile == 256 ? 8 : tile == 64 ? 4 : (f.stages == 1 ? 4 : (workgroups <= kComputeUnits * 3 / 2 ? 8 : 4));
+  // 64 tile: four wavefronts; fp32 forward / input-grad take eight (two groups that share every R
+  // step: a second wavefront per SIMD keeps the MFMA pipe fed while the first waits for LDS)
+  f.waves = tile == 256 ? 8
+            : tile == 64 ? ((elem_bytes == 4 && op != kWeightGrad) ? 8 : 4)
+                         : (f.stages == 1 ? 4 : (workgroups <= kComputeUnits * 3 / 2 ? 8 : 4));
   const bool direct_capable = elem_bytes == 2 && f.stages == 2 && tile >= 128;
   const int step_plain = 128 / elem_bytes;
   const int step_direct = (direct_capable && tile == 128 && f.waves == 8) ? 256 / elem_bytes : step_plain;
