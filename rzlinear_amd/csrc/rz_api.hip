@@ -440,6 +440,8 @@ static int weight_grad_impl(const void* X, const void* dY, void* dHW, void* dbia
     fp.h = p.h;
     fp.H = H;
     fp.pitch = (H + 3) & ~3;
+    fp.K = K;
+    fp.N = N;
     fp.tiles_k = p.out_tiles_k;
     fp.tiles_n = p.out_tiles_n;
     fp.slices = plan.splits;

@@ -106,7 +106,7 @@ struct GemmParams {
   int image_pitch;    // > 0 selects the LDS mode: floats per partial image (H rounded up to 4)
   float* tiles_out;   // weight-grad, non-null: no scatter at all; the C tile (scaled X^T.dY) is stored
                       // hashed tile by hashed tile, tile (tk, tn) of slice s as BK*BN contiguous floats
-                      // at ((s * tiles_k + tk) * tiles_n + tn) * BK*BN (zeros beyond K x N), and a
+                      // at ((s * tiles_k + tk) * tiles_n + tn) * BK*BN (only the part inside K x N is defined), and a
                       // second kernel folds the tiles into dHW
   int out_tiles_k, out_tiles_n;   // ... its tile grid: ceil(K / BK) x ceil(N / BN)
   float* colsum;      // weight-grad that also yields the bias gradient: partial column sums of B

@@ -6,7 +6,7 @@
 // additions is fixed (the order of the workgroup's tile list), so the result is the same on every call.
 //
 // A hashed tile is BK*BN contiguous elements of hashed_weight and BK*BN contiguous floats of the
-// tile-by-tile buffer, so its reads are whole cache lines whatever its offset.  Inside the
+// tile-by-tile buffer (of which only the part inside K x N is read), so its reads are whole cache lines whatever its offset.  Inside the
 // workgroup thread i owns the window positions i, i + 1024, i + 2048, ...: for every tile it
 // reads the elements that fall on its own positions (consecutive threads, consecutive addresses)
 // and adds them with plain LDS read-add-write.  No two threads ever touch the same LDS word, so
@@ -34,6 +34,7 @@ struct FoldParams {
   int accumulate;       //     added to what dHW holds, if set
   HashParams h;
   int H, pitch;
+  int K, N;             // extent of X^T.dY: what a tile holds beyond it was never written and is not read
   int tiles_k, tiles_n, slices;
   int window;           // floats per window, a multiple of kFoldThreads
   int windows, shares;
@@ -45,7 +46,7 @@ static constexpr int kFoldScan = 32;         // tile indices per thread and list
 static constexpr int kFoldWindowMax = 32768;
 
 static inline size_t fold_lds_bytes(int window) {
-  return (size_t)window * sizeof(float) + 2 * kFoldList * sizeof(int) + 32 * sizeof(int);
+  return (size_t)window * sizeof(float) + 3 * kFoldList * sizeof(int) + 32 * sizeof(int);
 }
 
 // LPE: loads per list entry and thread, BK*BN / 1024 (1 for smaller tiles: then only the first
@@ -57,7 +58,8 @@ __global__ __launch_bounds__(kFoldThreads) void fold_tiles_kernel(const FoldPara
   float* img = fold_lds;
   int* list_at = reinterpret_cast<int*>(fold_lds + p.window);   // first float of the entry's tile
   int* list_rel = list_at + kFoldList;                           // where the tile starts, relative to the window
-  int* wave_sum = list_rel + kFoldList;                          // [16] per-wavefront counts, [16] = total
+  int* list_lim = list_rel + kFoldList;                          // rows | columns << 16 of the tile inside K x N
+  int* wave_sum = list_lim + kFoldList;                          // [16] per-wavefront counts, [16] = total
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int win = blockIdx.x % p.windows, share = blockIdx.x / p.windows;
   const int w0 = win * p.window;
@@ -137,9 +139,13 @@ __global__ __launch_bounds__(kFoldThreads) void fold_tiles_kernel(const FoldPara
       if (rank >= want_lo && rank < want_hi) {
         const int id = lo + tid + j * kFoldThreads;
         const int rel = p.offsets[id] - w0;
+        const int tk = id / p.tiles_n, tn = id - tk * p.tiles_n;
+        const int rows = (p.K - tk * p.h.BK) < p.h.BK ? (p.K - tk * p.h.BK) : p.h.BK;
+        const int cols = (p.N - tn * p.h.BN) < p.h.BN ? (p.N - tn * p.h.BN) : p.h.BN;
         for (int s = 0; s < p.slices; s++) {
           list_at[(rank - want_lo) * p.slices + s] = (s * ntiles + id) << eshift;
           list_rel[(rank - want_lo) * p.slices + s] = rel;
+          list_lim[(rank - want_lo) * p.slices + s] = rows | cols << 16;
         }
       }
       rank++;
@@ -160,6 +166,7 @@ __global__ __launch_bounds__(kFoldThreads) void fold_tiles_kernel(const FoldPara
       const bool have = lane < kRound && t + lane < total;
       const int my_rel = have ? list_rel[t + lane] : -(1 << 29);   // (far away: no element lands in the window)
       const int my_at = have ? list_at[t + lane] : 0;
+      const int my_lim = have ? list_lim[t + lane] : 0;
       bool meets = false;
 #pragma unroll
       for (int d = 1; d < kRound; d++) {
@@ -171,9 +178,12 @@ __global__ __launch_bounds__(kFoldThreads) void fold_tiles_kernel(const FoldPara
 #pragma unroll
       for (int f = 0; f < 16; f++) {
         const int rel = __builtin_amdgcn_readlane(my_rel, f / LPE), at = __builtin_amdgcn_readlane(my_at, f / LPE);
+        const int lim = __builtin_amdgcn_readlane(my_lim, f / LPE);
         const int e = ((tid - rel) & (kFoldThreads - 1)) + (f % LPE) * kFoldThreads;   // my (f % LPE)-th element of the tile
         const int pos = rel + e;                                                       // (pos % 1024 == tid)
-        const bool ok = e < E && pos >= 0 && pos < wlen;
+        // (in the window, and inside K x N: the contraction wrote nothing beyond its own C tiles)
+        const bool ok = e < E && pos >= 0 && pos < wlen && (e >> p.h.bn_shift) < (lim & 0xffff) &&
+                        (e & (p.h.BN - 1)) < (lim >> 16);
         // (every thread loads, those without an element the tile's first float: with no branch
         //  around the loads their number is fixed, and the wait for this round's values can leave
         //  the next round's in flight)

@@ -132,6 +132,11 @@ FOLD_CASES = [
     (130, 300, 200, 37000, 16, 16, 0),         # tiles smaller than the workgroup: 256 of 1024 threads have an element
     (96, 512, 768, 60000, 128, 128, 256),      # sixteen loads per tile and thread
     (70, 1024, 1024, 1 << 20, 32, 32, 0),      # 32 windows; one load per tile and thread
+    # hashed tiles that reach beyond K x N, and beyond the C tiles that were computed (what they
+    # hold there was never written and must not be read); offsets confined to a few values
+    (32, 64, 776, 20000, 128, 128, 0),
+    (100, 16, 264, 2065, 128, 16, 0),
+    (512, 1024, 264, 16385, 128, 128, 0),
 ]
 
 
@@ -146,7 +151,7 @@ def test_tiles_stored_plainly_and_folded_into_the_gradient(oracle, tuned, shape,
     from rzlinear_amd.impl.RzLinearBackward import (rz_linear_backward_weight_bias_grad_tl,
                                                     rz_linear_backward_weight_grad_tl)
     M, K, N, H, BK, BN, tile = shape
-    tuned(fold=1, window=-1, tile=tile)
+    tuned(fold=1, window=-1, lds_image=-1, tile=tile)
     code = _lib.dtype_code(torch.empty(0, dtype=dtype))
     plan = _lib.plan_query(2, M, K, N, H, BK, BN, code)
     _say("fold", shape, dtype, plan)
@@ -169,7 +174,7 @@ def test_tiles_stored_plainly_and_folded_into_the_gradient(oracle, tuned, shape,
     torch.cuda.synchronize()
     assert rel_err(buf.cpu().numpy(), start.double().cpu().numpy() + ref) <= TOL[dtype]
     # and the atomic scatter agrees
-    tuned(fold=-1, window=-1, tile=tile)
+    tuned(fold=-1, window=-1, lds_image=-1, tile=tile)
     assert _lib.plan_query(2, M, K, N, H, BK, BN, code)["mode"] == "atomics"
     c = rz_linear_backward_weight_grad_tl(x, dy, 0.5, M, K, N, H, *rargs(R1024), **kw)
     torch.cuda.synchronize()
