@@ -78,6 +78,23 @@ static inline double tile_score(int I, int J, int t, int elem_bytes) {
   return tile_score_full(I, J, t, elem_bytes) * ((double)I * (double)J) / (wgs * t * t);
 }
 
+// Relative throughput of `wgs` workgroups of tile t (see tile_score_full, which this restates for
+// a workgroup count that includes the slices of a cut contraction).
+static inline double tile_rate(double wgs, int t, int elem_bytes) {
+  const double per_cu = wgs / kComputeUnits;
+  const bool f32 = elem_bytes == 4;
+  const int slots = (t == 256) ? 1 : (t == 128 ? 2 : 4);
+  const double lo = (t == 256) ? 1.0 : (t == 128 ? (f32 ? 0.86 : 0.51) : (f32 ? 0.60 : 0.16));
+  const double hi = (t == 256) ? 1.0 : (t == 128 ? (f32 ? 0.90 : 0.75) : (f32 ? 0.80 : 0.33));
+  if (per_cu <= 1.0) return lo * per_cu;
+  const double cap = (double)kComputeUnits * slots;
+  const double rounds = (double)((long long)((wgs + cap - 1) / cap));
+  const double util = wgs / (rounds * cap);
+  const double fill = per_cu >= slots ? 1.0 : (per_cu - 1.0) / (slots - 1.0);
+  const double e = lo + (hi - lo) * fill;
+  return per_cu >= slots ? e * util : e;
+}
+
 // C-tile edge for a contraction with an I x J result: the best-scoring of 256, 128, 64.
 static inline int pick_tile(int I, int J, int elem_bytes, const rz_tuning& tuning) {
   if (tuning.tile) return tuning.tile;
@@ -191,9 +208,28 @@ static inline WeightGradPlan plan_weight_grad(int M, int K, int N, int H, int BK
   // split the reduction over M when there are too few W tiles to fill the chip
   const long long target = (pl.tile >= 256) ? kComputeUnits : (pl.tile == 128 ? 2 * kComputeUnits : kTargetWorkgroups);
   long long want = (target + tiles - 1) / tiles;
-  if (!image && want > 8) want = 8;   // every slice repeats the K*N global atomics
   if (want > r_steps) want = r_steps;
   if (want < 1) want = 1;
+  if (!image) {
+    // every slice repeats the K*N adds of the scatter (global atomics, about 5.4 ps each, some 70 %
+    // of which the contraction does not hide): the number of slices with the least estimated time
+    if (want > 8) want = 8;
+    const double peak = elem_bytes == 4 ? 137e6 : 1150e6;   // flop per microsecond of the 256 tile on a full chip
+    double best_us = 0.0;
+    long long best = 1;
+    for (long long w = 1; w <= want; w++) {
+      const long long per = (r_steps + w - 1) / w;
+      if ((r_steps + per - 1) / per != w) continue;
+      const double steps = (double)per * (TR * elem_bytes / 128);
+      const double us = 2.0 * (double)M * K * N / (peak * tile_rate((double)tiles * w, pl.tile, elem_bytes) * steps / (steps + 2.0)) +
+                        (double)w * K * N * 3.8e-6;
+      if (best_us == 0.0 || us < best_us * 0.97) {
+        best_us = us;
+        best = w;
+      }
+    }
+    want = best;
+  }
   const int steps_per = (int)((r_steps + want - 1) / want);
   pl.splits = (r_steps + steps_per - 1) / steps_per;
   pl.r_chunk = steps_per * TR;
@@ -285,23 +321,6 @@ struct SplitPlan {
   int r_chunk;
   size_t workspace_bytes;
 };
-
-// Relative throughput of `wgs` workgroups of tile t (see tile_score_full, which this restates for
-// a workgroup count that includes the slices of a cut contraction).
-static inline double tile_rate(double wgs, int t, int elem_bytes) {
-  const double per_cu = wgs / kComputeUnits;
-  const bool f32 = elem_bytes == 4;
-  const int slots = (t == 256) ? 1 : (t == 128 ? 2 : 4);
-  const double lo = (t == 256) ? 1.0 : (t == 128 ? (f32 ? 0.86 : 0.51) : (f32 ? 0.60 : 0.16));
-  const double hi = (t == 256) ? 1.0 : (t == 128 ? (f32 ? 0.90 : 0.75) : (f32 ? 0.80 : 0.33));
-  if (per_cu <= 1.0) return lo * per_cu;
-  const double cap = (double)kComputeUnits * slots;
-  const double rounds = (double)((long long)((wgs + cap - 1) / cap));
-  const double util = wgs / (rounds * cap);
-  const double fill = per_cu >= slots ? 1.0 : (per_cu - 1.0) / (slots - 1.0);
-  const double e = lo + (hi - lo) * fill;
-  return per_cu >= slots ? e * util : e;
-}
 
 // Tile and number of slices together: the pair with the least estimated time.  A slice pays the
 // fill and drain of its pipeline (about three steps), the cut pays the fp32 partial planes
