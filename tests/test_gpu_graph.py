@@ -23,6 +23,7 @@ def _say(*a):
     (512, 512, 768, 9000, torch.bfloat16),      # LDS-image weight-grad, direct staging
     (96, 1024, 512, 70000, torch.float32),      # atomic scatter (zero-fill kernel inside the graph), split forward
     (32, 4096, 4096, 1 << 20, torch.bfloat16),  # window kernel (offset table built inside the graph)
+    (520, 4096, 4096, 200000, torch.bfloat16),  # tile-by-tile output + fold kernel + reduction of its images
 ], ids=lambda c: "x".join(map(str, c[:4])) + "-" + str(c[4]).split(".")[-1])
 def test_step_captured_in_a_graph_replays_correctly(cfg):
     from rzlinear_amd import _lib
