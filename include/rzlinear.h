@@ -288,6 +288,26 @@ int rz_materialize(const void* HW, void* W, int K, int N, int H, int BK, int BN,
 int rz_tile_offsets_device(int32_t* d_out, int K, int N, int H, int BK, int BN,
                            const int32_t R[8], int hash_levels, void* stream);
 
+/*
+ * Fused optimiser steps over a parameter vector of n elements (the hashed_weight that one or
+ * several layers share, or a bias): parameter, gradient and state are read and written once.
+ * No counterpart in the reference, which leaves the update to torch.optim; the rules are
+ * torch.optim.SGD's (momentum, dampening, weight_decay, nesterov) and torch.optim.Adam's /
+ * AdamW's (decoupled != 0), amsgrad off.  param_dtype is an rz_dtype; grad_dtype is the same or
+ * RZ_F32 (a gradient accumulated in fp32, RZ_WG_DHW_F32).  grad is multiplied by grad_scale
+ * first (1 / loss scale, 1 / number of micro-batches; 1.0f = none).  State buffers are fp32.
+ * master (optional) is an fp32 copy of the parameter that carries the update; the parameter
+ * then receives its rounded value (16-bit parameters, whose small updates would otherwise be
+ * rounded away).  rz_sgd_step: momentum_buf may be NULL when momentum == 0; first_step != 0
+ * makes the buffer start as the gradient, as torch does.  rz_adam_step: step counts from 1.
+ */
+int rz_sgd_step(void* param, const void* grad, float* momentum_buf, float* master, int64_t n,
+                int param_dtype, int grad_dtype, float lr, float momentum, float dampening,
+                float weight_decay, int nesterov, int first_step, float grad_scale, void* stream);
+int rz_adam_step(void* param, const void* grad, float* exp_avg, float* exp_avg_sq, float* master, int64_t n,
+                 int param_dtype, int grad_dtype, float lr, float beta1, float beta2, float eps,
+                 float weight_decay, int decoupled, int step, float grad_scale, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -23,6 +23,7 @@ EXPORTS = (
     "rz_weight_grad_ex", "rz_forward_hashed", "rz_input_grad_hashed", "rz_weight_grad_hashed", "rz_materialize",
     "rz_forward_hashed_workspace_bytes", "rz_input_grad_hashed_workspace_bytes",
     "rz_weight_grad_hashed_workspace_bytes", "rz_plan_query", "rz_weight_grad_static",
+    "rz_sgd_step", "rz_adam_step",
 )
 
 
@@ -141,6 +142,12 @@ def load():
     lib.rz_weight_grad_hashed_workspace_bytes.argtypes = [c_int] * 7 + [ctypes.c_uint, c_int, tun]
     lib.rz_plan_query.restype = c_int
     lib.rz_plan_query.argtypes = [c_int] * 8 + [ctypes.c_uint, c_int, tun, i32p]
+    f32p = c_vp
+    lib.rz_sgd_step.restype = c_int
+    lib.rz_sgd_step.argtypes = [c_vp, c_vp, f32p, f32p, c_i64, c_int, c_int, c_f, c_f, c_f, c_f, c_int, c_int, c_f, c_vp]
+    lib.rz_adam_step.restype = c_int
+    lib.rz_adam_step.argtypes = [c_vp, c_vp, f32p, f32p, f32p, c_i64, c_int, c_int, c_f, c_f, c_f, c_f, c_f, c_int,
+                                 c_int, c_f, c_vp]
     lib.rz_materialize.restype = c_int
     lib.rz_materialize.argtypes = [c_vp, c_vp, c_int, c_int, c_int, c_int, c_int, i32p, c_int, c_i64,
                                    c_int, c_vp]
