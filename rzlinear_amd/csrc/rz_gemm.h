@@ -183,6 +183,7 @@ struct GemmKernel {
   static constexpr int kOffBank = 16;
   static constexpr int kOffWindow = (TR / 16) * (TJ / 16);
   static constexpr int kOffEntries = (OP == kWeightGrad) ? (TI / 16) * (TJ / 16) : kOffSlots * kOffWindow;
+  static constexpr int kTurnEntries = 65;   // weight-grad, behind the offsets: the round of up to 64 hashed tiles, and the number of rounds
 
   struct Smem {
     alignas(16) T a[NSTAGE][LA::kElems];
@@ -935,7 +936,7 @@ struct GemmKernel {
         if (p.h.bk_shift >= 5 && p.h.bn_shift >= 5) {
           // Every 32x32 accumulator block lies inside one hashed tile, whose BK*BN addresses
           // are all distinct.  LDS float atomics are slow, so instead the tiles of the window
-          // take turns: in round t only the blocks of tile t are added, with plain
+          // take turns: in a round only the blocks of that round's tile(s) are added, with plain
           // read-add-write, and a barrier separates the rounds.
           int blk_tile[MI][MJ], blk_base[MI][MJ];
 #pragma unroll
@@ -949,7 +950,40 @@ struct GemmKernel {
               blk_base[a][b] = etab[t] + ((k0 & (p.h.BK - 1)) + (lane >> 5) * 4) * p.h.BN +
                                ((n0 + (lane & 31)) & (p.h.BN - 1));
             }
-          for (int t = 0; t < w.count; t++) {
+          // With many hashed tiles per C tile, tiles whose slices do not meet may share a round:
+          // a tile's round is one later than the latest round of the EARLIER tiles that meet its
+          // slice (round 0 if none does), so every element still receives its adds in tile order
+          // and the result has the same bits as with one round per tile.  The first wavefront
+          // works the rounds out, tile by tile: lane j keeps the tiles of round j as a bit mask.
+          int rounds = w.count;
+          const bool levelled = w.count > 16 && w.count <= 64;
+          if (levelled) {
+            int* turn = etab + kOffEntries;             // [count] rounds, then their number
+            if (wave == 0) {
+              const int off_u = lane < w.count ? etab[lane] : 0;
+              const int extent = p.h.BK * p.h.BN;
+              unsigned long long members = 0ull;
+              int my_turn = 0, turns = 1;
+              for (int t = 0; t < w.count; t++) {
+                const int d = off_u - __builtin_amdgcn_readlane(off_u, t);
+                const unsigned long long meets = __ballot(lane < t && d < extent && d > -extent);
+                const unsigned long long busy = __ballot((members & meets) != 0ull);   // rounds with a tile that meets t
+                const int k = busy ? 64 - __builtin_clzll(busy) : 0;
+                if (lane == k) members |= 1ull << t;
+                if (lane == t) my_turn = k;
+                turns = k + 1 > turns ? k + 1 : turns;
+              }
+              if (lane < w.count) turn[lane] = my_turn;
+              if (lane == 0) turn[64] = turns;
+            }
+            __syncthreads();
+            rounds = __builtin_amdgcn_readfirstlane(turn[64]);
+#pragma unroll
+            for (int a = 0; a < MI; a++)
+#pragma unroll
+              for (int b = 0; b < MJ; b++) blk_tile[a][b] = __builtin_amdgcn_readfirstlane(turn[blk_tile[a][b]]);
+          }
+          for (int t = 0; t < rounds; t++) {
             if (steps > 0) {
 #pragma unroll
               for (int a = 0; a < MI; a++)

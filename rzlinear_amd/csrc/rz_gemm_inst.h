@@ -53,7 +53,7 @@ static hipError_t launch_one(GemmParams p, const WeightGradPlan* plan, const Spl
   static_assert(sizeof(typename K::Smem) <= 160 * 1024, "tile does not fit the 160 KB LDS of a compute unit");
   if (OP == kWeightGrad && p.image_pitch > 0) {
     // the dHW image and the scatter's offset table behind it may need more than the stages
-    const size_t need = (size_t)p.image_pitch * sizeof(float) + K::kOffEntries * sizeof(int);
+    const size_t need = (size_t)p.image_pitch * sizeof(float) + (K::kOffEntries + K::kTurnEntries) * sizeof(int);
     if (need > smem) smem = need;
   }
   if (smem > 64 * 1024) {
