@@ -255,7 +255,9 @@ static inline WeightGradPlan plan_weight_grad(int M, int K, int N, int H, int BK
       const double fold_us = (store_us > product_us ? store_us - product_us : 0.0) + (all_us > one_us ? all_us : one_us) + 10.0;
       if (t.fold == 1 || fold_us < atomics_us) {
         pl.fold = f;
-        pl.fold_us = product_us + fold_us;
+        // (for the comparison with the window kernel: every round of workgroups of the contraction
+        //  kernel also pays its fill, drain and store, about 5 us, which matters when M is small)
+        pl.fold_us = product_us + fold_us + 5.0 * (double)((pl.workgroups + kComputeUnits - 1) / kComputeUnits);
       }
     }
   }
