@@ -50,27 +50,38 @@ static inline long long tile_count(int I, int J, int t) {
   return (long long)((I + t - 1) / t) * ((J + t - 1) / t);
 }
 
+// Rate of `wgs` equal workgroups on the chip relative to a full one, when a compute unit runs at
+// `lo` with one workgroup resident and at `hi` with `slots` (linear in between).  The hardware
+// deals workgroups out evenly, so the busiest compute unit holds c = ceil(wgs / CUs) of them; up to
+// `slots` they run side by side and finish together after c * w / e(c), while the chip's work is
+// wgs * w: the rate is (wgs / CUs) * e(c) / c.  (320 workgroups on 256 compute units leave 64 of
+// them with two: the launch takes as long as 512 would.)  Beyond `slots` per compute unit the
+// workgroups go in rounds of CUs * slots and a last, partly filled round costs a full one.
+static inline double occupancy_rate(double wgs, int slots, double lo, double hi) {
+  const double per_cu = wgs / kComputeUnits;
+  if (per_cu <= 1.0) return lo * per_cu;
+  auto e = [&](double c) { return slots > 1 ? lo + (hi - lo) * (c - 1.0) / (slots - 1.0) : hi; };
+  if (per_cu <= slots) {
+    const double c = (double)((long long)(per_cu + 0.999999));
+    return per_cu * e(c) / c;
+  }
+  const double cap = (double)kComputeUnits * slots;
+  const double rounds = (double)((long long)((wgs + cap - 1) / cap));
+  return hi * wgs / (rounds * cap);
+}
+
 // Relative throughput of a tile shape at a given number of workgroups, from measurements on
 // MI355X (256 tile at one workgroup per compute unit = 1).  16-bit types: the 128 tile reaches
 // 0.51 with one workgroup per compute unit and 0.75 with two or more, the 64 tile 0.16 and 0.33
 // (four or more).  fp32 is bound by the slower fp32 MFMA rate, so the small tiles lose far less:
-// 0.86 / 0.90 and 0.45 / 0.80.  Below one workgroup per compute unit the rate falls with the
-// idle compute units, and a last, partly filled round of workgroups costs a full one.
+// 0.86 / 0.90 and 0.45 / 0.80.  How the number of workgroups enters: occupancy_rate above.
 static inline double tile_score_full(int I, int J, int t, int elem_bytes) {
   const double wgs = (double)tile_count(I, J, t);
-  const double per_cu = wgs / kComputeUnits;
   const bool f32 = elem_bytes == 4;
   const int slots = (t == 256) ? 1 : (t == 128 ? 2 : 4);          // resident workgroups per CU
   const double lo = (t == 256) ? 1.0 : (t == 128 ? (f32 ? 0.86 : 0.51) : (f32 ? 0.45 : 0.16));  // one workgroup per CU
   const double hi = (t == 256) ? 1.0 : (t == 128 ? (f32 ? 0.90 : 0.75) : (f32 ? 0.80 : 0.33));  // `slots` per CU
-  if (per_cu <= 1.0) return lo * per_cu;
-  const double cap = (double)kComputeUnits * slots;
-  const double rounds = (double)((long long)((wgs + cap - 1) / cap));
-  const double util = wgs / (rounds * cap);                        // tail effect
-  const double fill = per_cu >= slots ? 1.0 : (per_cu - 1.0) / (slots - 1.0);
-  const double e = lo + (hi - lo) * fill;
-  // between one and `slots` workgroups per CU every CU is busy: no tail penalty yet
-  return per_cu >= slots ? e * util : e;
+  return occupancy_rate(wgs, slots, lo, hi);
 }
 // ... times the share of a tile grid's MFMA work that is not padding
 static inline double tile_score(int I, int J, int t, int elem_bytes) {
@@ -81,18 +92,11 @@ static inline double tile_score(int I, int J, int t, int elem_bytes) {
 // Relative throughput of `wgs` workgroups of tile t (see tile_score_full, which this restates for
 // a workgroup count that includes the slices of a cut contraction).
 static inline double tile_rate(double wgs, int t, int elem_bytes) {
-  const double per_cu = wgs / kComputeUnits;
   const bool f32 = elem_bytes == 4;
   const int slots = (t == 256) ? 1 : (t == 128 ? 2 : 4);
   const double lo = (t == 256) ? 1.0 : (t == 128 ? (f32 ? 0.86 : 0.51) : (f32 ? 0.60 : 0.16));
   const double hi = (t == 256) ? 1.0 : (t == 128 ? (f32 ? 0.90 : 0.75) : (f32 ? 0.80 : 0.33));
-  if (per_cu <= 1.0) return lo * per_cu;
-  const double cap = (double)kComputeUnits * slots;
-  const double rounds = (double)((long long)((wgs + cap - 1) / cap));
-  const double util = wgs / (rounds * cap);
-  const double fill = per_cu >= slots ? 1.0 : (per_cu - 1.0) / (slots - 1.0);
-  const double e = lo + (hi - lo) * fill;
-  return per_cu >= slots ? e * util : e;
+  return occupancy_rate(wgs, slots, lo, hi);
 }
 
 // C-tile edge for a contraction with an I x J result: the best-scoring of 256, 128, 64.
