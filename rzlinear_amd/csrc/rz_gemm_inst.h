@@ -151,12 +151,11 @@ static hipError_t launch_window_form(const WindowParams& p, int windows, hipStre
   return hipGetLastError();
 }
 
-// 16-bit operands whose rows hold whole 16-byte pieces go through the staged form.
+// Operands whose rows hold whole 16-byte pieces go through the staged form.
 template <typename T, int TBK, int TBN>
 static hipError_t launch_window_one(const WindowParams& p, int windows, hipStream_t stream) {
-  if constexpr (sizeof(T) == 2) {
-    if (p.K % 8 == 0 && p.N % 8 == 0) return launch_window_form<T, TBK, TBN, true>(p, windows, stream);
-  }
+  constexpr int kVec = 16 / (int)sizeof(T);
+  if (p.K % kVec == 0 && p.N % kVec == 0) return launch_window_form<T, TBK, TBN, true>(p, windows, stream);
   return launch_window_form<T, TBK, TBN, false>(p, windows, stream);
 }
 

@@ -44,11 +44,11 @@ struct WindowParams {
 // TBK x TBN is the hashed tile (compile time).  The unit of work is a strip of 32 rows of a tile
 // (its slice of hashed_weight is the 32 * TBN elements from off + 32 * TBN * strip on): a
 // wavefront holds the strip's 32x32 blocks in registers.
-// STAGED (16-bit types, K and N multiples of the 16-byte piece): operands travel as 16-byte
-// pieces through the wavefront's staging area; otherwise fragments are loaded element by element.
+// STAGED (K and N multiples of the 16-byte piece): operands travel as 16-byte pieces through the
+// wavefront's staging area (a quarter of the load instructions per byte for fp32, an eighth for the
+// 16-bit types); otherwise fragments are loaded element by element.
 template <typename T, int TBK, int TBN, bool STAGED>
 struct WindowKernel {
-  static_assert(!STAGED || sizeof(T) == 2, "staging serves the LDS transpose read of the 16-bit types");
   static_assert(TBK % 32 == 0 && TBN % 32 == 0, "a tile is whole 32x32 blocks");
   typedef ElemTraits<T> Tr;
   typedef typename Mfma<T>::Frag Frag;
@@ -62,12 +62,18 @@ struct WindowKernel {
   static constexpr int kGroupRows = sizeof(T) == 4 ? 8 : 16;
   static constexpr int GS = kGroupRows / KS;             // MFMA steps per group
   static constexpr int kBatch = STAGED ? 8 : 4;           // tile offsets a lane loads at a time
+  // Items (one group of rows of one strip) whose operand loads are in flight while one is being
+  // multiplied, plus that one: a ring of register sets.  An item is a few loads and a few MFMAs,
+  // so a wavefront's rate is (items in flight) / (memory latency).
+  static constexpr int kDepth = (STAGED || sizeof(T) == 4) ? 3 : 2;
   static constexpr bool k16 = sizeof(T) == 2;
-  // 16-bit types: a wavefront's own staging area, 16 rows of X (32 columns) and of dY (TBN
-  // columns) per group; the list is kept shorter to make room for it next to the window
-  static constexpr int kStageX = 16 * 32, kStageElems = STAGED ? kStageX + 16 * TBN : 8;
+  // staged: a wavefront's own staging area, one group of rows of X (32 columns) and of dY (TBN
+  // columns), 3 KB; the list is kept shorter to make room for it next to the window
+  static constexpr int VEC = Tr::kVec;                   // elements of a 16-byte piece
+  static constexpr int kStageX = kGroupRows * 32, kStageElems = STAGED ? kStageX + kGroupRows * TBN : 8;
   static constexpr int kList = STAGED ? 960 : kThreads * kStrips;   // capacity of the list of strips found
-  static_assert(!STAGED || TBN == 64, "the staged dY rows are swizzled as two 64-byte chunks");
+  static_assert(!STAGED || TBN == 64, "the staged dY rows are swizzled as two halves");
+  static_assert(!STAGED || (64 * VEC == kGroupRows * 32), "one piece of X and two of dY per lane and group");
 
   struct Smem {
     int list[kList];              // strips found in this pass (tile id * kStrips + strip), ascending
@@ -142,11 +148,11 @@ struct WindowKernel {
       for (int b = 0; b < BJ; b++)
 #pragma unroll
         for (int e = 0; e < 16; e++) acc[a][b][e] = 0.f;
-    // two register sets: the fragments of the next group are loaded while this one is multiplied
-    Frag fa[2][GS][BI], fb[2][GS][BJ];
+    // kDepth register sets: the fragments of the next groups are loaded while this one is multiplied
+    Frag fa[kDepth][GS][BI], fb[kDepth][GS][BJ];
     // 16-bit staged path: the raw 16-byte pieces instead (one of X, two of dY per lane and group)
-    u32x4_t px[2], py[2][2];
-    bool okx[2], oky[2][2];
+    u32x4_t px[kDepth], py[kDepth][2];
+    bool okx[kDepth], oky[kDepth][2];
 
     // Listing the strips that meet the window, in ascending (tile, strip) order.  The tile ids of
     // a range [lo, hi) are dealt to the wavefronts in contiguous chunks; every wavefront first
@@ -241,10 +247,16 @@ struct WindowKernel {
       const int my_tiles = found > wave ? (found - wave + kWaves - 1) / kWaves : 0;
       const int items = my_tiles * ngroups;
       int ft = 0, fg = 0;      // tile ordinal and group of the next item to load
+      // The loads of an item are issued unconditionally, in straight-line code: the compiler
+      // counts outstanding loads along every path, and a fetch under a branch would make it wait
+      // for ALL loads at the first use behind the join — the item just requested included.
+      // Beyond the wavefront's last item the last strip is fetched again (valid addresses, in
+      // cache; what arrives is multiplied into accumulators that nobody reads any more).
       auto fetch_next = [&](auto set) {
         constexpr int S = decltype(set)::value;
-        if (ft < my_tiles) {
-          const int v = __builtin_amdgcn_readfirstlane(sm.list[wave + ft * kWaves]);
+        {
+          const int ftc = ft < my_tiles ? ft : my_tiles - 1;
+          const int v = __builtin_amdgcn_readfirstlane(sm.list[wave + ftc * kWaves]);
           const int id = v / kStrips, strip = v % kStrips;
           const int tk = id / p.tiles_n, tn = id - tk * p.tiles_n;
           const int k0 = tk * TBK + strip * 32;              // the strip's first row of W
@@ -255,10 +267,12 @@ struct WindowKernel {
           const T* rows_y = gdY + (int64_t)m0 * p.lddy + (int64_t)tn * TBN;
           if constexpr (STAGED) {
             {
-              // X: lane -> row lane / 4, piece lane % 4; dY: rows lane / 8 and + 8, piece lane % 8.
-              // A piece outside the matrix is fetched from inside it and replaced by zero later.
+              // X: 32 / VEC pieces per row, the 64 lanes cover the group's rows; dY: TBN / VEC pieces per
+              // row, two passes.  (16-bit: X row lane / 4, piece lane % 4; dY rows lane / 8 and + 8, piece
+              // lane % 8.)  A piece outside the matrix is fetched from inside it and replaced by zero later.
+              constexpr int PX = 32 / VEC, PY = TBN / VEC;
               {
-                const int r = lane >> 2, c = (lane & 3) * 8;
+                const int r = lane / PX, c = (lane % PX) * VEC;
                 const bool ok = m0 + r < p.M && k0 + c < p.K;
                 const T* src = ok ? gX + (int64_t)(m0 + r) * p.ldx + (k0 + c) : gX + (int64_t)m0 * p.ldx;
                 __builtin_memcpy(&px[S], src, 16);
@@ -266,7 +280,7 @@ struct WindowKernel {
               }
 #pragma unroll
               for (int q = 0; q < 2; q++) {
-                const int r = (lane >> 3) + 8 * q, c = (lane & 7) * 8;
+                const int r = lane / PY + (64 / PY) * q, c = (lane % PY) * VEC;
                 const bool ok = m0 + r < p.M && tn * TBN + c < p.N;
                 const T* src = ok ? rows_y + (int64_t)r * p.lddy + c : gdY + (int64_t)m0 * p.lddy;
                 __builtin_memcpy(&py[S][q], src, 16);
@@ -373,42 +387,67 @@ struct WindowKernel {
       int pt = 0, pg = 0;      // tile ordinal and group of the item being multiplied
       auto item = [&](auto set) {
         constexpr int S = decltype(set)::value;
-        fetch_next(std::integral_constant<int, S ^ 1>{});   // the next item's loads fly meanwhile
+        // the set freed by the previous item takes the loads of the item kDepth - 1 ahead
+        fetch_next(std::integral_constant<int, (S + kDepth - 1) % kDepth>{});
         if constexpr (STAGED) {
           {
             // pieces -> this wavefront's staging area (LDS operations of one wavefront are carried
             // out in order, so neither the reads below nor the next group's writes need a barrier)
             T* st = sm.stage[wave];
             const u32x4_t z = {0u, 0u, 0u, 0u};
-            *reinterpret_cast<u32x4_t*>(st + (lane >> 2) * 32 + (lane & 3) * 8) = okx[S] ? px[S] : z;
+            constexpr int PX = 32 / VEC, PY = TBN / VEC;
+            *reinterpret_cast<u32x4_t*>(st + (lane / PX) * 32 + (lane % PX) * VEC) = okx[S] ? px[S] : z;
+            if constexpr (k16) {
 #pragma unroll
-            for (int q = 0; q < 2; q++) {
-              const int r = (lane >> 3) + 8 * q, pc = lane & 7;
-              // dY rows are two 64-byte chunks, swapped in every other pair of rows, so that the four
-              // rows of a transpose read fall on different banks
-              *reinterpret_cast<u32x4_t*>(st + kStageX + r * TBN + ((((pc >> 2) ^ ((r >> 1) & 1)) << 5) | ((pc & 3) << 3))) =
-                  oky[S][q] ? py[S][q] : z;
+              for (int q = 0; q < 2; q++) {
+                const int r = (lane >> 3) + 8 * q, pc = lane & 7;
+                // dY rows are two 64-byte chunks, swapped in every other pair of rows, so that the four
+                // rows of a transpose read fall on different banks
+                *reinterpret_cast<u32x4_t*>(st + kStageX + r * TBN + ((((pc >> 2) ^ ((r >> 1) & 1)) << 5) | ((pc & 3) << 3))) =
+                    oky[S][q] ? py[S][q] : z;
+              }
+              // fragments by the LDS transpose read: within 16 lanes, lane c receives column c of a
+              // 4 x 16 block whose rows the lanes address four-per-row
+              typedef s16x4_t __attribute__((address_space(3))) * lds_s16x4_ptr;
+              const int g = lane >> 4, jl = lane & 15;
+              const int row = 8 * (g >> 1) + (jl >> 2), col = 16 * (g & 1) + 4 * (jl & 3);
+              auto tr_frag = [&](const T* at, int pitch) -> Frag {
+                const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(at));
+                const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(at + 4 * pitch));
+                const u32x2_t l2 = __builtin_bit_cast(u32x2_t, lo), h2 = __builtin_bit_cast(u32x2_t, hi);
+                u32x4_t f = {l2[0], l2[1], h2[0], h2[1]};
+                return f;
+              };
+              const Frag a = tr_frag(st + row * 32 + col, 32);
+              Frag b[BJ];
+#pragma unroll
+              for (int j = 0; j < BJ; j++)
+                b[j] = tr_frag(st + kStageX + row * TBN + (((j ^ ((row >> 1) & 1)) << 5) | col), TBN);
+#pragma unroll
+              for (int j = 0; j < BJ; j++) acc[0][j] = Mfma<T>::run(a, b[j], acc[0][j]);
+            } else {
+              // fp32: the two 128-byte halves of a dY row are swapped in every other row, so that the
+              // two rows of an MFMA step (lanes 0-31 and 32-63) lie on different banks
+#pragma unroll
+              for (int q = 0; q < 2; q++) {
+                const int r = lane / PY + (64 / PY) * q, c = (lane % PY) * VEC;
+                *reinterpret_cast<u32x4_t*>(st + kStageX + r * TBN + (c ^ ((r & 1) << 5))) = oky[S][q] ? py[S][q] : z;
+              }
+              // fragments: lane l holds row 2 s + (l >> 5), column l & 31 of the block
+              const int mg = lane >> 5, cl = lane & 31;
+              Frag a[GS], b[GS][BJ];
+#pragma unroll
+              for (int g = 0; g < GS; g++) {
+                a[g] = st[(2 * g + mg) * 32 + cl];
+#pragma unroll
+                for (int j = 0; j < BJ; j++) b[g][j] = st[kStageX + (2 * g + mg) * TBN + (((j ^ mg) << 5) | cl)];
+              }
+#pragma unroll
+              for (int g = 0; g < GS; g++)
+#pragma unroll
+                for (int j = 0; j < BJ; j++) acc[0][j] = Mfma<T>::run(a[g], b[g][j], acc[0][j]);
             }
-            // fragments by the LDS transpose read: within 16 lanes, lane c receives column c of a
-            // 4 x 16 block whose rows the lanes address four-per-row
-            typedef s16x4_t __attribute__((address_space(3))) * lds_s16x4_ptr;
-            const int g = lane >> 4, jl = lane & 15;
-            const int row = 8 * (g >> 1) + (jl >> 2), col = 16 * (g & 1) + 4 * (jl & 3);
-            auto tr_frag = [&](const T* at, int pitch) -> Frag {
-              const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(at));
-              const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(at + 4 * pitch));
-              const u32x2_t l2 = __builtin_bit_cast(u32x2_t, lo), h2 = __builtin_bit_cast(u32x2_t, hi);
-              u32x4_t f = {l2[0], l2[1], h2[0], h2[1]};
-              return f;
-            };
-            const Frag a = tr_frag(st + row * 32 + col, 32);
-            Frag b[BJ];
-#pragma unroll
-            for (int j = 0; j < BJ; j++)
-              b[j] = tr_frag(st + kStageX + row * TBN + (((j ^ ((row >> 1) & 1)) << 5) | col), TBN);
-#pragma unroll
-            for (int j = 0; j < BJ; j++) acc[0][j] = Mfma<T>::run(a, b[j], acc[0][j]);
-            if (++pg == ngroups) {
+            if (pt < my_tiles && ++pg == ngroups) {
               add_tile(wave + pt * kWaves);
               pg = 0;
               pt++;
@@ -422,16 +461,31 @@ struct WindowKernel {
           for (int a = 0; a < BI; a++)
 #pragma unroll
             for (int b = 0; b < BJ; b++) acc[a][b] = Mfma<T>::run(fa[S][s][a], fb[S][s][b], acc[a][b]);
-        if (++pg == ngroups) {
+        if (pt < my_tiles && ++pg == ngroups) {
           add_tile(wave + pt * kWaves);
           pg = 0;
           pt++;
         }
       };
-      fetch_next(std::integral_constant<int, 0>{});
-      for (int i = 0; i < items; i += 2) {
-        item(std::integral_constant<int, 0>{});
-        if (i + 1 < items) item(std::integral_constant<int, 1>{});
+      if (my_tiles > 0) {
+        // whole turns of the ring: the up to kDepth - 1 items past the end are padding (see fetch_next)
+        static_assert(kDepth >= 2 && kDepth <= 4, "the ring below is written out for up to four sets");
+        fetch_next(std::integral_constant<int, 0>{});
+        if constexpr (kDepth > 2) fetch_next(std::integral_constant<int, 1>{});
+        if constexpr (kDepth > 3) fetch_next(std::integral_constant<int, 2>{});
+        for (int i = 0; i < items; i += kDepth) {
+          item(std::integral_constant<int, 0>{});
+          item(std::integral_constant<int, 1>{});
+          if constexpr (kDepth > 2) item(std::integral_constant<int, 2>{});
+          if constexpr (kDepth > 3) item(std::integral_constant<int, 3>{});
+        }
+        // (the padding items have left rubbish in the accumulators)
+#pragma unroll
+        for (int a = 0; a < BI; a++)
+#pragma unroll
+          for (int b = 0; b < BJ; b++)
+#pragma unroll
+            for (int e = 0; e < 16; e++) acc[a][b][e] = 0.f;
       }
       __syncthreads();   // every strip of the list has been added
     }
