@@ -121,9 +121,21 @@ def make_workload(torch, _lib, name, dname, dev):
         _lib.check(lib.rz_input_grad_ws(dy.data_ptr(), hw.data_ptr(), dx.data_ptr(), iws.data_ptr(), iws_bytes,
                                         M, K, N, H, BK, BN, R, 1.0, N, K, code, stream))
 
+    # A hashed_weight too large for an LDS image: the layer's plan (tile offsets and window lists, a
+    # function of the layer's constants alone, built once like the hash constants themselves and
+    # kept on the device) goes with every call, as the package's own launchers do it.
+    plan = None
+    if _lib.plan_query(2, M, K, N, H, BK, BN, code)["mode"] in ("window", "fold"):
+        plan = _lib.layer_plan(K, N, H, BK, BN, R, 2, dev)
+
     def wgrad():
-        _lib.check(lib.rz_weight_grad(x.data_ptr(), dy.data_ptr(), dhw.data_ptr(), ws.data_ptr(), ws_bytes,
-                                      M, K, N, H, BK, BN, R, 1.0, K, N, code, stream))
+        if plan is not None:
+            _lib.check(lib.rz_weight_grad_planned(x.data_ptr(), dy.data_ptr(), dhw.data_ptr(), None, ws.data_ptr(), ws_bytes,
+                                                  plan.data_ptr(), plan.numel() * 4, M, K, N, H, BK, BN, R, 2, 1.0, K, N,
+                                                  code, 0, None, stream))
+        else:
+            _lib.check(lib.rz_weight_grad(x.data_ptr(), dy.data_ptr(), dhw.data_ptr(), ws.data_ptr(), ws_bytes,
+                                          M, K, N, H, BK, BN, R, 1.0, K, N, code, stream))
 
     # the dense products of the same shapes, each in the operand layout that is fastest for
     # the library (all "NN"), into pre-allocated outputs
@@ -137,7 +149,7 @@ def make_workload(torch, _lib, name, dname, dev):
                   ("input_grad", lambda: torch.matmul(dy, wt, out=dxd)),
                   ("weight_grad", lambda: torch.matmul(xt, dy, out=dwd)))
     wl = dict(M=M, K=K, N=N, H=H, BK=BK, BN=BN, R=R, code=code, dtype=dtype, dname=dname, x=x, hw=hw, dy=dy, y=y,
-              dx=dx, dhw=dhw, legs=(("forward", fwd), ("input_grad", igrad), ("weight_grad", wgrad)),
+              dx=dx, dhw=dhw, layer_plan=plan is not None, legs=(("forward", fwd), ("input_grad", igrad), ("weight_grad", wgrad)),
               dense_legs=dense_legs, flop_gemm=2.0 * M * N * K)
     return wl
 
@@ -353,7 +365,8 @@ def main():
         "data": "synthetic",
         "config": {"workload": "%s: M=%d K=%d N=%d H=%d BLOCK_K=%d BLOCK_N=%d %s, fwd + input-grad + weight-grad"
                                % (args.workload, M, K, N, H, BK, BN, dname),
-                   "hash_seed": 1024, "init_factor": 1.0},
+                   "hash_seed": 1024, "init_factor": 1.0,
+                   "weight_grad_layer_plan": bool(wl["layer_plan"])},
         "pct_mfma_peak": round(100.0 * value / peak, 2),
         "output_check": check,
         "roofline": roofline,

@@ -259,6 +259,32 @@ int rz_weight_grad_hashed(const void* X, const void* dY, void* dHW, void* dbias,
                           int64_t lddy, int dtype, unsigned flags, const rz_tuning* tuning, void* stream);
 
 /*
+ * Layer plan: the part of a weight-grad call that depends only on the layer — K, N, H, the tile
+ * and the hash constants — and not on the batch: where every W tile starts in hashed_weight and,
+ * for every window of dHW that the window kernel works on, the ordered list of tile strips that
+ * land in it.  Without a plan every weight-grad call on a large hashed_weight hashes the tile
+ * offsets again and every workgroup searches them for its strips (some 25 us of an 85 us call at
+ * M = 32, K = N = 10240); with one it reads its list.  The result is the same bit for bit.
+ *   rz_layer_plan_bytes   size of the plan (0: bad arguments)
+ *   rz_layer_plan_build   fills plan_host[plan_bytes] on the HOST (no device is touched); the
+ *                         caller copies it to device memory once and keeps it with the layer
+ *   rz_weight_grad_planned  rz_weight_grad_hashed with that device copy; the workspace is asked
+ *                         for as for rz_weight_grad_hashed (never more is needed).  The plan must
+ *                         have been built for the same K, N, H, BK, BN, R and hash_levels: the
+ *                         size is checked, the contents cannot be from the host.
+ * No counterpart in the reference, whose kernels hash every tile offset on every call
+ * (impl/RzLinearBackward.py:369).
+ */
+size_t rz_layer_plan_bytes(int K, int N, int H, int BK, int BN);
+int rz_layer_plan_build(void* plan_host, size_t plan_bytes, int K, int N, int H, int BK, int BN,
+                        const int32_t R[8], int hash_levels);
+int rz_weight_grad_planned(const void* X, const void* dY, void* dHW, void* dbias, void* workspace,
+                           size_t workspace_bytes, const void* layer_plan, size_t layer_plan_bytes, int M,
+                           int K, int N, int H, int BK, int BN, const int32_t R[8], int hash_levels,
+                           float init_factor, int64_t ldx, int64_t lddy, int dtype, unsigned flags,
+                           const rz_tuning* tuning, void* stream);
+
+/*
  * How a call would be carried out (host-side, touches no device): which C tile, how many
  * slices of the contracted dimension and how long each, which kernel form.  op: 0 = forward,
  * 1 = input-grad, 2 = weight-grad (flags / with_dbias as for rz_weight_grad_hashed, else 0).

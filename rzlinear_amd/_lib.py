@@ -23,6 +23,7 @@ EXPORTS = (
     "rz_weight_grad_ex", "rz_forward_hashed", "rz_input_grad_hashed", "rz_weight_grad_hashed", "rz_materialize",
     "rz_forward_hashed_workspace_bytes", "rz_input_grad_hashed_workspace_bytes",
     "rz_weight_grad_hashed_workspace_bytes", "rz_plan_query", "rz_weight_grad_static",
+    "rz_layer_plan_bytes", "rz_layer_plan_build", "rz_weight_grad_planned",
     "rz_sgd_step", "rz_adam_step",
 )
 
@@ -140,6 +141,14 @@ def load():
     lib.rz_input_grad_hashed_workspace_bytes.argtypes = [c_int] * 7 + [tun]
     lib.rz_weight_grad_hashed_workspace_bytes.restype = c_sz
     lib.rz_weight_grad_hashed_workspace_bytes.argtypes = [c_int] * 7 + [ctypes.c_uint, c_int, tun]
+    lib.rz_layer_plan_bytes.restype = c_sz
+    lib.rz_layer_plan_bytes.argtypes = [c_int] * 5
+    lib.rz_layer_plan_build.restype = c_int
+    lib.rz_layer_plan_build.argtypes = [c_vp, c_sz, c_int, c_int, c_int, c_int, c_int, i32p, c_int]
+    lib.rz_weight_grad_planned.restype = c_int
+    lib.rz_weight_grad_planned.argtypes = [c_vp, c_vp, c_vp, c_vp, c_vp, c_sz, c_vp, c_sz, c_int, c_int, c_int,
+                                           c_int, c_int, c_int, i32p, c_int, c_f, c_i64, c_i64, c_int,
+                                           ctypes.c_uint, tun, c_vp]
     lib.rz_plan_query.restype = c_int
     lib.rz_plan_query.argtypes = [c_int] * 8 + [ctypes.c_uint, c_int, tun, i32p]
     f32p = c_vp
@@ -211,6 +220,29 @@ def tile_offsets(K, N, H, BLOCK_SIZE_K, BLOCK_SIZE_N, random_numbers, hash_level
     check(lib.rz_tile_offsets(ctypes.cast(out.data_ptr(), ctypes.POINTER(ctypes.c_int32)), K, N, H,
                               BLOCK_SIZE_K, BLOCK_SIZE_N, R, hash_levels))
     return out
+
+
+_layer_plans = {}
+# Whether the weight-grad launchers take a layer plan where one helps (tests switch it off to reach
+# the kernels' own search for their strips).
+use_layer_plans = True
+
+
+def layer_plan(K, N, H, BK, BN, R, hash_levels, device):
+    """The layer plan (rz_layer_plan_build) for these layer constants as an int32 tensor on `device`,
+    built on the host the first time it is asked for and kept for the life of the process (it depends
+    on the layer alone: shapes, tile and hash constants; about 10 bytes per W tile strip)."""
+    key = (K, N, H, BK, BN, tuple(int(v) for v in R), int(hash_levels), str(device))
+    plan = _layer_plans.get(key)
+    if plan is None:
+        lib = load()
+        nbytes = lib.rz_layer_plan_bytes(K, N, H, BK, BN)
+        if nbytes == 0:
+            raise ValueError("no layer plan for K=%d N=%d H=%d tile %dx%d" % (K, N, H, BK, BN))
+        host = torch.empty((nbytes // 4,), dtype=torch.int32)
+        check(lib.rz_layer_plan_build(host.data_ptr(), nbytes, K, N, H, BK, BN, R, hash_levels))
+        plan = _layer_plans[key] = host.to(device)
+    return plan
 
 
 PLAN_MODES = {0: "store", 1: "split", 2: "lds_image", 3: "atomics", 4: "window", 5: "fold"}

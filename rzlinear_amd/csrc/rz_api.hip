@@ -342,9 +342,9 @@ struct WeightGradWorkspace {
   size_t main_bytes, total_bytes;
 };
 static WeightGradWorkspace weight_grad_workspace(const WeightGradPlan& plan, const WindowPlan& window, int H,
-                                                 bool dhw_f32, bool with_dbias) {
+                                                 bool dhw_f32, bool with_dbias, bool planned = false) {
   WeightGradWorkspace w;
-  if (window.use) w.main_bytes = round256((size_t)window.tiles * sizeof(int32_t));  // tile offsets
+  if (window.use) w.main_bytes = planned ? 0 : round256((size_t)window.tiles * sizeof(int32_t));  // tile offsets
   else if (plan.image_pitch > 0 || plan.fold.use) w.main_bytes = plan.workspace_bytes;
   else w.main_bytes = dhw_f32 ? 0 : round256((size_t)H * sizeof(float));
   // (the window kernel does not stage dY by tile columns: its bias gradient is a pass of its own)
@@ -357,7 +357,8 @@ static int weight_grad_impl(const void* X, const void* dY, void* dHW, void* dbia
                             size_t workspace_bytes, int M, int K, int N, int H, int BK, int BN,
                             const int32_t R[8], float init_factor, int64_t ldx, int64_t lddy, int dtype,
                             unsigned flags, void* stream, int hash_levels = RZ_HASH_TWO_LEVEL,
-                            const rz_tuning* tuning_arg = nullptr) {
+                            const rz_tuning* tuning_arg = nullptr, const int32_t* layer_plan = nullptr,
+                            size_t layer_plan_bytes = 0) {
   if (X == nullptr || dY == nullptr || dHW == nullptr) return RZ_ERR_NULL_POINTER;
   if (dtype_bytes(dtype) == 0) return RZ_ERR_BAD_DTYPE;
   if (M < 1 || ldx < K || lddy < N) return RZ_ERR_BAD_SHAPE;
@@ -371,9 +372,17 @@ static int weight_grad_impl(const void* X, const void* dY, void* dHW, void* dbia
   const int dhw_dtype = (flags & RZ_WG_DHW_F32) ? RZ_F32 : dtype;
   const int dbias_dtype = (flags & RZ_WG_DBIAS_F32) ? RZ_F32 : dtype;
   const WeightGradPlan plan = plan_weight_grad(M, K, N, H, BK, BN, dtype_bytes(dtype), tuning);
+  // a layer plan (device memory, built for exactly this K, N, H, tile and hash) replaces the
+  // per-call hashing of the tile offsets and the window kernel's search for its strips
+  const bool planned = layer_plan != nullptr;
+  LayerPlanLayout lay = {};
+  if (planned) {
+    lay = layer_plan_layout(K, N, H, BK, BN);
+    if (!lay.ok || layer_plan_bytes != lay.words * sizeof(int32_t)) return RZ_ERR_BAD_ARGUMENT;
+  }
   WindowPlan wp = {};
-  if (!plan.lds_image()) wp = plan_window(M, K, N, H, BK, BN, dtype_bytes(dtype), tuning, plan);
-  const WeightGradWorkspace ws = weight_grad_workspace(plan, wp, H, dhw_dtype == RZ_F32, dbias != nullptr);
+  if (!plan.lds_image()) wp = plan_window(M, K, N, H, BK, BN, dtype_bytes(dtype), tuning, plan, planned && lay.windows > 0);
+  const WeightGradWorkspace ws = weight_grad_workspace(plan, wp, H, dhw_dtype == RZ_F32, dbias != nullptr, planned);
   if (ws.total_bytes > 0 && (workspace == nullptr || workspace_bytes < ws.total_bytes)) return RZ_ERR_WORKSPACE;
   hipStream_t s = (hipStream_t)stream;
   p.A = X;
@@ -389,12 +398,21 @@ static int weight_grad_impl(const void* X, const void* dY, void* dHW, void* dbia
     // large hashed_weight, short contraction: windows of dHW instead of K*N atomics.  The
     // tile offsets are hashed once into the workspace; every workgroup scans them.
     {
-      const int TK = (K + BK - 1) / BK, TN = (N + BN - 1) / BN;
-      hipLaunchKernelGGL(tile_offsets_kernel, dim3((TK * TN + 255) / 256), dim3(256), 0, s, (int32_t*)workspace,
-                         TK, TN, p.h);
-      if (hipGetLastError() != hipSuccess) return RZ_ERR_LAUNCH;
       WindowParams w = {};
-      w.offsets = (const int32_t*)workspace;
+      if (planned) {
+        if (lay.windows != wp.windows || lay.window != wp.window) return RZ_ERR_BAD_ARGUMENT;
+        w.offsets = layer_plan + lay.offsets_at;
+        w.plan_start = layer_plan + lay.start_at;
+        w.plan_list = layer_plan + lay.list_at;
+        w.plan_offs = layer_plan + lay.offs_at;
+        w.plan_header = layer_plan;
+      } else {
+        const int TK = (K + BK - 1) / BK, TN = (N + BN - 1) / BN;
+        hipLaunchKernelGGL(tile_offsets_kernel, dim3((TK * TN + 255) / 256), dim3(256), 0, s, (int32_t*)workspace,
+                           TK, TN, p.h);
+        if (hipGetLastError() != hipSuccess) return RZ_ERR_LAUNCH;
+        w.offsets = (const int32_t*)workspace;
+      }
       w.X = X; w.dY = dY; w.dHW = dHW;
       w.M = M; w.K = K; w.N = N; w.H = H;
       w.ldx = ldx; w.lddy = lddy;
@@ -428,11 +446,15 @@ static int weight_grad_impl(const void* X, const void* dY, void* dHW, void* dbia
     if (launch_gemm(dtype, kWeightGrad, p, &plan, nullptr, tuning, s) != hipSuccess) return RZ_ERR_LAUNCH;
     FoldParams fp;
     fp.tiles = p.tiles_out;
-    int32_t* offsets = (int32_t*)((char*)workspace + f.tiles_bytes + f.partial_bytes);
-    hipLaunchKernelGGL(tile_offsets_kernel, dim3((p.out_tiles_k * p.out_tiles_n + 255) / 256), dim3(256), 0, s, offsets,
-                       p.out_tiles_k, p.out_tiles_n, p.h);
-    if (hipGetLastError() != hipSuccess) return RZ_ERR_LAUNCH;
-    fp.offsets = offsets;
+    if (planned) {
+      fp.offsets = layer_plan + lay.offsets_at;
+    } else {
+      int32_t* offsets = (int32_t*)((char*)workspace + f.tiles_bytes + f.partial_bytes);
+      hipLaunchKernelGGL(tile_offsets_kernel, dim3((p.out_tiles_k * p.out_tiles_n + 255) / 256), dim3(256), 0, s, offsets,
+                         p.out_tiles_k, p.out_tiles_n, p.h);
+      if (hipGetLastError() != hipSuccess) return RZ_ERR_LAUNCH;
+      fp.offsets = offsets;
+    }
     fp.partial = f.shares > 1 ? (float*)((char*)workspace + f.tiles_bytes) : nullptr;
     fp.out = dHW;
     fp.out_dtype = dhw_dtype;
@@ -757,6 +779,71 @@ RZ_API int rz_weight_grad_hashed(const void* X, const void* dY, void* dHW, void*
                                  int64_t lddy, int dtype, unsigned flags, const rz_tuning* tuning, void* stream) {
   return weight_grad_impl(X, dY, dHW, dbias, workspace, workspace_bytes, M, K, N, H, BK, BN, R,
                           init_factor, ldx, lddy, dtype, flags, stream, hash_levels, tuning);
+}
+
+RZ_API size_t rz_layer_plan_bytes(int K, int N, int H, int BK, int BN) {
+  if (K < 1 || N < 1 || H < 1 || check_tile(BK, BN) != RZ_OK || (long long)H <= (long long)BK * BN) return 0;
+  const LayerPlanLayout l = layer_plan_layout(K, N, H, BK, BN);
+  return l.ok ? l.words * sizeof(int32_t) : 0;
+}
+
+RZ_API int rz_layer_plan_build(void* plan_host, size_t plan_bytes, int K, int N, int H, int BK, int BN,
+                               const int32_t R[8], int hash_levels) {
+  if (plan_host == nullptr) return RZ_ERR_NULL_POINTER;
+  HashParams h;
+  int st = make_hash(&h, K, N, H, BK, BN, R, hash_levels);
+  if (st != RZ_OK) return st;
+  const LayerPlanLayout l = layer_plan_layout(K, N, H, BK, BN);
+  if (!l.ok || plan_bytes != l.words * sizeof(int32_t)) return RZ_ERR_BAD_ARGUMENT;
+  int32_t* w = static_cast<int32_t*>(plan_host);
+  for (size_t i = 0; i < l.words; i++) w[i] = 0;
+  const int TK = (K + BK - 1) / BK, TN = (N + BN - 1) / BN;
+  int32_t* offsets = w + l.offsets_at;
+  for (int tk = 0; tk < TK; tk++)
+    for (int tn = 0; tn < TN; tn++) offsets[(size_t)tk * TN + tn] = (int32_t)tile_offset(h, (uint32_t)tk, (uint32_t)tn);
+  long long entries = 0;
+  if (l.windows > 0) {
+    // counting sort of (window, strip) pairs by window; visiting the strips in ascending order
+    // keeps every window's list ascending, which is the order the kernel's own search produces
+    int32_t* start = w + l.start_at;
+    int32_t* list = w + l.list_at;
+    int32_t* offs = w + l.offs_at;
+    auto for_each_pair = [&](auto&& f) {
+      for (int id = 0; id < l.tiles; id++)
+        for (int sidx = 0; sidx < l.strips_per_tile; sidx++) {
+          const long long so = (long long)offsets[id] + (long long)sidx * l.strip_elems;
+          const long long first = so / l.window, last = (so + l.strip_elems - 1) / l.window;
+          for (long long b = first; b <= last && b < l.windows; b++) f((int)b, id * l.strips_per_tile + sidx, (int32_t)so);
+        }
+    };
+    for_each_pair([&](int b, int, int32_t) { start[b + 1]++; });
+    for (int b = 0; b < l.windows; b++) start[b + 1] += start[b];
+    entries = start[l.windows];
+    if (entries > l.capacity) return RZ_ERR_BAD_ARGUMENT;   // (cannot happen: see layer_plan_layout)
+    // (start[b] is advanced while the lists are filled and restored afterwards)
+    for_each_pair([&](int b, int strip, int32_t so) {
+      list[start[b]] = strip;
+      offs[start[b]] = so;
+      start[b]++;
+    });
+    for (int b = l.windows; b > 0; b--) start[b] = start[b - 1];
+    start[0] = 0;
+  }
+  const int32_t header[kLayerPlanHeader] = {kLayerPlanMagic, kLayerPlanVersion, K, N, H, BK, BN, hash_levels, l.tiles,
+                                            l.windows, l.window, (int32_t)entries, l.strips_per_tile, 0, 0, 0};
+  for (int i = 0; i < kLayerPlanHeader; i++) w[i] = header[i];
+  return RZ_OK;
+}
+
+RZ_API int rz_weight_grad_planned(const void* X, const void* dY, void* dHW, void* dbias, void* workspace,
+                                  size_t workspace_bytes, const void* layer_plan, size_t layer_plan_bytes, int M,
+                                  int K, int N, int H, int BK, int BN, const int32_t R[8], int hash_levels,
+                                  float init_factor, int64_t ldx, int64_t lddy, int dtype, unsigned flags,
+                                  const rz_tuning* tuning, void* stream) {
+  if (layer_plan == nullptr) return RZ_ERR_NULL_POINTER;
+  return weight_grad_impl(X, dY, dHW, dbias, workspace, workspace_bytes, M, K, N, H, BK, BN, R, init_factor, ldx,
+                          lddy, dtype, flags, stream, hash_levels, tuning, static_cast<const int32_t*>(layer_plan),
+                          layer_plan_bytes);
 }
 
 RZ_API int rz_plan_query(int op, int M, int K, int N, int H, int BK, int BN, int dtype, unsigned flags,

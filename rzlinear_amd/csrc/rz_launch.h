@@ -289,20 +289,29 @@ static constexpr int kWindowFloats = 25600;   // LDS floats a workgroup can hold
 
 static inline bool window_tile_supported(int BK, int BN) { return BN == 64 && (BK == 64 || BK == 32); }
 
-static inline WindowPlan plan_window(int M, int K, int N, int H, int BK, int BN, int elem_bytes, const rz_tuning& t,
-                                     const WeightGradPlan& other) {
-  WindowPlan pl = {false, 0, 0, 0};
-  if (t.window == -1 || !window_tile_supported(BK, BN)) return pl;
-  const long long tiles = (long long)((K + BK - 1) / BK) * ((N + BN - 1) / BN);
-  if (tiles > (1 << 20)) return pl;              // every workgroup scans every tile's offset
-  pl.tiles = tiles;
+// Size and number of the windows for a hashed_weight of H elements (a function of H alone: a
+// layer plan built once per layer holds the strip lists of exactly these windows).
+static inline void window_geometry(int H, int* window, int* windows) {
   // one workgroup per compute unit when the windows can be that large, else whole rounds
   const long long rounds = ((long long)H + (long long)kWindowFloats * kComputeUnits - 1) /
                            ((long long)kWindowFloats * kComputeUnits);
   long long w = (((long long)H + rounds * kComputeUnits - 1) / (rounds * kComputeUnits) + 3) & ~3LL;
   if (w < 1024) w = 1024;                        // tiny windows would each redo most tiles
-  pl.window = (int)w;
-  pl.windows = (int)(((long long)H + w - 1) / w);
+  *window = (int)w;
+  *windows = (int)(((long long)H + w - 1) / w);
+}
+
+// planned: the caller holds a layer plan, so the kernel neither hashes the tile offsets nor scans
+// them for its strips (some 25 us less, measured at K = N = 10240).
+static inline WindowPlan plan_window(int M, int K, int N, int H, int BK, int BN, int elem_bytes, const rz_tuning& t,
+                                     const WeightGradPlan& other, bool planned = false) {
+  WindowPlan pl = {false, 0, 0, 0};
+  if (t.window == -1 || !window_tile_supported(BK, BN)) return pl;
+  const long long tiles = (long long)((K + BK - 1) / BK) * ((N + BN - 1) / BN);
+  if (tiles > (1 << 20)) return pl;              // every workgroup scans every tile's offset
+  pl.tiles = tiles;
+  window_geometry(H, &pl.window, &pl.windows);
+  const long long w = pl.window;
   // Rough times in microseconds, fitted to measurements at K = N = 10240, H = 6.5 M on MI355X.
   // Scatter kernel: K*N atomics at about 184 G/s plus the product.  Window kernel: every
   // workgroup works through tiles * (window + tile) / H tiles; a tile costs about 0.27 us plus
@@ -311,12 +320,52 @@ static inline WindowPlan plan_window(int M, int K, int N, int H, int BK, int BN,
   const double chunks = (double)((M + 31) / 32);
   const double per_wg = (double)tiles * ((double)w + (double)BK * BN) / (double)H;
   const double wg_rounds = (double)((pl.windows + kComputeUnits - 1) / kComputeUnits);
-  const double t_window = wg_rounds * per_wg * (0.27 + (elem_bytes == 4 ? 0.80 : 0.22) * chunks) + 28.0;
+  const double t_window = wg_rounds * per_wg * (0.27 + (elem_bytes == 4 ? 0.80 : 0.22) * chunks) + (planned ? 5.0 : 28.0);
   // ... against what the contraction kernel's plan would take: the fold, or the atomic scatter
   const double t_scatter = 0.9 * (double)K * N / 184e3 + 2.0 * M * (double)K * N / 800e6;
   const double t_other = other.fold.use ? other.fold_us : t_scatter;
   pl.use = t.window == 1 || t_window * 1.1 < t_other;
   return pl;
+}
+
+// A layer plan: what the weight-grad of one layer needs of its hash and nothing else (it depends on
+// K, N, H, the tile and the hash constants, not on M, the element type or the data), computed once
+// on the host and kept by the caller in device memory.  int32 words:
+//   [0, 16)   header: magic, version, K, N, H, BK, BN, hash_levels, tiles, windows, window,
+//             entries, strips per tile, 0, 0, 0
+//   offsets   [tiles]           where every W tile starts in hashed_weight (index tk * tiles_n + tn)
+//   start     [windows + 1]     first entry of every window of the window kernel (window_geometry)
+//   list      [capacity]        the strips (tile * strips per tile + strip) that meet the window, ascending
+//   offs      [capacity]        ... and where each starts in hashed_weight
+// The lists exist for the tiles the window kernel supports (windows = 0 otherwise).
+static constexpr int32_t kLayerPlanMagic = 0x525a4c50, kLayerPlanVersion = 1;
+static constexpr int kLayerPlanHeader = 16;
+struct LayerPlanLayout {
+  bool ok;
+  int tiles, windows, window, strips_per_tile, strip_elems;
+  long long capacity;                 // list entries reserved (an upper bound of those used)
+  size_t offsets_at, start_at, list_at, offs_at, words;
+};
+static inline LayerPlanLayout layer_plan_layout(int K, int N, int H, int BK, int BN) {
+  LayerPlanLayout l = {};
+  const long long tiles = (long long)((K + BK - 1) / BK) * ((N + BN - 1) / BN);
+  if (tiles > (1 << 22)) return l;
+  l.tiles = (int)tiles;
+  auto round16 = [](size_t v) { return (v + 15) & ~(size_t)15; };
+  l.offsets_at = kLayerPlanHeader;
+  l.start_at = round16(l.offsets_at + (size_t)tiles);
+  if (window_tile_supported(BK, BN) && tiles <= (1 << 20)) {
+    window_geometry(H, &l.window, &l.windows);
+    l.strips_per_tile = BK / 32;
+    l.strip_elems = 32 * BN;
+    // a strip of strip_elems consecutive elements meets at most ceil(strip_elems / window) + 1 windows
+    l.capacity = tiles * l.strips_per_tile * ((l.strip_elems + l.window - 1) / l.window + 1);
+  }
+  l.list_at = round16(l.start_at + (size_t)l.windows + 1);
+  l.offs_at = round16(l.list_at + (size_t)l.capacity);
+  l.words = round16(l.offs_at + (size_t)l.capacity);
+  l.ok = l.words < (1u << 30);
+  return l;
 }
 
 // Forward / input-grad with few C tiles and a long contraction (skinny batches): R is cut into

@@ -31,6 +31,13 @@ struct WindowParams {
   const void* dY;
   void* dHW;
   const int32_t* offsets;   // offset of every W tile, index tk * tiles_n + tn
+  // From a layer plan (null: every workgroup finds its strips by scanning `offsets`): the strips
+  // that meet window b are entries [plan_start[b], plan_start[b + 1]) of plan_list (tile *
+  // strips per tile + strip, ascending) and plan_offs (where each starts in hashed_weight).
+  const int32_t* plan_start;
+  const int32_t* plan_list;
+  const int32_t* plan_offs;
+  const int32_t* plan_header;   // K, N, H, BK, BN, window at words 2..6 and 10: checked against this call's
   int M, K, N, H;
   int64_t ldx, lddy;
   float scale;
@@ -173,68 +180,99 @@ struct WindowKernel {
       }
       return n;
     };
-    int lo = 0;
-    while (lo < total) {
-      int hi = total, found = 0, chunk = 0;
-      for (;;) {
-        chunk = (hi - lo + kWaves - 1) / kWaves;
-        const int begin = lo + wave * chunk, end = begin + chunk < hi ? begin + chunk : hi;
-        int mine = 0;
-        for (int id0 = begin; id0 < end; id0 += 64 * kBatch) {
-          // a lane's next kBatch offsets are loaded together (one memory latency, not kBatch)
-          int offv[kBatch];
-#pragma unroll
-          for (int u = 0; u < kBatch; u++) {
-            const int id = id0 + u * 64 + lane;
-            offv[u] = id < end ? p.offsets[id] : 0;
-          }
-#pragma unroll
-          for (int u = 0; u < kBatch; u++) {
-            const int id = id0 + u * 64 + lane;
-            unsigned long long mask[kStrips];
-            mine += strips_of(id < end ? id : -1, offv[u], mask);
-          }
+    const bool planned = p.plan_start != nullptr;   // (uniform)
+    if (planned) {
+      // A plan built for another layer would send the loads below anywhere: refuse it, loudly
+      // (the window of dHW becomes NaN), instead of reading outside X and dY.
+      const int32_t* hd = p.plan_header;
+      if (hd[2] != p.K || hd[3] != p.N || hd[4] != p.H || hd[5] != TBK || hd[6] != TBN || hd[10] != p.window ||
+          hd[12] != kStrips) {
+        const float nan = __builtin_nanf("");
+        if (p.out_f32 || sizeof(T) == 4) {
+          for (int i = tid; i < wlen; i += kThreads) (static_cast<float*>(p.dHW) + w0)[i] = nan;
+        } else {
+          for (int i = tid; i < wlen; i += kThreads) (static_cast<T*>(p.dHW) + w0)[i] = Tr::from_float(nan);
         }
-        __syncthreads();   // (the counts of the previous attempt or round have been read)
-        if (lane == 0) sm.count[0][wave] = mine;
-        __syncthreads();
-        found = 0;
-#pragma unroll
-        for (int w = 0; w < kWaves; w++) found += __builtin_amdgcn_readfirstlane(sm.count[0][w]);
-        if (found <= kList) break;
-        hi = lo + (hi - lo) / 2;   // (found > kList >= kStrips, so the range holds at least two tiles)
+        return;
       }
-      {
-        int at = 0;
-#pragma unroll
-        for (int w = 0; w < kWaves; w++) at += (w < wave) ? __builtin_amdgcn_readfirstlane(sm.count[0][w]) : 0;
-        const int begin = lo + wave * chunk, end = begin + chunk < hi ? begin + chunk : hi;
-        for (int id0 = begin; id0 < end; id0 += 64 * kBatch) {
-          int offv[kBatch];
-#pragma unroll
-          for (int u = 0; u < kBatch; u++) {
-            const int id = id0 + u * 64 + lane;
-            offv[u] = id < end ? p.offsets[id] : 0;
-          }
-#pragma unroll
-          for (int u = 0; u < kBatch; u++) {
-            const int id = id0 + u * 64 + lane;
-            unsigned long long mask[kStrips];
-            const int n = strips_of(id < end ? id : -1, offv[u], mask);
-            // the strips of the lanes below me, then my own in order
-            int mine = at;
-#pragma unroll
-            for (int s = 0; s < kStrips; s++) mine += __popcll(mask[s] & ((1ull << lane) - 1ull));
-#pragma unroll
-            for (int s = 0; s < kStrips; s++) {
-              if ((mask[s] >> lane) & 1ull) {
-                sm.list[mine] = id * kStrips + s;
-                sm.offs[mine] = offv[u] + s * kStripElems;
-                sm.done[mine] = 0;
-                mine++;
-              }
+    }
+    const int plan_lo = planned ? p.plan_start[blockIdx.x] : 0;
+    const int plan_n = planned ? p.plan_start[blockIdx.x + 1] - plan_lo : 0;
+    const int list_total = planned ? plan_n : total;   // what the rounds below work through: entries, or tile ids
+    int lo = 0;
+    while (lo < list_total) {
+      int hi = total, found = 0, chunk = 0;
+      if (planned) {
+        // the next kList entries of this window's precomputed list (same order as the scan finds them)
+        found = plan_n - lo < kList ? plan_n - lo : kList;
+        __syncthreads();   // (the previous round's list is no longer read)
+        for (int i = tid; i < found; i += kThreads) {
+          sm.list[i] = p.plan_list[plan_lo + lo + i];
+          sm.offs[i] = p.plan_offs[plan_lo + lo + i];
+          sm.done[i] = 0;
+        }
+        hi = lo + found;
+      } else {
+        for (;;) {
+          chunk = (hi - lo + kWaves - 1) / kWaves;
+          const int begin = lo + wave * chunk, end = begin + chunk < hi ? begin + chunk : hi;
+          int mine = 0;
+          for (int id0 = begin; id0 < end; id0 += 64 * kBatch) {
+            // a lane's next kBatch offsets are loaded together (one memory latency, not kBatch)
+            int offv[kBatch];
+  #pragma unroll
+            for (int u = 0; u < kBatch; u++) {
+              const int id = id0 + u * 64 + lane;
+              offv[u] = id < end ? p.offsets[id] : 0;
             }
-            at += n;
+  #pragma unroll
+            for (int u = 0; u < kBatch; u++) {
+              const int id = id0 + u * 64 + lane;
+              unsigned long long mask[kStrips];
+              mine += strips_of(id < end ? id : -1, offv[u], mask);
+            }
+          }
+          __syncthreads();   // (the counts of the previous attempt or round have been read)
+          if (lane == 0) sm.count[0][wave] = mine;
+          __syncthreads();
+          found = 0;
+  #pragma unroll
+          for (int w = 0; w < kWaves; w++) found += __builtin_amdgcn_readfirstlane(sm.count[0][w]);
+          if (found <= kList) break;
+          hi = lo + (hi - lo) / 2;   // (found > kList >= kStrips, so the range holds at least two tiles)
+        }
+        {
+          int at = 0;
+  #pragma unroll
+          for (int w = 0; w < kWaves; w++) at += (w < wave) ? __builtin_amdgcn_readfirstlane(sm.count[0][w]) : 0;
+          const int begin = lo + wave * chunk, end = begin + chunk < hi ? begin + chunk : hi;
+          for (int id0 = begin; id0 < end; id0 += 64 * kBatch) {
+            int offv[kBatch];
+  #pragma unroll
+            for (int u = 0; u < kBatch; u++) {
+              const int id = id0 + u * 64 + lane;
+              offv[u] = id < end ? p.offsets[id] : 0;
+            }
+  #pragma unroll
+            for (int u = 0; u < kBatch; u++) {
+              const int id = id0 + u * 64 + lane;
+              unsigned long long mask[kStrips];
+              const int n = strips_of(id < end ? id : -1, offv[u], mask);
+              // the strips of the lanes below me, then my own in order
+              int mine = at;
+  #pragma unroll
+              for (int s = 0; s < kStrips; s++) mine += __popcll(mask[s] & ((1ull << lane) - 1ull));
+  #pragma unroll
+              for (int s = 0; s < kStrips; s++) {
+                if ((mask[s] >> lane) & 1ull) {
+                  sm.list[mine] = id * kStrips + s;
+                  sm.offs[mine] = offv[u] + s * kStripElems;
+                  sm.done[mine] = 0;
+                  mine++;
+                }
+              }
+              at += n;
+            }
           }
         }
       }
@@ -337,20 +375,14 @@ struct WindowKernel {
 #pragma unroll
           for (int b = 0; b < BJ; b++) {
             float* at = win + rel + ((lane >> 5) * 4) * TBN + b * 32 + (lane & 31);
+            // (a block's sixteen reads go out together: one LDS round trip per block)
+            float cur[16];
 #pragma unroll
-            for (int half = 0; half < 2; half++) {
-              float cur[8];
+            for (int i = 0; i < 16; i++) cur[i] = at[((i >> 2) * 8 + (i & 3)) * TBN];
 #pragma unroll
-              for (int q = 0; q < 8; q++) {
-                const int i = half * 8 + q;
-                cur[q] = at[((i >> 2) * 8 + (i & 3)) * TBN];
-              }
-#pragma unroll
-              for (int q = 0; q < 8; q++) {
-                const int i = half * 8 + q;
-                at[((i >> 2) * 8 + (i & 3)) * TBN] = cur[q] + acc[0][b][i] * p.scale;
-                acc[0][b][i] = 0.f;
-              }
+            for (int i = 0; i < 16; i++) {
+              at[((i >> 2) * 8 + (i & 3)) * TBN] = cur[i] + acc[0][b][i] * p.scale;
+              acc[0][b][i] = 0.f;
             }
           }
         } else {

@@ -28,8 +28,15 @@ def rz_linear_backward_tl(input: torch.Tensor, hashed_weight: torch.Tensor, outp
 
 
 def weight_grad_hashed(input, output_grad, init_factor, M, K, N, H, R, BLOCK_SIZE_K, BLOCK_SIZE_N,
-                       out=None, accumulate=False, with_bias_grad=False, hash_levels=_lib.HASH_TWO_LEVEL):
-    """One rz_weight_grad_hashed call; returns (hashed_weight_grad, bias_grad or None)."""
+                       out=None, accumulate=False, with_bias_grad=False, hash_levels=_lib.HASH_TWO_LEVEL,
+                       use_layer_plan=None):
+    """One weight-grad call; returns (hashed_weight_grad, bias_grad or None).
+
+    Where the library would work by windows of dHW or fold stored tiles into dHW (a hashed_weight
+    too large for an image in LDS), the call goes through rz_weight_grad_planned with the layer's
+    plan, which _lib.layer_plan builds once per (K, N, H, tile, constants) and keeps on the device;
+    everything else, and use_layer_plan=False (default: _lib.use_layer_plans), goes through
+    rz_weight_grad_hashed."""
     stream = _lib.require_gpu(input, output_grad)
     if input.dtype != output_grad.dtype:
         raise TypeError("input is %s but output_grad is %s" % (input.dtype, output_grad.dtype))
@@ -61,10 +68,22 @@ def weight_grad_hashed(input, output_grad, init_factor, M, K, N, H, R, BLOCK_SIZ
     need = lib.rz_weight_grad_hashed_workspace_bytes(M, K, N, H, BLOCK_SIZE_K, BLOCK_SIZE_N, code, flags,
                                                      int(with_bias_grad), tuning)
     ws = _lib.workspace(need, output_grad.device)
-    _lib.check(lib.rz_weight_grad_hashed(
-        x.data_ptr(), dy.data_ptr(), out.data_ptr(), bias_grad.data_ptr() if with_bias_grad else None,
-        ws.data_ptr() if need else None, need, M, K, N, H, BLOCK_SIZE_K, BLOCK_SIZE_N, R, hash_levels,
-        float(init_factor), ldx, lddy, code, flags, tuning, stream))
+    plan = None
+    if use_layer_plan is None:
+        use_layer_plan = _lib.use_layer_plans
+    if use_layer_plan and _lib.plan_query(2, M, K, N, H, BLOCK_SIZE_K, BLOCK_SIZE_N, code, flags,
+                                          with_bias_grad)["mode"] in ("window", "fold"):
+        plan = _lib.layer_plan(K, N, H, BLOCK_SIZE_K, BLOCK_SIZE_N, R, hash_levels, output_grad.device)
+    if plan is not None:
+        _lib.check(lib.rz_weight_grad_planned(
+            x.data_ptr(), dy.data_ptr(), out.data_ptr(), bias_grad.data_ptr() if with_bias_grad else None,
+            ws.data_ptr() if need else None, need, plan.data_ptr(), plan.numel() * 4, M, K, N, H, BLOCK_SIZE_K,
+            BLOCK_SIZE_N, R, hash_levels, float(init_factor), ldx, lddy, code, flags, tuning, stream))
+    else:
+        _lib.check(lib.rz_weight_grad_hashed(
+            x.data_ptr(), dy.data_ptr(), out.data_ptr(), bias_grad.data_ptr() if with_bias_grad else None,
+            ws.data_ptr() if need else None, need, M, K, N, H, BLOCK_SIZE_K, BLOCK_SIZE_N, R, hash_levels,
+            float(init_factor), ldx, lddy, code, flags, tuning, stream))
     return out, bias_grad
 
 

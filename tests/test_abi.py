@@ -152,3 +152,70 @@ def test_plan_slices_begin_on_step_boundaries(lib):
     with _lib.tuning():
         q = _lib.plan_query(0, 1024, 4352, 2048, 1 << 20, 128, 128, _lib.RZ_BF16)
     assert q["tile"] == 128 and q["slices"] > 1 and q["slice_len"] % 128 == 0, q
+
+
+def _window_geometry(H):
+    """Size and number of the windows of dHW the window kernel works on: one workgroup per compute
+    unit (256) while a window fits its 25600 floats of LDS, else whole rounds of 256 workgroups;
+    never below 1024 floats."""
+    rounds = -(-H // (25600 * 256))
+    w = max((-(-H // (rounds * 256)) + 3) & ~3, 1024)
+    return w, -(-H // w)
+
+
+@pytest.mark.parametrize("cfg", [(1024, 1024, 65536, 64, 64), (300, 330, 70000, 32, 64), (4096, 8192, 40000, 64, 64),
+                                 (640, 640, 2000001, 64, 64), (192, 128, 7000000, 64, 64), (96, 72, 100000, 32, 64),
+                                 (512, 512, 30000, 128, 128), (256, 256, 1000, 16, 16)])
+@pytest.mark.parametrize("levels", [2, 3])
+def test_layer_plan_lists_every_strip_in_every_window_it_meets(lib, oracle, cfg, levels):
+    """rz_layer_plan_build against a brute-force restatement: the tile offsets are the oracle's, and
+    the list of window b holds exactly the 32-row strips [off + 32*BN*s, + 32*BN) that meet
+    [b*w, (b+1)*w), in ascending (tile, strip) order, with their offsets.  Tiles the window kernel
+    does not serve (BN != 64, BK not 32 or 64) get a plan with the offsets alone."""
+    K, N, H, BK, BN = cfg
+    R = R1024 if levels == 2 else oracle.legacy_constants(1024)
+    nbytes = lib.rz_layer_plan_bytes(K, N, H, BK, BN)
+    assert nbytes > 0 and nbytes % 64 == 0
+    plan = np.zeros(nbytes // 4, dtype=np.int32)
+    assert lib.rz_layer_plan_build(plan.ctypes.data, nbytes, K, N, H, BK, BN, _R(R), levels) == 0
+    TK, TN = -(-K // BK), -(-N // BN)
+    tiles = TK * TN
+    want = oracle.c_tile_offsets(K, N, H, BK, BN, R, levels).reshape(-1)
+    assert plan[0] == 0x525A4C50 and list(plan[2:9]) == [K, N, H, BK, BN, levels, tiles]
+    assert np.array_equal(plan[16:16 + tiles].astype(np.int64), want)
+    served = BN == 64 and BK in (32, 64)
+    windows, w = int(plan[9]), int(plan[10])
+    if not served:
+        assert windows == 0 and plan[11] == 0
+        return
+    assert (w, windows) == _window_geometry(H)
+    r16 = lambda v: (v + 15) & ~15
+    start_at = r16(16 + tiles)
+    strips, selems = BK // 32, 32 * BN
+    cap = tiles * strips * (-(-selems // w) + 1)
+    list_at = r16(start_at + windows + 1)
+    offs_at = r16(list_at + cap)
+    assert nbytes == 4 * r16(offs_at + cap)
+    start = plan[start_at:start_at + windows + 1]
+    assert start[0] == 0 and start[-1] == plan[11] and np.all(np.diff(start) >= 0) and start[-1] <= cap
+    so = (want[:, None] + np.arange(strips)[None, :] * selems).reshape(-1)       # index = tile * strips + strip
+    for b in range(windows):
+        meets = np.nonzero((so < (b + 1) * w) & (so + selems > b * w))[0]
+        got = plan[list_at + start[b]:list_at + start[b + 1]]
+        assert np.array_equal(got, meets), b
+        assert np.array_equal(plan[offs_at + start[b]:offs_at + start[b + 1]], so[meets])
+
+
+def test_layer_plan_argument_checks(lib):
+    assert lib.rz_layer_plan_bytes(1024, 1024, 4096, 64, 64) == 0         # H must exceed the tile
+    assert lib.rz_layer_plan_bytes(1024, 1024, 65536, 48, 64) == 0        # not a power of two
+    n = lib.rz_layer_plan_bytes(1024, 1024, 65536, 64, 64)
+    buf = np.zeros(n // 4 + 16, dtype=np.int32)
+    assert lib.rz_layer_plan_build(None, n, 1024, 1024, 65536, 64, 64, _R(R1024), 2) != 0
+    assert lib.rz_layer_plan_build(buf.ctypes.data, n + 64, 1024, 1024, 65536, 64, 64, _R(R1024), 2) != 0
+    assert lib.rz_layer_plan_build(buf.ctypes.data, n, 1024, 1024, 65536, 64, 64, _R(R1024), 2) == 0
+    # a planned call checks the plan's size against its own shape before anything is launched
+    assert lib.rz_weight_grad_planned(1, 1, 1, None, None, 0, buf.ctypes.data, n - 64, 32, 1024, 1024, 65536, 64, 64,
+                                      _R(R1024), 2, 1.0, 1024, 1024, 0, 0, None, None) != 0
+    assert lib.rz_weight_grad_planned(1, 1, 1, None, None, 0, None, n, 32, 1024, 1024, 65536, 64, 64,
+                                      _R(R1024), 2, 1.0, 1024, 1024, 0, 0, None, None) != 0

@@ -36,18 +36,28 @@ def _say(*a):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16], ids=_dt_id)
 @pytest.mark.parametrize("shape", CASES, ids=_shape_id)
-def test_windowed_weight_grad(oracle, tuned, shape, dtype):
+def test_windowed_weight_grad(oracle, tuned, monkeypatch, shape, dtype):
+    from rzlinear_amd import _lib
     from rzlinear_amd.impl.RzLinearBackward import rz_linear_backward_weight_grad_tl
     tuned(window=1)
     M, K, N, H, BK, BN = shape
     _say("windowed weight grad", shape, dtype)
     (x, _, dy), (x64, _, dy64) = make_inputs(M, K, N, H, dtype, seed=31)
+    # without a layer plan (every workgroup searches the tile offsets for its strips) ...
+    monkeypatch.setattr(_lib, "use_layer_plans", False)
     dhw = rz_linear_backward_weight_grad_tl(x, dy, 0.5, M, K, N, H, *rargs(R1024), BLOCK_SIZE_K=BK,
                                             BLOCK_SIZE_N=BN)
     torch.cuda.synchronize()
     ref = oracle.weight_grad(x64, dy64, H, BK, BN, R1024, 0.5)
     got = dhw.float().cpu().numpy()
     assert rel_err(got, ref) <= TOL[dtype]
+    # ... and with one (the lists come from the plan): the same strips in the same order, the same bits
+    monkeypatch.setattr(_lib, "use_layer_plans", True)
+    _say("  with a layer plan")
+    planned = rz_linear_backward_weight_grad_tl(x, dy, 0.5, M, K, N, H, *rargs(R1024), BLOCK_SIZE_K=BK,
+                                                BLOCK_SIZE_N=BN)
+    torch.cuda.synchronize()
+    assert torch.equal(planned, dhw)
     assert (got[ref == 0] == 0).all()          # slots that no tile covers stay exactly zero
     # the summation order is fixed: a second call gives the same bits
     again = rz_linear_backward_weight_grad_tl(x, dy, 0.5, M, K, N, H, *rargs(R1024), BLOCK_SIZE_K=BK,
@@ -141,3 +151,42 @@ def test_windowed_weight_grad_random_shapes(oracle, tuned, shape):
     dhw = rz_linear_backward_weight_grad_tl(x, dy, 1.25, M, K, N, H, *rargs(R), BLOCK_SIZE_K=BK, BLOCK_SIZE_N=BN)
     torch.cuda.synchronize()
     assert rel_err(dhw.float().cpu().numpy(), oracle.weight_grad(x64, dy64, H, BK, BN, R, 1.25)) <= TOL[dtype]
+
+
+def test_a_plan_of_another_layer_is_refused_on_the_device(tuned):
+    """The host can check a plan's size only; the kernel checks its header against the call and
+    turns dHW into NaN instead of following lists that belong to other shapes."""
+    from rzlinear_amd import _lib
+    tuned(window=1)
+    M, K, N, H, BK, BN = 32, 512, 512, 300000, 64, 64
+    _say("foreign layer plan")
+    (x, _, dy), _ = make_inputs(M, K, N, H, torch.float32, seed=41)
+    lib = _lib.load()
+    R = _lib.hash_constants(*rargs(R1024))
+    plan = _lib.layer_plan(K, N, H, BK, BN, R, 2, x.device).clone()
+    plan[2] = K + 64                                   # the header now names another K
+    out = torch.zeros((H,), device=x.device)
+    _lib.check(lib.rz_weight_grad_planned(x.data_ptr(), dy.data_ptr(), out.data_ptr(), None, None, 0, plan.data_ptr(),
+                                          plan.numel() * 4, M, K, N, H, BK, BN, R, 2, 1.0, K, N, _lib.RZ_F32, 0,
+                                          _lib.current_tuning(), torch.cuda.current_stream().cuda_stream))
+    torch.cuda.synchronize()
+    assert torch.isnan(out).all()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=_dt_id)
+def test_fold_path_takes_its_tile_offsets_from_the_plan(oracle, tuned, monkeypatch, dtype):
+    from rzlinear_amd import _lib
+    from rzlinear_amd.impl.RzLinearBackward import rz_linear_backward_weight_grad_tl
+    tuned(fold=1, window=-1)
+    M, K, N, H, BK, BN = 300, 512, 768, 90000, 64, 64
+    code = _lib.dtype_code(torch.empty(0, dtype=dtype))
+    assert _lib.plan_query(2, M, K, N, H, BK, BN, code)["mode"] == "fold"
+    _say("fold with a layer plan", dtype)
+    (x, _, dy), (x64, _, dy64) = make_inputs(M, K, N, H, dtype, seed=43)
+    monkeypatch.setattr(_lib, "use_layer_plans", False)
+    a = rz_linear_backward_weight_grad_tl(x, dy, 1.0, M, K, N, H, *rargs(R1024), BLOCK_SIZE_K=BK, BLOCK_SIZE_N=BN)
+    monkeypatch.setattr(_lib, "use_layer_plans", True)
+    b = rz_linear_backward_weight_grad_tl(x, dy, 1.0, M, K, N, H, *rargs(R1024), BLOCK_SIZE_K=BK, BLOCK_SIZE_N=BN)
+    torch.cuda.synchronize()
+    assert torch.equal(a, b)
+    assert rel_err(b.float().cpu().numpy(), oracle.weight_grad(x64, dy64, H, BK, BN, R1024, 1.0)) <= TOL[dtype]
