@@ -182,6 +182,17 @@ static inline long long tile_cover(int K, int N, int t) {
   return (long long)((K + t - 1) / t) * ((N + t - 1) / t) * t * t;
 }
 
+// Slices of M for the 128 and 256 tiles with LDS images: as many as fill the compute units once.  A
+// few workgroups beyond one per compute unit would make a second round that costs as much as the
+// first (300 workgroups take as long as 512), so the count stays at or below the compute units
+// (K = N = 2560, M = 2048 bf16: 3 slices x 100 tiles 57.9 us, 2 slices 46.8 us).
+static inline long long image_slices(long long tiles, long long r_steps) {
+  long long want = (kComputeUnits + tiles - 1) / tiles;
+  if (want > 1 && tiles * want > kComputeUnits) want--;
+  if (want > r_steps) want = r_steps;
+  return want < 1 ? 1 : want;
+}
+
 static inline WeightGradPlan plan_weight_grad(int M, int K, int N, int H, int BK, int BN, int elem_bytes,
                                               const rz_tuning& t) {
   WeightGradPlan pl;
@@ -199,10 +210,30 @@ static inline WeightGradPlan plan_weight_grad(int M, int K, int N, int H, int BK
     // and its scatter: the 128 tile then has less to set up and to scatter per workgroup
     const long long tiles256 = tile_count(K, N, 256);
     const int step256 = slice_unit(256, elem_bytes);
-    if (pl.tile == 256 && tiles256 < kComputeUnits &&
-        (long long)((M + step256 - 1) / step256) * tiles256 < 4LL * kComputeUnits &&
-        tile_cover(K, N, 128) * 10 <= tile_cover(K, N, 256) * 13)
+    const bool cover128 = tile_cover(K, N, 128) * 10 <= tile_cover(K, N, 256) * 13;
+    if (pl.tile == 256 && elem_bytes == 4 && tiles256 < kComputeUnits &&
+        (long long)((M + step256 - 1) / step256) * tiles256 < 4LL * kComputeUnits && cover128)
       pl.tile = 128;
+    if (pl.tile == 256 && elem_bytes == 2 && cover128) {
+      // 16-bit: the two tiles by estimated time.  Fitted on MI355X (weight-grad, 256 workgroups):
+      // a 256 workgroup pays about 5.5 steps of 64 rows for its fill, its image rounds and the
+      // store of its image, whatever the length of its loop; the 128 tile in its eight-wavefront
+      // form (steps of 128 rows, up to 384 workgroups) runs at 0.82 of the 256 tile's rate and
+      // pays about 4 of its steps.  Both write one image per workgroup.  (2048^3: 32.4 -> 30.5 us;
+      // M = 8192, K = N = 2048 stays with the 256 tile: 72.8 against 82.1 us.)
+      const long long tiles128 = tile_count(K, N, 128);
+      const long long s256 = image_slices(tiles256, (M + 63) / 64), s128 = image_slices(tiles128, (M + 127) / 128);
+      const long long w256 = tiles256 * s256, w128 = tiles128 * s128;
+      if (w128 <= kComputeUnits * 3 / 2) {
+        auto filled = [](long long w, long long cap) { return (double)w / (double)((w + cap - 1) / cap * cap); };
+        const double st256 = (double)(((M + 63) / 64 + s256 - 1) / s256), st128 = (double)(((M + 127) / 128 + s128 - 1) / s128);
+        const double work_us = 2.0 * (double)M * K * N / 1200e6;
+        const double image_us = (double)pitch * 8.0 / 5e6;   // written once, read once
+        const double t256 = work_us * (st256 + 5.5) / st256 / filled(w256, kComputeUnits) + (double)w256 * image_us;
+        const double t128 = work_us * (st128 + 4.0) / st128 / (0.82 * filled(w128, kComputeUnits)) + (double)w128 * image_us;
+        if (t128 < t256 * 0.97) pl.tile = 128;
+      }
+    }
   } else {
     pl.tile = pick_tile(K, N, elem_bytes, t);
     // fp32 with the tiles stored for the fold kernel: a 256 workgroup is alone on its compute unit
@@ -220,6 +251,7 @@ static inline WeightGradPlan plan_weight_grad(int M, int K, int N, int H, int BK
   long long want = (target + tiles - 1) / tiles;
   if (want > r_steps) want = r_steps;
   if (want < 1) want = 1;
+  if (image && pl.tile >= 128) want = image_slices(tiles, r_steps);
   if (!image) {
     // every slice repeats the K*N adds of the scatter (global atomics, about 5.4 ps each, some 70 %
     // of which the contraction does not hide): the number of slices with the least estimated time
