@@ -204,6 +204,46 @@ def output_check(torch, _lib, wl):
     return {k: float("%.3g" % v) for k, v in errs.items()}
 
 
+def api_level(torch, wl, warmup, steps):
+    """ms per forward + backward of rzlinear_amd.RzLinear (bias fused into the forward store, bias
+    gradient from the weight-grad pass, gradients allocated by autograd) and of torch.nn.Linear,
+    `warmup` + `steps` calls each, HIP events around the whole run."""
+    from rzlinear_amd import RzLinear
+    M, K, N, H, BK, BN = (wl[k] for k in ("M", "K", "N", "H", "BK", "BN"))
+    dev, dtype = wl["x"].device, wl["dtype"]
+    layer = RzLinear(K, N, hashed_weight=torch.nn.Parameter(wl["hw"].clone()), seed=1024, bias=True, dtype=dtype,
+                     block_size_k=BK, block_size_n=BN).to(dev)
+    dense = torch.nn.Linear(K, N, bias=True, dtype=dtype, device=dev)
+    x = wl["x"].clone().requires_grad_(True)
+    dy = wl["dy"]
+
+    def run(mod):
+        def step():
+            x.grad = None
+            for prm in mod.parameters():
+                prm.grad = None
+            mod(x).backward(dy)
+        for _ in range(warmup):
+            step()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        a.record()
+        for _ in range(steps):
+            step()
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) / steps
+
+    d_ms = run(dense)
+    rz_ms = run(layer)
+    fl = 3 * wl["flop_gemm"]
+    return {"what": "RzLinear module forward + backward through autograd (bias, bias gradient, allocations included), "
+                    "%d + %d steps; torch.nn.Linear the same way" % (warmup, steps),
+            "rz_ms": round(rz_ms, 4), "rz_tflops": round(tflops(fl, rz_ms), 2),
+            "nn_linear_ms": round(d_ms, 4), "nn_linear_tflops": round(tflops(fl, d_ms), 2),
+            "rz_over_nn_linear": round(d_ms / rz_ms, 4)}
+
+
 def tflops(flop, ms):
     return flop / (ms * 1e-3) / 1e12
 
@@ -219,6 +259,7 @@ def main():
     ap.add_argument("--no-dense", action="store_true")
     ap.add_argument("--no-sweep", action="store_true")
     ap.add_argument("--no-check", action="store_true")
+    ap.add_argument("--no-api", action="store_true", help="skip the module-level (autograd) timing")
     ap.add_argument("--cpu-budget", type=float, default=15.0, help="seconds of CPU-path timing")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MiB",
                     help="only run a plain device-to-device copy of this many MiB (five launches) and exit: "
@@ -328,6 +369,13 @@ def main():
         sweep = {"protocol": "warm-up %d + %d timed steps per configuration (dense legs first, then rz); the headline "
                              "configuration's row repeats the headline run" % (sw_warm, sw_steps), "rows": sweep}
 
+    # ---- the same step through the package's module and autograd (what a user of the reference
+    # calls: python/bench/bench.py:44 times `rz(a)`), outputs allocated by the API, beside
+    # torch.nn.Linear of the same shape timed the same way; short, outside the headline ----------
+    api = None
+    if not args.no_api:
+        api = api_level(torch, wl, 5, 20)
+
     cpu_baseline = None
     if not args.no_cpu_baseline:
         from oracle import cpu_path   # checker/baseline only: never on the measured GPU path
@@ -371,6 +419,7 @@ def main():
         "output_check": check,
         "roofline": roofline,
         "dense_gemm": dense,
+        "api_level": api,
         "cpu_baseline": cpu_baseline,
         "sweep": sweep,
     }

@@ -7,10 +7,9 @@ random_numbers, output_dim, chunk_size, init_factor)`` and a backward that hands
 """
 import torch
 
-from .impl.RzLinearBackward import (rz_linear_backward_input_grad_tl,
-                                    rz_linear_backward_weight_bias_grad_tl,
-                                    rz_linear_backward_weight_grad_tl)
-from .impl.RzLinearForward import rz_linear_forward_bias_tl
+from . import _lib
+from .impl.RzLinearBackward import input_grad_hashed, weight_grad_hashed
+from .impl.RzLinearForward import forward_hashed
 
 # Code written against the reference sets these two switches; they are accepted and have no
 # effect here (no autotuner; fp32 is true fp32).  block_size_k / block_size_n give the hashed
@@ -24,15 +23,11 @@ controls = {
 }
 
 
-def _launcher_kwargs(block_k, block_n):
-    return dict(allow_tf32=controls['triton_allow_tf32'], allow_autotune=controls['triton_allow_autotune'],
-                BLOCK_SIZE_K=block_k, BLOCK_SIZE_N=block_n)
-
-
-def _hash_args(random_numbers):
-    """R7..R0, the positional order of the launchers, from the 8-element CPU tensor."""
+def _hash_constants(random_numbers):
+    """The int32[8] array of the C ABI (index = subscript) from the 8-element CPU tensor."""
     assert random_numbers.numel() == 8
-    return tuple(int(v) for v in reversed(random_numbers.tolist()))
+    r = random_numbers.tolist()
+    return _lib.hash_constants(r[7], r[6], r[5], r[4], r[3], r[2], r[1], r[0])
 
 
 class RzLinearFunction(torch.autograd.Function):
@@ -51,17 +46,18 @@ class RzLinearFunction(torch.autograd.Function):
     @staticmethod
     def forward(ctx, input, hashed_weight, random_numbers, output_dim, chunk_size, init_factor,
                 block_size_k=None, block_size_n=None, bias=None, fuse_grad_accumulation=False):
-        consts = _hash_args(random_numbers)
+        R = _hash_constants(random_numbers)
         tile = (int(controls['block_size_k'] if block_size_k is None else block_size_k),
                 int(controls['block_size_n'] if block_size_n is None else block_size_n))
         M, K = input.shape
         H = hashed_weight.shape[0]
-        output = rz_linear_forward_bias_tl(input, hashed_weight.data, None if bias is None else bias.data,
-                                           init_factor, M, K, output_dim, H, *consts,
-                                           **_launcher_kwargs(*tile))
+        assert (H > (tile[0] * tile[1]))   # (the launchers' assertion, impl/RzLinearForward.py:28 in the reference)
+        output = forward_hashed(input, hashed_weight.data, None if bias is None else bias.data, init_factor,
+                                M, K, output_dim, H, R, tile[0], tile[1], _lib.HASH_TWO_LEVEL)
         ctx.save_for_backward(input, hashed_weight, random_numbers)
         ctx.output_dim, ctx.chunk_size, ctx.init_factor = output_dim, chunk_size, init_factor
         ctx.tile = tile
+        ctx.hash_constants = R   # (the ctypes array: backward need not convert the tensor again)
         ctx.has_bias = bias is not None
         ctx.fuse_grad_accumulation = bool(fuse_grad_accumulation)
         return output
@@ -71,18 +67,18 @@ class RzLinearFunction(torch.autograd.Function):
         """One value per argument of forward (autograd drops trailing Nones that apply() was not
         given).  A gradient that autograd does not need is not computed — the reference always
         computes both."""
-        input, hashed_weight, random_numbers = ctx.saved_tensors
-        consts = _hash_args(random_numbers)
+        input, hashed_weight, _ = ctx.saved_tensors
+        R = ctx.hash_constants
         M, K = input.shape
         N, H = ctx.output_dim, hashed_weight.shape[0]
-        kwargs = _launcher_kwargs(*ctx.tile)
+        BK, BN = ctx.tile
         need_input, need_weight = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
         need_bias = ctx.has_bias and ctx.needs_input_grad[8]
 
         input_grad = weight_grad = bias_grad = None
         if need_input:      # enqueued first, like the reference's rz_linear_backward_tl
-            input_grad = rz_linear_backward_input_grad_tl(grad, hashed_weight.data, ctx.init_factor,
-                                                          M, K, N, H, *consts, **kwargs)
+            input_grad = input_grad_hashed(grad, hashed_weight.data, ctx.init_factor, M, K, N, H, R, BK, BN,
+                                           _lib.HASH_TWO_LEVEL)
         if need_weight and ctx.fuse_grad_accumulation:
             # Add into the parameter's gradient buffer inside the kernels.  The first layer to
             # reach a parameter without a gradient overwrites a fresh buffer (no zero-fill), the
@@ -94,16 +90,11 @@ class RzLinearFunction(torch.autograd.Function):
                     hashed_weight.grad = torch.empty_like(hashed_weight)
                     accumulate = False
                 target = hashed_weight.grad
-            launcher = rz_linear_backward_weight_bias_grad_tl if need_bias else rz_linear_backward_weight_grad_tl
-            result = launcher(input, grad, ctx.init_factor, M, K, N, H, *consts, out=target, accumulate=accumulate,
-                              **kwargs)
-            bias_grad = result[1] if need_bias else None
-        elif need_weight and need_bias:   # one pass over grad yields both
-            weight_grad, bias_grad = rz_linear_backward_weight_bias_grad_tl(input, grad, ctx.init_factor,
-                                                                            M, K, N, H, *consts, **kwargs)
-        elif need_weight:
-            weight_grad = rz_linear_backward_weight_grad_tl(input, grad, ctx.init_factor,
-                                                            M, K, N, H, *consts, **kwargs)
+            _, bias_grad = weight_grad_hashed(input, grad, ctx.init_factor, M, K, N, H, R, BK, BN, out=target,
+                                              accumulate=accumulate, with_bias_grad=need_bias)
+        elif need_weight:   # (with a bias: one pass over grad yields both gradients)
+            weight_grad, bias_grad = weight_grad_hashed(input, grad, ctx.init_factor, M, K, N, H, R, BK, BN,
+                                                        with_bias_grad=need_bias)
         elif need_bias:
             bias_grad = grad.sum(dim=0)
         return input_grad, weight_grad, None, None, None, None, None, None, bias_grad, None

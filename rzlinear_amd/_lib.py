@@ -64,6 +64,22 @@ def current_tuning():
     return ctypes.byref(_tuning) if _tuning is not None else None
 
 _lib = None
+_host_answers = {}
+
+
+def host_query(name, *args):
+    """lib.<name>(*args, tuning) for the host-only queries (workspace sizes), remembered per
+    argument tuple and tuning: a layer asks the same question on every step, and the answer is a
+    pure function of the arguments."""
+    t = _tuning
+    key = (name, args, None if t is None else tuple(getattr(t, f) for f, _ in Tuning._fields_))
+    try:
+        return _host_answers[key]
+    except KeyError:
+        if len(_host_answers) > 4096:
+            _host_answers.clear()
+        v = _host_answers[key] = getattr(load(), name)(*args, current_tuning())
+        return v
 
 
 class RzLinearError(RuntimeError):
@@ -187,15 +203,25 @@ def dtype_code(t):
         raise TypeError("rzlinear_amd supports float32, bfloat16 and float16, got %s" % t.dtype)
 
 
+try:   # the raw handle of the current stream, without building a torch.cuda.Stream object around it
+    _raw_stream = torch._C._cuda_getCurrentRawStream
+except AttributeError:   # pragma: no cover
+    def _raw_stream(index):
+        return torch.cuda.current_stream(index).cuda_stream
+
+
 def require_gpu(*tensors):
     """All tensors must live on one ROCm device; returns the raw HIP stream handle to use."""
-    dev = tensors[0].device
+    first = tensors[0]
+    if not first.is_cuda:
+        raise RuntimeError("rzlinear_amd runs on a ROCm GPU only; got a tensor on %s" % first.device)
+    index = first.get_device()
     for t in tensors:
-        if t.device.type != "cuda":
+        if not t.is_cuda:
             raise RuntimeError("rzlinear_amd runs on a ROCm GPU only; got a tensor on %s" % t.device)
-        if t.device != dev:
-            raise RuntimeError("rzlinear_amd: tensors on different devices (%s, %s)" % (dev, t.device))
-    return torch.cuda.current_stream(dev).cuda_stream
+        if t.get_device() != index:
+            raise RuntimeError("rzlinear_amd: tensors on different devices (%s, %s)" % (first.device, t.device))
+    return _raw_stream(index)
 
 
 def rows(t):
@@ -251,6 +277,13 @@ PLAN_MODES = {0: "store", 1: "split", 2: "lds_image", 3: "atomics", 4: "window",
 def plan_query(op, M, K, N, H, BK, BN, dtype_code_, flags=0, with_dbias=False):
     """How the library would carry out a call (rz_plan_query), under the current tuning:
     dict(tile, slices, slice_len, step, mode, workgroups).  op: 0 forward, 1 input-grad, 2 weight-grad."""
-    out = (ctypes.c_int32 * 8)()
-    check(load().rz_plan_query(op, M, K, N, H, BK, BN, dtype_code_, flags, int(with_dbias), current_tuning(), out))
-    return dict(tile=out[0], slices=out[1], slice_len=out[2], step=out[3], mode=PLAN_MODES[out[4]], workgroups=out[5])
+    t = _tuning
+    key = ("rz_plan_query", (op, M, K, N, H, BK, BN, dtype_code_, flags, int(with_dbias)),
+           None if t is None else tuple(getattr(t, f) for f, _ in Tuning._fields_))
+    ans = _host_answers.get(key)
+    if ans is None:
+        out = (ctypes.c_int32 * 8)()
+        check(load().rz_plan_query(op, M, K, N, H, BK, BN, dtype_code_, flags, int(with_dbias), current_tuning(), out))
+        ans = _host_answers[key] = dict(tile=out[0], slices=out[1], slice_len=out[2], step=out[3],
+                                        mode=PLAN_MODES[out[4]], workgroups=out[5])
+    return dict(ans)

@@ -65,8 +65,8 @@ def weight_grad_hashed(input, output_grad, init_factor, M, K, N, H, R, BLOCK_SIZ
             out.zero_()
         return out, (bias_grad.zero_() if with_bias_grad else None)
     tuning = _lib.current_tuning()
-    need = lib.rz_weight_grad_hashed_workspace_bytes(M, K, N, H, BLOCK_SIZE_K, BLOCK_SIZE_N, code, flags,
-                                                     int(with_bias_grad), tuning)
+    need = _lib.host_query("rz_weight_grad_hashed_workspace_bytes", M, K, N, H, BLOCK_SIZE_K, BLOCK_SIZE_N, code,
+                           flags, int(with_bias_grad))
     ws = _lib.workspace(need, output_grad.device)
     plan = None
     if use_layer_plan is None:
@@ -160,7 +160,7 @@ def input_grad_hashed(output_grad, hashed_weight, init_factor, M, K, N, H, R, BK
     lib = _lib.load()
     code = _lib.dtype_code(output_grad)
     tuning = _lib.current_tuning()
-    need = lib.rz_input_grad_hashed_workspace_bytes(M, K, N, H, BK, BN, code, tuning)
+    need = _lib.host_query("rz_input_grad_hashed_workspace_bytes", M, K, N, H, BK, BN, code)
     ws = _lib.workspace(need, output_grad.device)
     _lib.check(lib.rz_input_grad_hashed(
         dy.data_ptr(), hw.data_ptr(), input_grad.data_ptr(), ws.data_ptr() if need else None, need,

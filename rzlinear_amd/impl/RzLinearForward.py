@@ -60,7 +60,7 @@ def forward_hashed(input, hashed_weight, bias, init_factor, M, K, N, H, R, BK, B
     code = _lib.dtype_code(input)
     # skinny problems split the contraction and need a scratch buffer for the partial results
     tuning = _lib.current_tuning()
-    need = lib.rz_forward_hashed_workspace_bytes(M, K, N, H, BK, BN, code, tuning)
+    need = _lib.host_query("rz_forward_hashed_workspace_bytes", M, K, N, H, BK, BN, code)
     ws = _lib.workspace(need, input.device)
     _lib.check(lib.rz_forward_hashed(
         x.data_ptr(), hw.data_ptr(), bias.data_ptr() if bias is not None else None, output.data_ptr(),
