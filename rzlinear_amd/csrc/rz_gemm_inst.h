@@ -155,7 +155,9 @@ static hipError_t launch_window_form(const WindowParams& p, int windows, hipStre
 template <typename T, int TBK, int TBN>
 static hipError_t launch_window_one(const WindowParams& p, int windows, hipStream_t stream) {
   constexpr int kVec = 16 / (int)sizeof(T);
-  if (p.K % kVec == 0 && p.N % kVec == 0) return launch_window_form<T, TBK, TBN, true>(p, windows, stream);
+  // (the staged form keeps a lane's piece offsets, up to sixteen rows, in 32-bit registers)
+  if (p.K % kVec == 0 && p.N % kVec == 0 && p.ldx < (1 << 26) && p.lddy < (1 << 26))
+    return launch_window_form<T, TBK, TBN, true>(p, windows, stream);
   return launch_window_form<T, TBK, TBN, false>(p, windows, stream);
 }
 

@@ -354,13 +354,14 @@ static inline WindowPlan plan_window(int M, int K, int N, int H, int BK, int BN,
   const long long w = pl.window;
   // Rough times in microseconds, fitted to measurements at K = N = 10240, H = 6.5 M on MI355X.
   // Scatter kernel: K*N atomics at about 184 G/s plus the product.  Window kernel: every
-  // workgroup works through tiles * (window + tile) / H tiles; a tile costs about 0.27 us plus
-  // 0.22 us (16-bit), or 0.8 us (fp32: the fp32 MFMA rate), per 32 rows of M (the operands of every
-  // tile come out of L2 again: tiles that share a window share no rows or columns of W).
+  // workgroup works through tiles * (window + tile) / H tiles; a tile costs about 0.31 us plus
+  // 0.18 us (16-bit), or 0.43 us plus 0.63 us (fp32: the fp32 MFMA rate), per 32 rows of M (the
+  // operands of every tile come out of L2 again: tiles that share a window share no rows or
+  // columns of W; a wavefront has three groups of rows in flight, which is what its registers hold).
   const double chunks = (double)((M + 31) / 32);
   const double per_wg = (double)tiles * ((double)w + (double)BK * BN) / (double)H;
   const double wg_rounds = (double)((pl.windows + kComputeUnits - 1) / kComputeUnits);
-  const double t_window = wg_rounds * per_wg * (0.27 + (elem_bytes == 4 ? 0.80 : 0.22) * chunks) + (planned ? 5.0 : 28.0);
+  const double t_window = wg_rounds * per_wg * ((elem_bytes == 4 ? 0.43 + 0.63 * chunks : 0.31 + 0.18 * chunks)) + (planned ? 5.0 : 28.0);
   // ... against what the contraction kernel's plan would take: the fold, or the atomic scatter
   const double t_scatter = 0.9 * (double)K * N / 184e3 + 2.0 * M * (double)K * N / 800e6;
   const double t_other = other.fold.use ? other.fold_us : t_scatter;

@@ -159,7 +159,10 @@ struct WindowKernel {
     Frag fa[kDepth][GS][BI], fb[kDepth][GS][BJ];
     // 16-bit staged path: the raw 16-byte pieces instead (one of X, two of dY per lane and group)
     u32x4_t px[kDepth], py[kDepth][2];
-    bool okx[kDepth], oky[kDepth][2];
+    // element offset of this lane's piece of X, and of its two pieces of dY, from the first row of a group
+    const int lane_x = STAGED ? (lane / (32 / VEC)) * (int)p.ldx + (lane % (32 / VEC)) * VEC : 0;
+    const int lane_y[2] = {STAGED ? (lane / (TBN / VEC)) * (int)p.lddy + (lane % (TBN / VEC)) * VEC : 0,
+                           STAGED ? (lane / (TBN / VEC) + 64 / (TBN / VEC)) * (int)p.lddy + (lane % (TBN / VEC)) * VEC : 0};
 
     // Listing the strips that meet the window, in ascending (tile, strip) order.  The tile ids of
     // a range [lo, hi) are dealt to the wavefronts in contiguous chunks; every wavefront first
@@ -290,8 +293,69 @@ struct WindowKernel {
       // for ALL loads at the first use behind the join — the item just requested included.
       // Beyond the wavefront's last item the last strip is fetched again (valid addresses, in
       // cache; what arrives is multiplied into accumulators that nobody reads any more).
+      // Staged form: what a fetch needs of its strip is worked out once per strip and kept in
+      // scalar registers (the strip's first column in X and in dY, whether all its columns
+      // exist), and what it needs of the lane once per kernel (lane_x / lane_y: element
+      // offset of the lane's piece from the group's first row); an item then costs two scalar
+      // multiply-adds and three loads with a uniform base.  Only groups with rows beyond M and
+      // strips at the edge of the matrix take the path with per-lane checks.
+      // (offsets, not pointers: a pointer carried round the loop would lose its address space
+      //  and turn the loads into flat ones, which also count as LDS traffic)
+      int strip_x = 0, strip_k0 = 0, strip_n0 = 0;
+      bool strip_whole = false;
+      // which of a lane's three pieces of the group at row m0 of strip (k0, n0) lie inside the matrices
+      auto pieces_inside = [&](int m0, int k0, int n0, bool& okx, bool& oky0, bool& oky1) {
+        constexpr int PX = 32 / VEC, PY = TBN / VEC;
+        okx = m0 + lane / PX < p.M && k0 + (lane % PX) * VEC < p.K;
+        const bool col_ok = n0 + (lane % PY) * VEC < p.N;
+        oky0 = m0 + lane / PY < p.M && col_ok;
+        oky1 = m0 + lane / PY + 64 / PY < p.M && col_ok;
+      };
+      // ... and the same for the strip being multiplied
+      int mult_k0 = 0, mult_n0 = 0;
+      bool mult_whole = false;
       auto fetch_next = [&](auto set) {
         constexpr int S = decltype(set)::value;
+        if constexpr (STAGED) {
+          if (fg == 0) {   // (uniform) a new strip
+            const int ftc = ft < my_tiles ? ft : my_tiles - 1;
+            const int v = __builtin_amdgcn_readfirstlane(sm.list[wave + ftc * kWaves]);
+            const int id = v / kStrips, strip = v % kStrips;
+            const int tk = id / p.tiles_n, tn = id - tk * p.tiles_n;
+            strip_k0 = tk * TBK + strip * 32;              // the strip's first row of W
+            strip_n0 = tn * TBN;
+            strip_whole = strip_k0 + 32 <= p.K && strip_n0 + TBN <= p.N;
+            // (a strip that begins beyond K contributes nothing; its base is kept inside the matrix)
+            strip_x = strip_k0 < p.K ? strip_k0 : p.K - 1;
+          }
+          const int m0 = fg * kGroupRows;
+          const T* rows_x = gX + ((int64_t)m0 * p.ldx + strip_x);
+          const T* rows_y = gdY + ((int64_t)m0 * p.lddy + strip_n0);
+          const T* src_x = rows_x + lane_x;
+          const T* src_y0 = rows_y + lane_y[0];
+          const T* src_y1 = rows_y + lane_y[1];
+          if (!(strip_whole && m0 + kGroupRows <= p.M)) {   // (uniform, rare)
+            // a piece outside the matrix is fetched from inside it (and replaced by zero when the
+            // item is multiplied, where the same checks are made again: nothing about a set is
+            // carried round the ring but its data)
+            // (the empty statement keeps this block out of the usual path: its arithmetic would
+            //  otherwise be carried out for every item and thrown away)
+            asm volatile("" ::: "memory");
+            bool okx, oky0, oky1;
+            pieces_inside(m0, strip_k0, strip_n0, okx, oky0, oky1);
+            src_x = okx ? src_x : gX + (int64_t)m0 * p.ldx;
+            src_y0 = oky0 ? src_y0 : gdY + (int64_t)m0 * p.lddy;
+            src_y1 = oky1 ? src_y1 : gdY + (int64_t)m0 * p.lddy;
+          }
+          __builtin_memcpy(&px[S], src_x, 16);
+          __builtin_memcpy(&py[S][0], src_y0, 16);
+          __builtin_memcpy(&py[S][1], src_y1, 16);
+          if (++fg == ngroups) {
+            fg = 0;
+            ft++;
+          }
+          return;
+        }
         {
           const int ftc = ft < my_tiles ? ft : my_tiles - 1;
           const int v = __builtin_amdgcn_readfirstlane(sm.list[wave + ftc * kWaves]);
@@ -303,34 +367,6 @@ struct WindowKernel {
           // (a strip that begins beyond K contributes nothing; its base is kept inside the matrix)
           const T* rows_x = gX + (int64_t)m0 * p.ldx + (int64_t)(k0 < p.K ? k0 : p.K - 1);
           const T* rows_y = gdY + (int64_t)m0 * p.lddy + (int64_t)tn * TBN;
-          if constexpr (STAGED) {
-            {
-              // X: 32 / VEC pieces per row, the 64 lanes cover the group's rows; dY: TBN / VEC pieces per
-              // row, two passes.  (16-bit: X row lane / 4, piece lane % 4; dY rows lane / 8 and + 8, piece
-              // lane % 8.)  A piece outside the matrix is fetched from inside it and replaced by zero later.
-              constexpr int PX = 32 / VEC, PY = TBN / VEC;
-              {
-                const int r = lane / PX, c = (lane % PX) * VEC;
-                const bool ok = m0 + r < p.M && k0 + c < p.K;
-                const T* src = ok ? gX + (int64_t)(m0 + r) * p.ldx + (k0 + c) : gX + (int64_t)m0 * p.ldx;
-                __builtin_memcpy(&px[S], src, 16);
-                okx[S] = ok;
-              }
-#pragma unroll
-              for (int q = 0; q < 2; q++) {
-                const int r = lane / PY + (64 / PY) * q, c = (lane % PY) * VEC;
-                const bool ok = m0 + r < p.M && tn * TBN + c < p.N;
-                const T* src = ok ? rows_y + (int64_t)r * p.lddy + c : gdY + (int64_t)m0 * p.lddy;
-                __builtin_memcpy(&py[S][q], src, 16);
-                oky[S][q] = ok;
-              }
-              if (++fg == ngroups) {
-                fg = 0;
-                ft++;
-              }
-              return;
-            }
-          }
 #pragma unroll
           for (int a = 0; a < BI; a++) {
             const int col = a * 32 + (lane & 31);
@@ -375,14 +411,21 @@ struct WindowKernel {
 #pragma unroll
           for (int b = 0; b < BJ; b++) {
             float* at = win + rel + ((lane >> 5) * 4) * TBN + b * 32 + (lane & 31);
-            // (a block's sixteen reads go out together: one LDS round trip per block)
-            float cur[16];
+            // (eight elements at a time: 16 wavefronts per compute unit leave few registers)
 #pragma unroll
-            for (int i = 0; i < 16; i++) cur[i] = at[((i >> 2) * 8 + (i & 3)) * TBN];
+            for (int half = 0; half < 2; half++) {
+              float cur[8];
 #pragma unroll
-            for (int i = 0; i < 16; i++) {
-              at[((i >> 2) * 8 + (i & 3)) * TBN] = cur[i] + acc[0][b][i] * p.scale;
-              acc[0][b][i] = 0.f;
+              for (int q = 0; q < 8; q++) {
+                const int i = half * 8 + q;
+                cur[q] = at[((i >> 2) * 8 + (i & 3)) * TBN];
+              }
+#pragma unroll
+              for (int q = 0; q < 8; q++) {
+                const int i = half * 8 + q;
+                at[((i >> 2) * 8 + (i & 3)) * TBN] = cur[q] + acc[0][b][i] * p.scale;
+                acc[0][b][i] = 0.f;
+              }
             }
           }
         } else {
@@ -428,7 +471,25 @@ struct WindowKernel {
             T* st = sm.stage[wave];
             const u32x4_t z = {0u, 0u, 0u, 0u};
             constexpr int PX = 32 / VEC, PY = TBN / VEC;
-            *reinterpret_cast<u32x4_t*>(st + (lane / PX) * 32 + (lane % PX) * VEC) = okx[S] ? px[S] : z;
+            // (pieces outside the matrix become zero; the usual set has none: a uniform branch, no selects)
+            u32x4_t wx = px[S], wy[2] = {py[S][0], py[S][1]};
+            if (pg == 0) {   // (uniform) a new strip
+              const int ptc = pt < my_tiles ? pt : my_tiles - 1;
+              const int v = __builtin_amdgcn_readfirstlane(sm.list[wave + ptc * kWaves]);
+              const int id = v / kStrips, tk = id / p.tiles_n;
+              mult_k0 = tk * TBK + (v % kStrips) * 32;
+              mult_n0 = (id - tk * p.tiles_n) * TBN;
+              mult_whole = mult_k0 + 32 <= p.K && mult_n0 + TBN <= p.N;
+            }
+            if (!(mult_whole && (pg + 1) * kGroupRows <= p.M)) {
+              asm volatile("" ::: "memory");
+              bool okx, oky0, oky1;
+              pieces_inside(pg * kGroupRows, mult_k0, mult_n0, okx, oky0, oky1);
+              wx = okx ? wx : z;
+              wy[0] = oky0 ? wy[0] : z;
+              wy[1] = oky1 ? wy[1] : z;
+            }
+            *reinterpret_cast<u32x4_t*>(st + (lane / PX) * 32 + (lane % PX) * VEC) = wx;
             if constexpr (k16) {
 #pragma unroll
               for (int q = 0; q < 2; q++) {
@@ -436,7 +497,7 @@ struct WindowKernel {
                 // dY rows are two 64-byte chunks, swapped in every other pair of rows, so that the four
                 // rows of a transpose read fall on different banks
                 *reinterpret_cast<u32x4_t*>(st + kStageX + r * TBN + ((((pc >> 2) ^ ((r >> 1) & 1)) << 5) | ((pc & 3) << 3))) =
-                    oky[S][q] ? py[S][q] : z;
+                    wy[q];
               }
               // fragments by the LDS transpose read: within 16 lanes, lane c receives column c of a
               // 4 x 16 block whose rows the lanes address four-per-row
@@ -463,7 +524,7 @@ struct WindowKernel {
 #pragma unroll
               for (int q = 0; q < 2; q++) {
                 const int r = lane / PY + (64 / PY) * q, c = (lane % PY) * VEC;
-                *reinterpret_cast<u32x4_t*>(st + kStageX + r * TBN + (c ^ ((r & 1) << 5))) = oky[S][q] ? py[S][q] : z;
+                *reinterpret_cast<u32x4_t*>(st + kStageX + r * TBN + (c ^ ((r & 1) << 5))) = wy[q];
               }
               // fragments: lane l holds row 2 s + (l >> 5), column l & 31 of the block
               const int mg = lane >> 5, cl = lane & 31;
