@@ -5,8 +5,9 @@
 // however small M is (K = N = 10240: 105 M atomics, about 0.57 ms on MI355X, for a product
 // that takes microseconds).  Here a workgroup keeps dHW[w0, w0 + window) as an fp32 image in
 // LDS, finds the W tiles whose slice [off, off + BK*BN) meets that range by scanning the table
-// of tile offsets (hashed into the workspace by a small kernel of the same call; nothing is
-// kept between calls) and lists them, cut into strips of 32 rows, in ascending order.  Then
+// of tile offsets (hashed into the workspace by a small kernel of the same call) and lists them,
+// cut into strips of 32 rows, in ascending order — or, when the caller holds a layer plan, reads
+// that list from it (offsets and lists depend on the layer alone).  Then
 // every WAVEFRONT takes strips from the list on its own: it computes the whole X^T.dY product
 // of a strip — the operands are small and stay in L2; a wavefront fetches its own operand
 // pieces (16-bit types: 16-byte pieces through a small LDS area of its own and the LDS
@@ -562,16 +563,20 @@ struct WindowKernel {
       };
       if (my_tiles > 0) {
         // whole turns of the ring: the up to kDepth - 1 items past the end are padding (see fetch_next)
-        static_assert(kDepth >= 2 && kDepth <= 4, "the ring below is written out for up to four sets");
-        fetch_next(std::integral_constant<int, 0>{});
-        if constexpr (kDepth > 2) fetch_next(std::integral_constant<int, 1>{});
-        if constexpr (kDepth > 3) fetch_next(std::integral_constant<int, 2>{});
-        for (int i = 0; i < items; i += kDepth) {
-          item(std::integral_constant<int, 0>{});
-          item(std::integral_constant<int, 1>{});
-          if constexpr (kDepth > 2) item(std::integral_constant<int, 2>{});
-          if constexpr (kDepth > 3) item(std::integral_constant<int, 3>{});
-        }
+        static_assert(kDepth >= 2 && kDepth <= 8, "the ring below is written out for up to eight sets");
+        auto each_set = [&](auto&& f, auto count) {   // f(0), ..., f(count - 1) with compile-time arguments
+          constexpr int C = decltype(count)::value;
+          f(std::integral_constant<int, 0>{});
+          if constexpr (C > 1) f(std::integral_constant<int, 1>{});
+          if constexpr (C > 2) f(std::integral_constant<int, 2>{});
+          if constexpr (C > 3) f(std::integral_constant<int, 3>{});
+          if constexpr (C > 4) f(std::integral_constant<int, 4>{});
+          if constexpr (C > 5) f(std::integral_constant<int, 5>{});
+          if constexpr (C > 6) f(std::integral_constant<int, 6>{});
+          if constexpr (C > 7) f(std::integral_constant<int, 7>{});
+        };
+        each_set(fetch_next, std::integral_constant<int, kDepth - 1>{});
+        for (int i = 0; i < items; i += kDepth) each_set(item, std::integral_constant<int, kDepth>{});
         // (the padding items have left rubbish in the accumulators)
 #pragma unroll
         for (int a = 0; a < BI; a++)
