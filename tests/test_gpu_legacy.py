@@ -98,3 +98,24 @@ def test_legacy_module(oracle):
     assert sorted(m.state_dict().keys()) == ["bias", "random_numbers", "weight"]
     with pytest.raises(NotImplementedError):
         LegacyRzLinear(96, 80, 1, hw, tiled=False)
+
+
+def test_legacy_hash_through_the_fold_path_with_a_layer_plan(oracle, tuned, monkeypatch):
+    """hash_levels = 3 with the tiles folded by the second kernel: the tile offsets come from a layer
+    plan built with the legacy hash, or are hashed by the call itself — the same bits either way."""
+    from rzlinear_amd import _lib
+    from rzlinear_amd.impl.RzLinearBackward import weight_grad_hashed
+    tuned(fold=1, window=-1)
+    M, K, N, H = 96, 400, 336, 100000
+    _say("legacy fold + plan")
+    R = oracle.legacy_constants(5)
+    Rc = (ctypes.c_int32 * 8)(*R)
+    (x, _, dy), (x64, _, dy64) = make_inputs(M, K, N, H, torch.float32, seed=23)
+    assert _lib.plan_query(2, M, K, N, H, 16, 16, _lib.RZ_F32)["mode"] == "fold"
+    monkeypatch.setattr(_lib, "use_layer_plans", False)
+    a = weight_grad_hashed(x, dy, 1.0, M, K, N, H, Rc, 16, 16, hash_levels=_lib.HASH_LEGACY)[0]
+    monkeypatch.setattr(_lib, "use_layer_plans", True)
+    b = weight_grad_hashed(x, dy, 1.0, M, K, N, H, Rc, 16, 16, hash_levels=_lib.HASH_LEGACY)[0]
+    torch.cuda.synchronize()
+    assert torch.equal(a, b)
+    assert rel_err(b.cpu().numpy(), oracle.weight_grad(x64, dy64, H, 16, 16, R, 1.0, 3)) <= TOL[torch.float32]
