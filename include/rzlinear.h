@@ -73,7 +73,8 @@ typedef enum rz_hash {
  * No counterpart in the reference, whose tile choice is the autotuner's.
  */
 typedef struct rz_tuning {
-  int tile;       /* C-tile edge of the contraction kernels: 0 = automatic, 64, 128 or 256 */
+  int tile;       /* C-tile edge of the contraction kernels: 0 = automatic, 64, 128 or 256; 32 = the 32 x 64
+                     tile of fp32 forward / input-grad (elsewhere it reads as 64) */
   int stages;     /* 0 = automatic, 1 = the single-stage form of the 128 tile */
   int lds_image;  /* weight-grad: 0 = automatic, -1 = never sum tiles in an LDS image of dHW */
   int window;     /* weight-grad: 0 = automatic, 1 = dHW by windows whenever possible, -1 = never */

@@ -68,23 +68,23 @@ static hipError_t launch_one(GemmParams p, const WeightGradPlan* plan, const Spl
 // FULL kernels carry no bounds checks: every tile and every R step must be complete.  Ragged
 // shapes: 16-bit tiles can still be staged directly, with edge pieces fetched from inside the
 // operands (CLAMP); everything else takes the bounds-checked kernel.
-template <typename T, int OP, int TILE, int WI, int WJ, int NSTAGE, bool COLSUM = false, int WK = 1>
+template <typename T, int OP, int TILE, int WI, int WJ, int NSTAGE, bool COLSUM = false, int WK = 1, int TILE_J = TILE>
 static hipError_t launch_tile(GemmParams p, const WeightGradPlan* plan, const SplitPlan* split,
                               const KernelForm& form, hipStream_t stream) {
   // (the form was derived on the host from the same rules that select the instantiation here:
   //  refuse to launch if the two ever disagree about the step length)
   if (form.full) {
-    if (form.step != GemmKernel<T, OP, TILE, TILE, WI, WJ, NSTAGE, true>::TR) return hipErrorInvalidValue;
-    return launch_one<T, OP, TILE, TILE, WI, WJ, NSTAGE, true, COLSUM, false, WK>(p, plan, split, stream);
+    if (form.step != GemmKernel<T, OP, TILE, TILE_J, WI, WJ, NSTAGE, true>::TR) return hipErrorInvalidValue;
+    return launch_one<T, OP, TILE, TILE_J, WI, WJ, NSTAGE, true, COLSUM, false, WK>(p, plan, split, stream);
   }
   if constexpr (sizeof(T) == 2 && NSTAGE == 2 && TILE >= 128) {
     if (form.clamp) {
-      if (form.step != GemmKernel<T, OP, TILE, TILE, WI, WJ, NSTAGE, false, false, true>::TR) return hipErrorInvalidValue;
-      return launch_one<T, OP, TILE, TILE, WI, WJ, NSTAGE, false, COLSUM, true>(p, plan, split, stream);
+      if (form.step != GemmKernel<T, OP, TILE, TILE_J, WI, WJ, NSTAGE, false, false, true>::TR) return hipErrorInvalidValue;
+      return launch_one<T, OP, TILE, TILE_J, WI, WJ, NSTAGE, false, COLSUM, true>(p, plan, split, stream);
     }
   }
-  if (form.clamp || form.step != GemmKernel<T, OP, TILE, TILE, WI, WJ, NSTAGE, false>::TR) return hipErrorInvalidValue;
-  return launch_one<T, OP, TILE, TILE, WI, WJ, NSTAGE, false, COLSUM, false, WK>(p, plan, split, stream);
+  if (form.clamp || form.step != GemmKernel<T, OP, TILE, TILE_J, WI, WJ, NSTAGE, false>::TR) return hipErrorInvalidValue;
+  return launch_one<T, OP, TILE, TILE_J, WI, WJ, NSTAGE, false, COLSUM, false, WK>(p, plan, split, stream);
 }
 
 template <typename T, int TILE, int WI, int WJ, int NSTAGE, int WK = 1>
@@ -112,6 +112,7 @@ static hipError_t launch_op(int op, GemmParams p, const WeightGradPlan* plan, co
 //        instead of a pipeline (tuning aid)
 //    64:  64 x  64, four wavefronts of 32 x 32, for problems with few tiles; fp32 forward /
 //        input-grad: eight, in two groups that share every R step between them
+//    32:  32 x  64 (fp32 forward / input-grad of at most 32 rows): four wavefronts of 32 x 32 in two such groups
 template <typename T>
 static hipError_t launch_gemm_t(int op, GemmParams p, const WeightGradPlan* plan, const SplitPlan* split,
                                 const rz_tuning& tuning, hipStream_t stream) {
@@ -126,6 +127,12 @@ static hipError_t launch_gemm_t(int op, GemmParams p, const WeightGradPlan* plan
     case 6442: return launch_op<T, 64, 2, 2, 2>(op, p, plan, split, form, stream);
     case 6482:   // fp32 forward / input-grad: two groups of four wavefronts share every R step
       if constexpr (sizeof(T) == 4) return launch_op<T, 64, 2, 2, 2, 2>(op, p, plan, split, form, stream);
+      return hipErrorInvalidValue;
+    case 3242:   // fp32 forward / input-grad of at most 32 rows: 32 x 64, two groups of two wavefronts
+      if constexpr (sizeof(T) == 4) {
+        if (op == kForward) return launch_tile<T, kForward, 32, 1, 2, 2, false, 2, 64>(p, plan, split, form, stream);
+        if (op == kInputGrad) return launch_tile<T, kInputGrad, 32, 1, 2, 2, false, 2, 64>(p, plan, split, form, stream);
+      }
       return hipErrorInvalidValue;
     case 12841: return launch_op<T, 128, 2, 2, 1>(op, p, plan, split, form, stream);
     case 12882: return launch_op<T, 128, 2, 4, 2>(op, p, plan, split, form, stream);

@@ -16,7 +16,7 @@ static inline rz_tuning tuning_or_default(const rz_tuning* t) {
   return t != nullptr ? *t : d;
 }
 static inline bool tuning_valid(const rz_tuning& t) {
-  return (t.tile == 0 || t.tile == 64 || t.tile == 128 || t.tile == 256) && (t.stages == 0 || t.stages == 1) &&
+  return (t.tile == 0 || t.tile == 32 || t.tile == 64 || t.tile == 128 || t.tile == 256) && (t.stages == 0 || t.stages == 1) &&
          (t.lds_image == 0 || t.lds_image == -1) && (t.window >= -1 && t.window <= 1) &&
          (t.split == 0 || t.split == -1) && (t.clamp == 0 || t.clamp == -1) &&
          (t.fold >= -1 && t.fold <= 1) && t.reserved == 0;
@@ -46,8 +46,11 @@ static inline int slice_unit(int tile, int elem_bytes) {
   return ((tile == 128 && elem_bytes == 2) ? 256 : 128) / elem_bytes;
 }
 
+// Tile codes: 64, 128, 256 are square C tiles; 32 stands for the 32 x 64 tile of the fp32 forward /
+// input-grad kernels for batches of at most 32 rows (half of a 64-row tile would be padding).
+static inline int tile_cols(int t) { return t == 32 ? 64 : t; }
 static inline long long tile_count(int I, int J, int t) {
-  return (long long)((I + t - 1) / t) * ((J + t - 1) / t);
+  return (long long)((I + t - 1) / t) * ((J + tile_cols(t) - 1) / tile_cols(t));
 }
 
 // Rate of `wgs` equal workgroups on the chip relative to a full one, when a compute unit runs at
@@ -93,6 +96,8 @@ static inline double tile_score(int I, int J, int t, int elem_bytes) {
 // a workgroup count that includes the slices of a cut contraction).
 static inline double tile_rate(double wgs, int t, int elem_bytes) {
   const bool f32 = elem_bytes == 4;
+  // (32 x 64, four wavefronts: half a 64 workgroup's work in about its time, up to eight resident)
+  if (t == 32) return occupancy_rate(wgs, 8, 0.40, 0.80);
   const int slots = (t == 256) ? 1 : (t == 128 ? 2 : 4);
   const double lo = (t == 256) ? 1.0 : (t == 128 ? (f32 ? 0.86 : 0.51) : (f32 ? 0.60 : 0.16));
   const double hi = (t == 256) ? 1.0 : (t == 128 ? (f32 ? 0.90 : 0.75) : (f32 ? 0.80 : 0.33));
@@ -101,7 +106,7 @@ static inline double tile_rate(double wgs, int t, int elem_bytes) {
 
 // C-tile edge for a contraction with an I x J result: the best-scoring of 256, 128, 64.
 static inline int pick_tile(int I, int J, int elem_bytes, const rz_tuning& tuning) {
-  if (tuning.tile) return tuning.tile;
+  if (tuning.tile) return (tuning.tile == 32 && elem_bytes != 4) ? 64 : tuning.tile;
   int best = 256;
   double best_score = tile_score(I, J, 256, elem_bytes);
   const int others[2] = {128, 64};
@@ -199,7 +204,7 @@ static inline WeightGradPlan plan_weight_grad(int M, int K, int N, int H, int BK
   const int pitch = (H + 3) & ~3;
   const bool image = t.lds_image != -1 && (size_t)pitch * sizeof(float) <= kMaxImageBytes;
   if (t.tile) {
-    pl.tile = t.tile;
+    pl.tile = t.tile == 32 ? 64 : t.tile;   // (the 32 x 64 tile serves forward / input-grad only)
   } else if (image) {
     // with the LDS image the M loop can be cut freely (a slice costs one partial image), so
     // the pipelined 256 tile is used unless it would mostly compute padding
@@ -425,13 +430,16 @@ static inline SplitPlan plan_split(int I, int J, int R, int elem_bytes, const rz
   SplitPlan best = {};
   double best_us = 0.0;
   const double peak = elem_bytes == 4 ? 137e6 : 1150e6;   // flop per microsecond of the 256 tile on a full chip
-  const int tiles_of[3] = {256, 128, 64};
+  const int tiles_of[4] = {256, 128, 64, 32};
+  // (an override that asks for the 32 x 64 tile where it does not exist gets the 64 tile)
+  const int forced = (t.tile == 32 && elem_bytes != 4) ? 64 : t.tile;
   for (int tile : tiles_of) {
-    if (t.tile && tile != t.tile) continue;
+    if (forced && tile != forced) continue;
+    if (tile == 32 && !forced && (elem_bytes != 4 || I > 32)) continue;
     const int TR = slice_unit(tile, elem_bytes);
     const long long tiles = tile_count(I, J, tile);
     const int r_steps = (R + TR - 1) / TR;
-    const double useful = (double)I * (double)J / ((double)tiles * tile * tile);
+    const double useful = (double)I * (double)J / ((double)tiles * tile * tile_cols(tile));
     for (int want = 1; want <= 16; want++) {
       if (want > 1 && t.split == -1) break;
       const int steps_per = (r_steps + want - 1) / want;
@@ -477,12 +485,13 @@ static inline KernelForm kernel_form(int op, int I, int J, int R, int chunk, int
   // 64 tile: four wavefronts; fp32 forward / input-grad take eight (two groups that share every R
   // step: a second wavefront per SIMD keeps the MFMA pipe fed while the first waits for LDS)
   f.waves = tile == 256 ? 8
+            : tile == 32 ? 4
             : tile == 64 ? ((elem_bytes == 4 && op != kWeightGrad) ? 8 : 4)
                          : (f.stages == 1 ? 4 : (workgroups <= kComputeUnits * 3 / 2 ? 8 : 4));
   const bool direct_capable = elem_bytes == 2 && f.stages == 2 && tile >= 128;
   const int step_plain = 128 / elem_bytes;
   const int step_direct = (direct_capable && tile == 128 && f.waves == 8) ? 256 / elem_bytes : step_plain;
-  f.full = (I % tile == 0) && (J % tile == 0) && (R % step_direct == 0) && (chunk % step_direct == 0);
+  f.full = (I % tile == 0) && (J % tile_cols(tile) == 0) && (R % step_direct == 0) && (chunk % step_direct == 0);
   // a plain operand's 16-byte pieces must not straddle the end of its rows: forward / input-grad
   // need R, weight-grad needs I and J, to be multiples of the piece
   const int vec = 16 / elem_bytes;

@@ -129,7 +129,7 @@ TILE_CASES = [
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=lambda d: str(d).split(".")[-1])
-@pytest.mark.parametrize("env", [{"tile": 64}, {"tile": 128}, {"tile": 256}, {"tile": 128, "stages": 1},
+@pytest.mark.parametrize("env", [{"tile": 32}, {"tile": 64}, {"tile": 128}, {"tile": 256}, {"tile": 128, "stages": 1},
                                  {"tile": 256, "lds_image": -1}],
                          ids=lambda e: "-".join("%s=%s" % (k, v) for k, v in e.items()))
 @pytest.mark.parametrize("shape", TILE_CASES, ids=lambda s: "x".join(map(str, s)))
@@ -149,6 +149,31 @@ def test_every_tile_shape_and_scatter_mode(oracle, shape, env, dtype):
     assert rel_err(y.float().cpu().numpy(), oracle.forward(x64, hw64, N, BK, BN, R1024)) <= TOL[dtype]
     assert rel_err(dx.float().cpu().numpy(), oracle.input_grad(dy64, hw64, K, BK, BN, R1024)) <= TOL[dtype]
     assert rel_err(dhw.float().cpu().numpy(), oracle.weight_grad(x64, dy64, H, BK, BN, R1024)) <= TOL[dtype]
+
+
+@pytest.mark.parametrize("split", [0, -1], ids=["cut", "whole"])
+@pytest.mark.parametrize("shape", [(32, 1536, 2048, 200000, 64, 64), (17, 100, 150, 5000, 32, 64),
+                                   (8, 4096, 320, 70000, 64, 64), (32, 10240, 1024, 1 << 20, 64, 64),
+                                   (1, 64, 64, 8192, 64, 64)], ids=lambda s: "x".join(map(str, s)))
+def test_fp32_batches_of_at_most_32_rows_take_the_32_row_tile(oracle, shape, split):
+    """The 32 x 64 tile of fp32 forward / input-grad (for M <= 32 a 64-row tile is half padding;
+    large problems choose it by themselves), with and without a cut contraction, with a bias."""
+    from rzlinear_amd import _lib
+    from rzlinear_amd.impl.RzLinearBackward import rz_linear_backward_input_grad_tl
+    from rzlinear_amd.impl.RzLinearForward import rz_linear_forward_bias_tl
+    M, K, N, H, BK, BN = shape
+    _say("32-row tile", shape, split)
+    (x, hw, dy), (x64, hw64, dy64) = make_inputs(M, K, N, H, torch.float32, seed=12)
+    bias = torch.randn((N,), generator=torch.Generator().manual_seed(3))
+    tn = dict(split=split) if split else {}
+    with _lib.tuning(tile=32, **tn):
+        assert _lib.plan_query(1, M, K, N, H, BK, BN, _lib.RZ_F32)["tile"] == 32
+        y = rz_linear_forward_bias_tl(x, hw, bias.cuda(), 0.5, M, K, N, H, *rargs(R1024), BLOCK_SIZE_K=BK, BLOCK_SIZE_N=BN)
+        dx = rz_linear_backward_input_grad_tl(dy, hw, 0.5, M, K, N, H, *rargs(R1024), BLOCK_SIZE_K=BK, BLOCK_SIZE_N=BN)
+    torch.cuda.synchronize()
+    ref = oracle.forward(x64, hw64, N, BK, BN, R1024, 0.5) + bias.double().numpy()[None, :]
+    assert rel_err(y.cpu().numpy(), ref) <= TOL[torch.float32]
+    assert rel_err(dx.cpu().numpy(), oracle.input_grad(dy64, hw64, K, BK, BN, R1024, 0.5)) <= TOL[torch.float32]
 
 
 def test_kernels_match_vectors_produced_by_the_reference_kernels():
