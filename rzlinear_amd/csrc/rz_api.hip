@@ -117,21 +117,23 @@ __global__ void convert_from_f32_kernel(const float* __restrict__ src, T* __rest
 }
 
 // dHW[h] = sum over the partial images of part[p][h] (+ dHW[h] when ACC), converted to the
-// element type.  A workgroup of 256 threads owns 16 groups of four slots; 16 thread groups each
-// add up every 16th partial image, then the groups are combined through LDS in a fixed order,
-// so the result does not depend on scheduling.
-template <typename T, bool ACC>
+// element type.  A workgroup of 256 threads owns 256 / GROUPS groups of four slots; GROUPS thread
+// groups each add up every GROUPS-th partial image (all their loads in flight together when
+// there are at most eight each), then the groups are combined through LDS in a fixed order, so the
+// result does not depend on scheduling.
+template <typename T, bool ACC, int GROUPS>
 __global__ __launch_bounds__(256) void reduce_partials_kernel(const float* __restrict__ part,
                                                               T* __restrict__ out, int H, int pitch,
                                                               int nparts) {
-  __shared__ float4 sums[16][16];
-  const int q = threadIdx.x & 15, g = threadIdx.x >> 4;
-  const int slot = (blockIdx.x * 16 + q) * 4;
+  constexpr int kSlots = 256 / GROUPS;
+  __shared__ float4 sums[GROUPS][kSlots];
+  const int q = threadIdx.x % kSlots, g = threadIdx.x / kSlots;
+  const int slot = (blockIdx.x * kSlots + q) * 4;
   float4 s = {0.f, 0.f, 0.f, 0.f};
   if (slot < pitch) {
     // eight loads in flight per thread; the order of the additions stays fixed
 #pragma unroll 8
-    for (int p = g; p < nparts; p += 16) {
+    for (int p = g; p < nparts; p += GROUPS) {
       const float4 v = *reinterpret_cast<const float4*>(part + (size_t)p * pitch + slot);
       s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
     }
@@ -139,7 +141,7 @@ __global__ __launch_bounds__(256) void reduce_partials_kernel(const float* __res
   sums[g][q] = s;
   __syncthreads();
   if (g == 0 && slot < pitch) {
-    for (int i = 1; i < 16; i++) {
+    for (int i = 1; i < GROUPS; i++) {
       const float4 v = sums[i][q];
       s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
     }
@@ -276,13 +278,16 @@ static hipError_t zero_words(void* p, size_t bytes, hipStream_t s) {
 template <bool ACC>
 static void launch_reduce_partials(int out_dtype, const float* part, void* out, int H, int pitch, int nparts,
                                    hipStream_t s) {
-  const dim3 grid((pitch / 4 + 15) / 16), block(256);
+  // (16 groups of 16 slots; 32 groups of 8 slots — twice the workgroups, every load of a thread in
+  //  flight at once — were no faster: 7.0 against 5.7 us for 256 images of 67 KB)
+  constexpr int GROUPS = 16, kSlots = 256 / GROUPS;
+  const dim3 grid((pitch / 4 + kSlots - 1) / kSlots), block(256);
   if (out_dtype == RZ_F32)
-    hipLaunchKernelGGL((reduce_partials_kernel<float, ACC>), grid, block, 0, s, part, (float*)out, H, pitch, nparts);
+    hipLaunchKernelGGL((reduce_partials_kernel<float, ACC, GROUPS>), grid, block, 0, s, part, (float*)out, H, pitch, nparts);
   else if (out_dtype == RZ_BF16)
-    hipLaunchKernelGGL((reduce_partials_kernel<bf16_t, ACC>), grid, block, 0, s, part, (bf16_t*)out, H, pitch, nparts);
+    hipLaunchKernelGGL((reduce_partials_kernel<bf16_t, ACC, GROUPS>), grid, block, 0, s, part, (bf16_t*)out, H, pitch, nparts);
   else
-    hipLaunchKernelGGL((reduce_partials_kernel<f16_t, ACC>), grid, block, 0, s, part, (f16_t*)out, H, pitch, nparts);
+    hipLaunchKernelGGL((reduce_partials_kernel<f16_t, ACC, GROUPS>), grid, block, 0, s, part, (f16_t*)out, H, pitch, nparts);
 }
 
 // Enqueues the fold kernel for tiles of `loads` * 1024 elements (smaller tiles: loads = 1).
@@ -541,7 +546,7 @@ extern "C" {
 
 #define RZ_API __attribute__((visibility("default")))
 
-RZ_API int rz_version(void) { return 300; }
+RZ_API int rz_version(void) { return 400; }
 
 RZ_API const char* rz_status_string(int status) {
   switch (status) {
