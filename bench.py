@@ -78,10 +78,10 @@ TRAFFIC = {
     },
     ("ffn", "bf16"): {
         "profile": "profiles/rz_gemm_fold_bf16_ffn.txt",
-        "bytes": {"forward": int((71090.8 * 2.0 + 262144.0) * 1024),      # algorithmic: 320.1 MiB
-                  "input_grad": int((132349.0 * 2.0 + 65536.0) * 1024),
+        "bytes": {"forward": int((71071.4 * 2.0 + 262144.0) * 1024),      # algorithmic: 320.1 MiB
+                  "input_grad": int((132344.1 * 2.0 + 65536.0) * 1024),
                   # contraction (X, dY re-read by the XCDs' tile groups; X^T.dY written tile by tile: 256 MiB)
-                  "weight_grad": int((786642.5 * 2.0 + 262144.0) * 1024)},
+                  "weight_grad": int((786592.1 * 2.0 + 262144.0) * 1024)},
     },
 }
 
