@@ -364,7 +364,8 @@ static inline WindowPlan plan_window(int M, int K, int N, int H, int BK, int BN,
   // operands of every tile come out of L2 again: tiles that share a window share no rows or
   // columns of W; a wavefront has three groups of rows in flight, which is what its registers hold).
   const double chunks = (double)((M + 31) / 32);
-  const double per_wg = (double)tiles * ((double)w + (double)BK * BN) / (double)H;
+  // (in units of 64-row tiles, i.e. of two strips: the figures below were fitted on those)
+  const double per_wg = (double)tiles * ((double)w + (double)BK * BN) / (double)H * ((double)BK / 64.0);
   const double wg_rounds = (double)((pl.windows + kComputeUnits - 1) / kComputeUnits);
   const double t_window = wg_rounds * per_wg * ((elem_bytes == 4 ? 0.43 + 0.63 * chunks : 0.31 + 0.18 * chunks)) + (planned ? 5.0 : 28.0);
   // ... against what the contraction kernel's plan would take: the fold, or the atomic scatter
