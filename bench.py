@@ -31,7 +31,8 @@ if ROOT not in sys.path:
 
 HASH_SEED_1024 = [45007, 20011, 38363, 15263, 24507, 36489, 12234, 43027]
 
-# name -> (M, K, N, H, default dtype, input distributions); tiles are 64x64 throughout.
+# name -> (M, K, N, H, default dtype, input distributions[, (BLOCK_K, BLOCK_N)]); tiles are 64x64 (what the
+# baseline configurations ask for) except on the reference's own grid, which runs its launchers' defaults.
 # "normal": X ~ N(0,1), dY ~ N(0,1); "relu": X = relu(N(0,1)), dY ~ N(0, variance 1e-2).
 WORKLOADS = {
     "square4096": (4096, 4096, 4096, 16778, "bf16", "normal"),      # the metric's configuration
@@ -41,14 +42,14 @@ WORKLOADS = {
     "rec_mlp": (16384, 512, 1024, 5243, "bf16", "relu"),
     "ffn": (8192, 4096, 16384, 67109, "bf16", "normal"),
     "collision": (32768, 2048, 2048, 32768, "fp32", "normal"),
-    # the shape grid of the reference's own benchmark script (python/bench/bench.py:10-11),
-    # with its default compress_ratio 0.0625
-    "grid_32_1024": (32, 1024, 1024, 65536, "fp32", "normal"),
-    "grid_128_1024": (128, 1024, 1024, 65536, "fp32", "normal"),
-    "grid_1024_1024": (1024, 1024, 1024, 65536, "fp32", "normal"),
-    "grid_32_10240": (32, 10240, 10240, 6553600, "fp32", "normal"),
-    "grid_128_10240": (128, 10240, 10240, 6553600, "fp32", "normal"),
-    "grid_1024_10240": (1024, 10240, 10240, 6553600, "fp32", "normal"),
+    # the shape grid of the reference's own benchmark script (python/bench/bench.py:10-11), with its
+    # default compress_ratio 0.0625 and its launchers' default tile (BLOCK_SIZE_K = 32, BLOCK_SIZE_N = 64)
+    "grid_32_1024": (32, 1024, 1024, 65536, "fp32", "normal", (32, 64)),
+    "grid_128_1024": (128, 1024, 1024, 65536, "fp32", "normal", (32, 64)),
+    "grid_1024_1024": (1024, 1024, 1024, 65536, "fp32", "normal", (32, 64)),
+    "grid_32_10240": (32, 10240, 10240, 6553600, "fp32", "normal", (32, 64)),
+    "grid_128_10240": (128, 10240, 10240, 6553600, "fp32", "normal", (32, 64)),
+    "grid_1024_10240": (1024, 10240, 10240, 6553600, "fp32", "normal", (32, 64)),
 }
 # the baseline configurations beside the headline one: (workload, dtype) rows of the sweep
 SWEEP = [("cpu_ref_1024", "fp32"), ("square1024", "fp32"), ("square1024", "bf16"), ("square2048", "fp32"),
@@ -88,11 +89,11 @@ TRAFFIC = {
 
 def make_workload(torch, _lib, name, dname, dev):
     """Resident inputs, outputs and workspaces of one workload and its three legs."""
-    M, K, N, H, _, dist = WORKLOADS[name]
+    M, K, N, H, _, dist = WORKLOADS[name][:6]
+    BK, BN = WORKLOADS[name][6] if len(WORKLOADS[name]) > 6 else (64, 64)
     dtype = {"bf16": torch.bfloat16, "fp16": torch.float16, "fp32": torch.float32}[dname]
     code = {"bf16": _lib.RZ_BF16, "fp16": _lib.RZ_F16, "fp32": _lib.RZ_F32}[dname]
     lib = _lib.load()
-    BK = BN = 64
     R = (ctypes.c_int32 * 8)(*HASH_SEED_1024)
     g = torch.Generator().manual_seed(1024)
     x = torch.randn((M, K), generator=g)
