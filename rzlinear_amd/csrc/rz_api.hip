@@ -290,30 +290,19 @@ static void launch_reduce_partials(int out_dtype, const float* part, void* out, 
     hipLaunchKernelGGL((reduce_partials_kernel<f16_t, ACC, GROUPS>), grid, block, 0, s, part, (f16_t*)out, H, pitch, nparts);
 }
 
-// Enqueues the fold kernel for tiles of `loads` * 1024 elements (smaller tiles: loads = 1).
-static hipError_t launch_fold(const FoldParams& fp, int loads, hipStream_t s) {
-  static std::atomic<uint64_t> raised[5];
+static hipError_t launch_fold(const FoldParams& fp, hipStream_t s) {
+  static std::atomic<uint64_t> raised{0};
   const size_t lds = fold_lds_bytes(fp.window);
-  if ((fp.partial == nullptr && (fp.shares != 1 || fp.out == nullptr)) || fp.window <= 0 || fp.window % kFoldThreads != 0 || fp.window > kFoldWindowMax || fp.slices > kFoldList ||
-      (long long)fp.windows * fp.window < fp.H)
+  const int E = fp.h.BK * fp.h.BN, runs = E > kFoldRun ? E / kFoldRun : 1;
+  if ((fp.partial == nullptr && (fp.shares != 1 || fp.out == nullptr)) || fp.window <= 0 || fp.window % kFoldThreads != 0 || fp.window > kFoldWindowMax ||
+      fp.slices * runs * 4 > kFoldList || runs > 8 || fp.h.BK > 16384 || fp.h.BN > 16384 || (long long)fp.windows * fp.window < fp.H)
     return hipErrorInvalidValue;
-  const dim3 grid((unsigned)(fp.windows * fp.shares)), block(kFoldThreads);
-  auto go = [&](auto kernel, int slot) -> hipError_t {
-    if (lds > 64 * 1024) {
-      hipError_t e = raise_lds_limit(reinterpret_cast<const void*>(kernel), raised[slot]);
-      if (e != hipSuccess) return e;
-    }
-    hipLaunchKernelGGL(kernel, grid, block, lds, s, fp);
-    return hipGetLastError();
-  };
-  switch (loads) {
-    case 1: return go(fold_tiles_kernel<1>, 0);
-    case 2: return go(fold_tiles_kernel<2>, 1);
-    case 4: return go(fold_tiles_kernel<4>, 2);
-    case 8: return go(fold_tiles_kernel<8>, 3);
-    case 16: return go(fold_tiles_kernel<16>, 4);
-    default: return hipErrorInvalidValue;
+  if (lds > 64 * 1024) {
+    hipError_t e = raise_lds_limit(reinterpret_cast<const void*>(fold_tiles_kernel), raised);
+    if (e != hipSuccess) return e;
   }
+  hipLaunchKernelGGL(fold_tiles_kernel, dim3((unsigned)(fp.windows * fp.shares)), dim3(kFoldThreads), lds, s, fp);
+  return hipGetLastError();
 }
 
 template <bool ACC>
@@ -445,7 +434,7 @@ static int weight_grad_impl(const void* X, const void* dY, void* dHW, void* dbia
     // the tiles), and the shares' images are added up (no atomics, fixed summation order)
     const FoldPlan& f = plan.fold;
     p.scatter = nullptr;
-    p.tiles_out = (float*)workspace;
+    p.tiles_out = (float*)((char*)workspace + kFoldMarginBytes);   // (the fold kernel's loads reach a few floats beyond the tiles)
     p.out_tiles_k = (K + BK - 1) / BK;
     p.out_tiles_n = (N + BN - 1) / BN;
     if (launch_gemm(dtype, kWeightGrad, p, &plan, nullptr, tuning, s) != hipSuccess) return RZ_ERR_LAUNCH;
@@ -475,7 +464,7 @@ static int weight_grad_impl(const void* X, const void* dY, void* dHW, void* dbia
     fp.window = f.window;
     fp.windows = f.windows;
     fp.shares = f.shares;
-    if (launch_fold(fp, f.loads, s) != hipSuccess) return RZ_ERR_LAUNCH;
+    if (launch_fold(fp, s) != hipSuccess) return RZ_ERR_LAUNCH;
     if (f.shares > 1) {
       if (accumulate) launch_reduce_partials<true>(dhw_dtype, fp.partial, dHW, H, fp.pitch, f.shares, s);
       else launch_reduce_partials<false>(dhw_dtype, fp.partial, dHW, H, fp.pitch, f.shares, s);

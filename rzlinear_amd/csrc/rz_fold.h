@@ -6,11 +6,20 @@
 // additions is fixed (the order of the workgroup's tile list), so the result is the same on every call.
 //
 // A hashed tile is BK*BN contiguous elements of hashed_weight and BK*BN contiguous floats of the
-// tile-by-tile buffer (of which only the part inside K x N is read), so its reads are whole cache lines whatever its offset.  Inside the
-// workgroup thread i owns the window positions i, i + 1024, i + 2048, ...: for every tile it
-// reads the elements that fall on its own positions (consecutive threads, consecutive addresses)
-// and adds them with plain LDS read-add-write.  No two threads ever touch the same LDS word, so
-// no barrier is needed between tiles.
+// tile-by-tile buffer, so its reads are whole cache lines whatever its offset.  The list holds
+// the tiles in runs of at most 2048 floats.  The window is cut into blocks of 256 positions;
+// wavefront w owns the blocks w, w + 16, w + 32, ..., and inside a block lane l owns the four
+// positions 4 l .. 4 l + 3.  A run meets at most nine blocks in a row, so at most one of a
+// wavefront's: the wavefront walks down the list, skips the runs that miss its blocks, and for
+// each of the others reads the 256 floats that fall on its block with ONE 16-byte load per lane
+// (from a scalar base: the run starts anywhere, on a 4-byte boundary) and adds them with one
+// 16-byte LDS read, four additions and one 16-byte LDS write per lane.  What a run needs per
+// wavefront is scalar arithmetic; no two lanes ever touch the same LDS word, so the wavefronts
+// need no barrier between runs and each goes down the list at its own pace.  Only the blocks
+// at the two ends of a run, and runs of tiles that stick out of K x N (whose buffer holds floats
+// that the contraction never wrote), need their elements masked one by one: a branch of its
+// own.  The loads reach up to 258 floats before and after a run: the buffer is allocated with a
+// margin on both sides.
 //
 // A window is at most 32768 floats (128 KB of LDS).  When hashed_weight has fewer windows than
 // the chip has compute units, `shares` workgroups share a window: each takes an equal part of the
@@ -41,42 +50,55 @@ struct FoldParams {
 };
 
 static constexpr int kFoldThreads = 1024;
-static constexpr int kFoldList = 2048;       // entries of the tile list in LDS
+static constexpr int kFoldList = 2048;       // entries of the run list in LDS
 static constexpr int kFoldScan = 32;         // tile indices per thread and listing pass
 static constexpr int kFoldWindowMax = 32768;
+static constexpr int kFoldRun = 2048;        // floats of a run at most (tiles are powers of two: whole runs)
+static constexpr int kFoldRound = 8;         // runs whose loads a wavefront issues together
+static constexpr int kFoldBlock = 256;       // window positions of a wavefront's block: four per lane
 
 static inline size_t fold_lds_bytes(int window) {
   return (size_t)window * sizeof(float) + 3 * kFoldList * sizeof(int) + 32 * sizeof(int);
 }
 
-// LPE: loads per list entry and thread, BK*BN / 1024 (1 for smaller tiles: then only the first
-// BK*BN threads of an entry have an element).  A round of 16 loads per thread is issued before
-// its additions.
-template <int LPE>
+typedef float fold_f4 __attribute__((ext_vector_type(4)));
+typedef float fold_f4u __attribute__((ext_vector_type(4), aligned(4)));
+
 __global__ __launch_bounds__(kFoldThreads) void fold_tiles_kernel(const FoldParams p) {
   extern __shared__ __align__(16) float fold_lds[];
   float* img = fold_lds;
-  int* list_at = reinterpret_cast<int*>(fold_lds + p.window);   // first float of the entry's tile
-  int* list_rel = list_at + kFoldList;                           // where the tile starts, relative to the window
-  int* list_lim = list_rel + kFoldList;                          // rows | columns << 16 of the tile inside K x N
+  int* list_at = reinterpret_cast<int*>(fold_lds + p.window);   // first float of the run in the buffer
+  int* list_rel = list_at + kFoldList;                           // where the run starts, relative to the window
+  int* list_lim = list_rel + kFoldList;                          // (rows - 1) | (columns - 1) << 14 of the tile inside K x N | run << 28
   int* wave_sum = list_lim + kFoldList;                          // [16] per-wavefront counts, [16] = total
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int lane4 = lane * 4;
+  const unsigned lane16 = lane * 16;
   const int win = blockIdx.x % p.windows, share = blockIdx.x / p.windows;
   const int w0 = win * p.window;
   const int wlen = (p.H - w0) < p.window ? (p.H - w0) : p.window;
   const int E = p.h.BK * p.h.BN, eshift = p.h.bk_shift + p.h.bn_shift;
   const int ntiles = p.tiles_k * p.tiles_n;
+  const int run = E < kFoldRun ? E : kFoldRun, runs = E / run;   // (E is a power of two)
+  const int per_tile = p.slices * runs;                          // list entries of a tile
+  const int full_lim = (p.h.BK - 1) | (p.h.BN - 1) << 14;
   for (int q = tid; q < p.window; q += kFoldThreads) img[q] = 0.f;   // (own positions only)
 
-  // bit j: tile first + i + 1024 j (below `stop`) lands in the window; the offsets are fetched together
+  // bit j: tile first + i + 1024 j (below `stop`) lands in the window.  The offsets are fetched
+  // together, by loads that depend on no condition (one load under a branch per index would
+  // cost a round trip to the L2 each).
   auto scan = [&](int first, int stop) -> unsigned {
+    int rel[kFoldScan];
+#pragma unroll
+    for (int j = 0; j < kFoldScan; j++) {
+      const int id = first + tid + j * kFoldThreads;
+      rel[j] = p.offsets[id < stop ? id : stop - 1];
+    }
     unsigned mask = 0u;
 #pragma unroll
     for (int j = 0; j < kFoldScan; j++) {
-      // (no branch around the loads: they are issued together)
-      const int id = first + tid + j * kFoldThreads;
-      const int rel = p.offsets[id < stop ? id : stop - 1] - w0;
-      mask |= (id < stop && rel > -E && rel < wlen) ? 1u << j : 0u;
+      const int id = first + tid + j * kFoldThreads, r = rel[j] - w0;
+      mask |= (unsigned)((id < stop) & (r > -E) & (r < wlen)) << j;
     }
     return mask;
   };
@@ -127,8 +149,8 @@ __global__ __launch_bounds__(kFoldThreads) void fold_tiles_kernel(const FoldPara
     const int found = total_of(incl, &before);
     const int want_lo = rank_lo > seen ? rank_lo : seen;
     const int want_hi = rank_hi < seen + found ? rank_hi : seen + found;
-    const int total = (want_hi > want_lo ? want_hi - want_lo : 0) * p.slices;
-    if (total > kFoldList) {   // does not fit: look at half the range (a range of kFoldList / slices tiles always fits)
+    const int total = (want_hi > want_lo ? want_hi - want_lo : 0) * per_tile;
+    if (total > kFoldList) {   // does not fit: look at half the range (a range of kFoldList / per_tile >= 4 tiles always fits)
       span = (span + 1) / 2;
       continue;
     }
@@ -142,83 +164,104 @@ __global__ __launch_bounds__(kFoldThreads) void fold_tiles_kernel(const FoldPara
         const int tk = id / p.tiles_n, tn = id - tk * p.tiles_n;
         const int rows = (p.K - tk * p.h.BK) < p.h.BK ? (p.K - tk * p.h.BK) : p.h.BK;
         const int cols = (p.N - tn * p.h.BN) < p.h.BN ? (p.N - tn * p.h.BN) : p.h.BN;
-        for (int s = 0; s < p.slices; s++) {
-          list_at[(rank - want_lo) * p.slices + s] = (s * ntiles + id) << eshift;
-          list_rel[(rank - want_lo) * p.slices + s] = rel;
-          list_lim[(rank - want_lo) * p.slices + s] = rows | cols << 16;
-        }
+        for (int s = 0; s < p.slices; s++)
+          for (int c = 0; c < runs; c++) {
+            const int slot = ((rank - want_lo) * p.slices + s) * runs + c;
+            list_at[slot] = ((s * ntiles + id) << eshift) + c * run;
+            list_rel[slot] = rel + c * run;
+            list_lim[slot] = (rows - 1) | (cols - 1) << 14 | c << 28;
+          }
       }
       rank++;
     }
     seen += found;
     __syncthreads();
-    // --- add the listed tiles into the window -------------------------------------------------
-    // Rounds of 16 loads per thread (16 / LPE entries); the next round's loads are in flight
-    // while this round's values are added, in list order.  Lane u of every wavefront fetches
-    // entry u of the round from the list; the entries are then uniform values (scalar registers).
-    constexpr int kRound = 16 / LPE;
+    // --- add the listed runs into the window ---------------------------------------------------
+    // Every wavefront on its own: lane u holds entry u of a chunk of 64 list entries; the entries
+    // that meet one of the wavefront's blocks are taken in list order, in rounds of kFoldRound;
+    // the next round's loads are in flight while this round's values are added.  What describes
+    // an entry to the wavefront is uniform (scalar registers).
     struct Round {
-      float v[16];
-      int q[16];      // window position of v[f], -1: none
-      bool clash;     // (uniform) two tiles of the round overlap: their adds must stay in order
+      fold_f4 v[kFoldRound];
+      int pos[kFoldRound];   // window position of the block
+      int e0[kFoldRound];    // float of the run that falls on the block's first position (-255 .. run - 1)
+      int lim[kFoldRound];   // the entry's, -1: no entry
     };
-    auto issue = [&](int t, Round& r) {
-      const bool have = lane < kRound && t + lane < total;
-      const int my_rel = have ? list_rel[t + lane] : -(1 << 29);   // (far away: no element lands in the window)
-      const int my_at = have ? list_at[t + lane] : 0;
-      const int my_lim = have ? list_lim[t + lane] : 0;
-      bool meets = false;
-#pragma unroll
-      for (int d = 1; d < kRound; d++) {
-        const int other = __shfl_down(my_rel, d, 64);
-        const int gap = my_rel - other;
-        meets |= have && lane + d < kRound && gap < E && gap > -E;
+    unsigned long long todo = 0ull;   // entries of the chunk that this wavefront still has to add
+    int next = 0;                     // first list entry behind the chunk
+    int c_pos = 0, c_e0 = 0, c_off = 0, c_lim = 0;
+    auto refill = [&]() {
+      while (todo == 0ull && next < total) {   // (uniform)
+        const int t = next + lane;
+        const bool have = t < total;
+        const int rel = have ? list_rel[t] : 0, at = have ? list_at[t] : 0;
+        c_lim = have ? list_lim[t] : 0;
+        const int first = rel >> 8;                    // (arithmetic shift: the block of the run's first float)
+        const int b = first + ((wave - first) & 15);   // the wavefront's only block among the sixteen from there on
+        c_pos = b * kFoldBlock;
+        c_e0 = c_pos - rel;
+        c_off = at + c_e0;
+        todo = __ballot(have && b >= 0 && c_pos < wlen && c_e0 < run);
+        next += 64;
       }
-      r.clash = __ballot(meets) != 0ull;
+    };
+    auto issue = [&](Round& r) {
 #pragma unroll
-      for (int f = 0; f < 16; f++) {
-        const int rel = __builtin_amdgcn_readlane(my_rel, f / LPE), at = __builtin_amdgcn_readlane(my_at, f / LPE);
-        const int lim = __builtin_amdgcn_readlane(my_lim, f / LPE);
-        const int e = ((tid - rel) & (kFoldThreads - 1)) + (f % LPE) * kFoldThreads;   // my (f % LPE)-th element of the tile
-        const int pos = rel + e;                                                       // (pos % 1024 == tid)
-        // (in the window, and inside K x N: the contraction wrote nothing beyond its own C tiles)
-        const bool ok = e < E && pos >= 0 && pos < wlen && (e >> p.h.bn_shift) < (lim & 0xffff) &&
-                        (e & (p.h.BN - 1)) < (lim >> 16);
-        // (every thread loads, those without an element the tile's first float: with no branch
-        //  around the loads their number is fixed, and the wait for this round's values can leave
-        //  the next round's in flight)
-        const float x = p.tiles[(uint32_t)(ok ? at + e : at)];
-        r.v[f] = ok ? x : 0.f;
-        r.q[f] = ok ? pos : -1;
+      for (int u = 0; u < kFoldRound; u++) {
+        const bool any = todo != 0ull;
+        const int src = any ? (int)__builtin_ctzll(todo) : 0;
+        todo &= todo - 1ull;
+        const int off = __builtin_amdgcn_readlane(c_off, src), lim = __builtin_amdgcn_readlane(c_lim, src);
+        r.pos[u] = __builtin_amdgcn_readlane(c_pos, src);
+        r.e0[u] = __builtin_amdgcn_readlane(c_e0, src);
+        r.lim[u] = any ? lim : -1;
+        // (every slot loads, an empty one the buffer's first floats: with no branch around the
+        //  loads their number is fixed, and the wait for this round's values can leave the next
+        //  round's in flight)
+        const long long first = any ? (long long)off : 0ll;
+        r.v[u] = *reinterpret_cast<const fold_f4u*>(reinterpret_cast<const char*>(p.tiles) + first * 4 + lane16);
       }
     };
     // (plain read-add-write: LDS float atomics are several times slower, and nobody else touches
-    //  this thread's words)
+    //  this lane's words; runs that overlap are added one after the other, in list order)
     auto add = [&](const Round& r) {
-      if (!r.clash) {   // all positions of the round differ: read them together
-        float cur[16];
 #pragma unroll
-        for (int f = 0; f < 16; f++) cur[f] = img[r.q[f] >= 0 ? r.q[f] : tid];
+      for (int u = 0; u < kFoldRound; u++) {
+        if (r.lim[u] == -1) continue;   // (uniform)
+        fold_f4 v = r.v[u];
+        const int lim = r.lim[u];
+        if (r.e0[u] < 0 || r.e0[u] + kFoldBlock > run || (lim & 0x0fffffff) != full_lim) {
+          // an end of the run, or a tile that sticks out of K x N: what is not the run's counts as zero
+          asm volatile("" ::: "memory");   // (keeps this arithmetic out of the common path)
+          const int rows = (lim & 0x3fff) + 1, cols = ((lim >> 14) & 0x3fff) + 1, base = (lim >> 28) * run;
 #pragma unroll
-        for (int f = 0; f < 16; f++)
-          if (r.q[f] >= 0) img[r.q[f]] = cur[f] + r.v[f];
-      } else {
-#pragma unroll
-        for (int f = 0; f < 16; f++)
-          if (r.q[f] >= 0) img[r.q[f]] += r.v[f];
+          for (int f = 0; f < 4; f++) {
+            const int e = r.e0[u] + lane4 + f, in_tile = base + e;
+            const bool ok = e >= 0 && e < run && (in_tile >> p.h.bn_shift) < rows && (in_tile & (p.h.BN - 1)) < cols;
+            v[f] = ok ? v[f] : 0.f;
+          }
+        }
+        fold_f4* at = reinterpret_cast<fold_f4*>(img + r.pos[u] + lane4);
+        *at = *at + v;
       }
     };
     Round r0, r1;
-    issue(0, r0);
-    for (int t = 0; t < total; t += 2 * kRound) {
-      issue(t + kRound, r1);
+    refill();
+    issue(r0);
+    while (true) {   // (uniform per wavefront; no barrier inside)
+      refill();
+      issue(r1);
       add(r0);
-      issue(t + 2 * kRound, r0);
+      if (r1.lim[0] == -1) break;   // (entries fill a round from its first slot)
+      refill();
+      issue(r0);
       add(r1);
+      if (r0.lim[0] == -1) break;
     }
     lo += span;
   }
   // --- the window of this share's image ---------------------------------------------------------
+  __syncthreads();   // (the words below were added up by other threads)
   if (p.partial != nullptr) {
     float* out = p.partial + (size_t)share * (size_t)p.pitch + w0;
     for (int q = tid; q < wlen; q += kFoldThreads) out[q] = img[q];

@@ -122,12 +122,14 @@ static inline int pick_tile(int I, int J, int elem_bytes, const rz_tuning& tunin
 
 // Weight-grad without any scatter in the contraction kernel: X^T.dY is stored tile by tile and a
 // second kernel, whose workgroups own windows of hashed_weight, folds the tiles into dHW.
+// (the fold kernel reads a kilobyte per wavefront from any 4-byte boundary: up to 1032 bytes before and after the tiles)
+static constexpr size_t kFoldMarginBytes = 2048;
+
 struct FoldPlan {
   int use;
   int window, windows;   // floats per window (a multiple of 1024, at most 32768) and their number
   int shares;            // workgroups per window, each with an equal part of the window's tiles and an image of its own
-  int loads;             // per list entry and thread: BK*BN / 1024, at least 1
-  size_t tiles_bytes;    // the tile-by-tile X^T.dY: slices * tiles * BK*BN floats
+  size_t tiles_bytes;    // the tile-by-tile X^T.dY: slices * tiles * BK*BN floats, with a margin before and after
   size_t partial_bytes;  // shares images of dHW (none with a single share: the fold kernel writes dHW)
   size_t offsets_bytes;  // where every tile starts in hashed_weight, one int32 per tile
 };
@@ -150,8 +152,7 @@ static inline FoldPlan plan_fold(int K, int N, int H, int BK, int BN, int slices
   if (shares > slices * tiles / 8) shares = slices * tiles / 8;   // a share is worth a workgroup from some tiles on
   if (shares < 1) shares = 1;
   f.shares = (int)shares;
-  f.loads = E >= 1024 ? (int)(E / 1024) : 1;
-  f.tiles_bytes = ((size_t)slices * tiles * E * sizeof(float) + 255) & ~(size_t)255;
+  f.tiles_bytes = (((size_t)slices * tiles * E * sizeof(float) + 255) & ~(size_t)255) + 2 * kFoldMarginBytes;
   const size_t pitch = (size_t)((H + 3) & ~3);
   f.partial_bytes = f.shares > 1 ? ((size_t)f.shares * pitch * sizeof(float) + 255) & ~(size_t)255 : 0;
   f.offsets_bytes = ((size_t)tiles * sizeof(int32_t) + 255) & ~(size_t)255;
