@@ -18,8 +18,10 @@
 // need no barrier between runs and each goes down the list at its own pace.  Only the blocks
 // at the two ends of a run, and runs of tiles that stick out of K x N (whose buffer holds floats
 // that the contraction never wrote), need their elements masked one by one: a branch of its
-// own.  The loads reach up to 258 floats before and after a run: the buffer is allocated with a
-// margin on both sides.
+// own; there, lanes wholly outside the run re-fetch floats of the run, so that a block costs no
+// memory traffic beyond the run's own cache lines.  The loads reach up to three floats before
+// and after a run (an empty slot of a round reads the buffer's first kilobyte): the buffer is
+// allocated with a margin on both sides.
 //
 // A window is at most 32768 floats (128 KB of LDS).  When hashed_weight has fewer windows than
 // the chip has compute units, `shares` workgroups share a window: each takes an equal part of the
@@ -219,7 +221,15 @@ __global__ __launch_bounds__(kFoldThreads) void fold_tiles_kernel(const FoldPara
         //  loads their number is fixed, and the wait for this round's values can leave the next
         //  round's in flight)
         const long long first = any ? (long long)off : 0ll;
-        r.v[u] = *reinterpret_cast<const fold_f4u*>(reinterpret_cast<const char*>(p.tiles) + first * 4 + lane16);
+        unsigned mine = lane16;   // byte offset of the lane's four floats from the block's first
+        if (any && (r.e0[u] < 0 || r.e0[u] + kFoldBlock > run)) {   // (uniform) an end of the run:
+          // lanes that lie wholly outside the run fetch floats of the run that other lanes fetch
+          // anyway (their values count as zero below) instead of a neighbouring tile's
+          const int e = r.e0[u] + lane4;
+          const int inside = e <= -4 ? 0 : (e >= run ? max(run - 4, r.e0[u]) : e);
+          mine = (unsigned)(inside - r.e0[u]) * 4u;
+        }
+        r.v[u] = *reinterpret_cast<const fold_f4u*>(reinterpret_cast<const char*>(p.tiles) + first * 4 + mine);
       }
     };
     // (plain read-add-write: LDS float atomics are several times slower, and nobody else touches
