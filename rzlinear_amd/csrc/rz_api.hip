@@ -246,6 +246,9 @@ static hipError_t reduce_slices_dtype(int dtype, const float* part, void* C, con
 // workspace the contraction may be split over R (skinny problems).
 static int run_plain_op(int op, int dtype, GemmParams p, const void* bias, void* workspace,
                         size_t workspace_bytes, bool may_split, const rz_tuning& tuning, hipStream_t s) {
+  // an output of more than twice an L2 goes out with streaming stores (a smaller one may still be
+  // in cache when the next kernel reads it)
+  p.stream_c = (size_t)p.I * (size_t)p.J * dtype_bytes(dtype) >= ((size_t)8 << 20) ? 1 : 0;
   if (may_split) {
     // tile and slices are chosen together
     const SplitPlan sp = plan_split(p.I, p.J, p.R, dtype_bytes(dtype), tuning);

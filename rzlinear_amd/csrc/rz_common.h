@@ -98,6 +98,7 @@ struct GemmParams {
   const void* B;      // plain B operand (weight-grad) — else unused
   const void* HW;     // hashed weight (forward, input-grad)
   void* C;            // plain output (forward, input-grad)
+  int stream_c;       // ... stored with streaming (non-temporal) stores: for outputs far larger than the L2
   const void* bias;   // optional [J] vector added to every row of C (forward), or null
   float* partial;     // forward/input-grad with R split over blockIdx.y: fp32 partial results
                       // [slices][I][J] (scaled, no bias) instead of C; null = no split
