@@ -53,7 +53,7 @@ struct FoldParams {
 
 static constexpr int kFoldThreads = 1024;
 static constexpr int kFoldList = 2048;       // entries of the run list in LDS
-static constexpr int kFoldScan = 32;         // tile indices per thread and listing pass
+static constexpr int kFoldScan = 64;         // tile indices per thread and listing pass (one bit each of a 64-bit mask)
 static constexpr int kFoldWindowMax = 32768;
 static constexpr int kFoldRun = 2048;        // floats of a run at most (tiles are powers of two: whole runs)
 static constexpr int kFoldRound = 8;         // runs whose loads a wavefront issues together
@@ -87,20 +87,25 @@ __global__ __launch_bounds__(kFoldThreads) void fold_tiles_kernel(const FoldPara
   for (int q = tid; q < p.window; q += kFoldThreads) img[q] = 0.f;   // (own positions only)
 
   // bit j: tile first + i + 1024 j (below `stop`) lands in the window.  The offsets are fetched
-  // together, by loads that depend on no condition (one load under a branch per index would
-  // cost a round trip to the L2 each).
-  auto scan = [&](int first, int stop) -> unsigned {
-    int rel[kFoldScan];
+  // sixteen at a time, by loads that depend on no condition (one load under a branch per index
+  // would cost a round trip to the L2 each); batches wholly beyond `stop` are skipped.
+  auto scan = [&](int first, int stop) -> unsigned long long {
+    unsigned long long mask = 0ull;
+    constexpr int kBatch = 16;
 #pragma unroll
-    for (int j = 0; j < kFoldScan; j++) {
-      const int id = first + tid + j * kFoldThreads;
-      rel[j] = p.offsets[id < stop ? id : stop - 1];
-    }
-    unsigned mask = 0u;
+    for (int c = 0; c < kFoldScan / kBatch; c++) {
+      if (first + c * kBatch * kFoldThreads >= stop) break;   // (uniform)
+      int rel[kBatch];
 #pragma unroll
-    for (int j = 0; j < kFoldScan; j++) {
-      const int id = first + tid + j * kFoldThreads, r = rel[j] - w0;
-      mask |= (unsigned)((id < stop) & (r > -E) & (r < wlen)) << j;
+      for (int j = 0; j < kBatch; j++) {
+        const int id = first + tid + (c * kBatch + j) * kFoldThreads;
+        rel[j] = p.offsets[id < stop ? id : stop - 1];
+      }
+#pragma unroll
+      for (int j = 0; j < kBatch; j++) {
+        const int id = first + tid + (c * kBatch + j) * kFoldThreads, r = rel[j] - w0;
+        mask |= (unsigned long long)((id < stop) & (r > -E) & (r < wlen)) << (c * kBatch + j);
+      }
     }
     return mask;
   };
@@ -134,7 +139,7 @@ __global__ __launch_bounds__(kFoldThreads) void fold_tiles_kernel(const FoldPara
   int rank_lo = 0, rank_hi = 0x7fffffff;
   if (p.shares > 1) {
     int mine = 0, before;
-    for (int first = 0; first < ntiles; first += kFoldScan * kFoldThreads) mine += __popc(scan(first, ntiles));
+    for (int first = 0; first < ntiles; first += kFoldScan * kFoldThreads) mine += __popcll(scan(first, ntiles));
     const int all = total_of(wave_scan(mine), &before);
     rank_lo = (int)((long long)share * all / p.shares);
     rank_hi = (int)((long long)(share + 1) * all / p.shares);
@@ -144,8 +149,8 @@ __global__ __launch_bounds__(kFoldThreads) void fold_tiles_kernel(const FoldPara
   while (lo < ntiles && seen < rank_hi) {   // (uniform: every thread of the workgroup goes round together)
     if (span > ntiles - lo) span = ntiles - lo;
     // --- list the share's tiles among [lo, lo + span) ---------------------------------------------
-    unsigned mask = scan(lo, lo + span);
-    const int mine = __popc(mask);
+    unsigned long long mask = scan(lo, lo + span);
+    const int mine = __popcll(mask);
     const int incl = wave_scan(mine);
     int before;
     const int found = total_of(incl, &before);
@@ -157,9 +162,9 @@ __global__ __launch_bounds__(kFoldThreads) void fold_tiles_kernel(const FoldPara
       continue;
     }
     int rank = seen + before + incl - mine;   // of this thread's first tile
-    while (mask != 0u) {
-      const int j = __ffs(mask) - 1;
-      mask &= mask - 1u;
+    while (mask != 0ull) {
+      const int j = __ffsll((long long)mask) - 1;
+      mask &= mask - 1ull;
       if (rank >= want_lo && rank < want_hi) {
         const int id = lo + tid + j * kFoldThreads;
         const int rel = p.offsets[id] - w0;
