@@ -112,7 +112,7 @@ static hipError_t launch_op(int op, GemmParams p, const WeightGradPlan* plan, co
 //        instead of a pipeline (tuning aid)
 //    64:  64 x  64, four wavefronts of 32 x 32, for problems with few tiles; fp32 forward /
 //        input-grad: eight, in two groups that share every R step between them
-//    32:  32 x  64 (fp32 forward / input-grad of at most 32 rows): four wavefronts of 32 x 32 in two such groups
+//    32:  32 x  64 (fp32 forward / input-grad whose rows would leave a 64-row tile at most half full): four wavefronts of 32 x 32 in two such groups
 template <typename T>
 static hipError_t launch_gemm_t(int op, GemmParams p, const WeightGradPlan* plan, const SplitPlan* split,
                                 const rz_tuning& tuning, hipStream_t stream) {
@@ -128,7 +128,7 @@ static hipError_t launch_gemm_t(int op, GemmParams p, const WeightGradPlan* plan
     case 6482:   // fp32 forward / input-grad: two groups of four wavefronts share every R step
       if constexpr (sizeof(T) == 4) return launch_op<T, 64, 2, 2, 2, 2>(op, p, plan, split, form, stream);
       return hipErrorInvalidValue;
-    case 3242:   // fp32 forward / input-grad of at most 32 rows: 32 x 64, two groups of two wavefronts
+    case 3242:   // fp32 forward / input-grad, rows in 32s: 32 x 64, two groups of two wavefronts
       if constexpr (sizeof(T) == 4) {
         if (op == kForward) return launch_tile<T, kForward, 32, 1, 2, 2, false, 2, 64>(p, plan, split, form, stream);
         if (op == kInputGrad) return launch_tile<T, kInputGrad, 32, 1, 2, 2, false, 2, 64>(p, plan, split, form, stream);

@@ -47,7 +47,8 @@ static inline int slice_unit(int tile, int elem_bytes) {
 }
 
 // Tile codes: 64, 128, 256 are square C tiles; 32 stands for the 32 x 64 tile of the fp32 forward /
-// input-grad kernels for batches of at most 32 rows (half of a 64-row tile would be padding).
+// input-grad kernels, for batches whose rows would leave the last 64-row tile at most half full
+// (M = 32, 96, 160: that half would be padding).
 static inline int tile_cols(int t) { return t == 32 ? 64 : t; }
 static inline long long tile_count(int I, int J, int t) {
   return (long long)((I + t - 1) / t) * ((J + tile_cols(t) - 1) / tile_cols(t));
@@ -437,7 +438,9 @@ static inline SplitPlan plan_split(int I, int J, int R, int elem_bytes, const rz
   const int forced = (t.tile == 32 && elem_bytes != 4) ? 64 : t.tile;
   for (int tile : tiles_of) {
     if (forced && tile != forced) continue;
-    if (tile == 32 && !forced && (elem_bytes != 4 || I > 32)) continue;
+    // (the 32 x 64 tile: fp32 only, and only where 64-row tiles would end in a tile at most half full —
+    //  K = N = 10240: M = 96 259 -> 232 us, M = 160 428 -> 353 us, M = 288 668 -> 620 us)
+    if (tile == 32 && !forced && (elem_bytes != 4 || (I > 32 && (I - 1) % 64 >= 32))) continue;
     const int TR = slice_unit(tile, elem_bytes);
     const long long tiles = tile_count(I, J, tile);
     const int r_steps = (R + TR - 1) / TR;

@@ -154,10 +154,12 @@ def test_every_tile_shape_and_scatter_mode(oracle, shape, env, dtype):
 @pytest.mark.parametrize("split", [0, -1], ids=["cut", "whole"])
 @pytest.mark.parametrize("shape", [(32, 1536, 2048, 200000, 64, 64), (17, 100, 150, 5000, 32, 64),
                                    (8, 4096, 320, 70000, 64, 64), (32, 10240, 1024, 1 << 20, 64, 64),
-                                   (1, 64, 64, 8192, 64, 64)], ids=lambda s: "x".join(map(str, s)))
+                                   (1, 64, 64, 8192, 64, 64), (96, 2048, 4096, 300000, 32, 64),
+                                   (150, 1000, 2100, 70000, 64, 64)], ids=lambda s: "x".join(map(str, s)))
 def test_fp32_batches_of_at_most_32_rows_take_the_32_row_tile(oracle, shape, split):
-    """The 32 x 64 tile of fp32 forward / input-grad (for M <= 32 a 64-row tile is half padding;
-    large problems choose it by themselves), with and without a cut contraction, with a bias."""
+    """The 32 x 64 tile of fp32 forward / input-grad (where a 64-row tile would be half padding:
+    M <= 32, 65..96, 129..160, ...; large problems choose it by themselves), with and without a
+    cut contraction, with a bias; also several tile rows, the last one ragged."""
     from rzlinear_amd import _lib
     from rzlinear_amd.impl.RzLinearBackward import rz_linear_backward_input_grad_tl
     from rzlinear_amd.impl.RzLinearForward import rz_linear_forward_bias_tl
@@ -174,6 +176,28 @@ def test_fp32_batches_of_at_most_32_rows_take_the_32_row_tile(oracle, shape, spl
     ref = oracle.forward(x64, hw64, N, BK, BN, R1024, 0.5) + bias.double().numpy()[None, :]
     assert rel_err(y.cpu().numpy(), ref) <= TOL[torch.float32]
     assert rel_err(dx.cpu().numpy(), oracle.input_grad(dy64, hw64, K, BK, BN, R1024, 0.5)) <= TOL[torch.float32]
+
+
+@pytest.mark.parametrize("M", [32, 96, 160, 288])
+def test_the_32_row_tile_is_chosen_where_64_rows_would_be_half_padding(oracle, M):
+    """K = N = 4096, fp32: the plan takes the 32 x 64 tile by itself for these batch sizes (and not for
+    M = 128 or 192), and the result matches the oracle."""
+    from rzlinear_amd import _lib
+    from rzlinear_amd.impl.RzLinearBackward import rz_linear_backward_input_grad_tl
+    from rzlinear_amd.impl.RzLinearForward import rz_linear_forward_tl
+    K = N = 4096
+    H, BK, BN = 1 << 20, 32, 64
+    _say("32-row tile by plan", M)
+    for op in (0, 1):
+        assert _lib.plan_query(op, M, K, N, H, BK, BN, _lib.RZ_F32)["tile"] == 32
+        assert _lib.plan_query(op, 128, K, N, H, BK, BN, _lib.RZ_F32)["tile"] != 32
+        assert _lib.plan_query(op, 192, K, N, H, BK, BN, _lib.RZ_F32)["tile"] != 32
+    (x, hw, dy), (x64, hw64, dy64) = make_inputs(M, K, N, H, torch.float32, seed=14)
+    y = rz_linear_forward_tl(x, hw, 1.0, M, K, N, H, *rargs(R1024), BLOCK_SIZE_K=BK, BLOCK_SIZE_N=BN)
+    dx = rz_linear_backward_input_grad_tl(dy, hw, 1.0, M, K, N, H, *rargs(R1024), BLOCK_SIZE_K=BK, BLOCK_SIZE_N=BN)
+    torch.cuda.synchronize()
+    assert_close(y.cpu().numpy(), oracle.forward(x64, hw64, N, BK, BN, R1024, 1.0), torch.float32, "Y")
+    assert_close(dx.cpu().numpy(), oracle.input_grad(dy64, hw64, K, BK, BN, R1024, 1.0), torch.float32, "dX")
 
 
 def test_kernels_match_vectors_produced_by_the_reference_kernels():
