@@ -61,10 +61,12 @@ static inline long long tile_count(int I, int J, int t) {
 // wgs * w: the rate is (wgs / CUs) * e(c) / c.  (320 workgroups on 256 compute units leave 64 of
 // them with two: the launch takes as long as 512 would.)  Beyond `slots` per compute unit the
 // workgroups go in rounds of CUs * slots and a last, partly filled round costs a full one.
-static inline double occupancy_rate(double wgs, int slots, double lo, double hi) {
+static inline double occupancy_rate(double wgs, int slots, double lo, double hi, int knee = 0) {
   const double per_cu = wgs / kComputeUnits;
   if (per_cu <= 1.0) return lo * per_cu;
-  auto e = [&](double c) { return slots > 1 ? lo + (hi - lo) * (c - 1.0) / (slots - 1.0) : hi; };
+  // (`knee`: the number of resident workgroups from which the compute unit runs at `hi`, if fewer than `slots`)
+  const double full = knee > 1 ? knee : slots;
+  auto e = [&](double c) { return full > 1 ? lo + (hi - lo) * (c < full ? (c - 1.0) / (full - 1.0) : 1.0) : hi; };
   if (per_cu <= slots) {
     const double c = (double)((long long)(per_cu + 0.999999));
     return per_cu * e(c) / c;
@@ -100,9 +102,11 @@ static inline double tile_rate(double wgs, int t, int elem_bytes) {
   // (32 x 64, four wavefronts: half a 64 workgroup's work in about its time, up to eight resident)
   if (t == 32) return occupancy_rate(wgs, 8, 0.40, 0.80);
   const int slots = (t == 256) ? 1 : (t == 128 ? 2 : 4);
-  const double lo = (t == 256) ? 1.0 : (t == 128 ? (f32 ? 0.86 : 0.51) : (f32 ? 0.60 : 0.16));
+  // (the 16-bit 64 tile: 0.24 with one workgroup per compute unit, 0.33 from two on — K = 2048, N = 8192:
+  //  M = 128 14.9 us, M = 256 22.7 us; priced at 0.16 it lost to cut 128 tiles that take 21 and 30 us)
+  const double lo = (t == 256) ? 1.0 : (t == 128 ? (f32 ? 0.86 : 0.51) : (f32 ? 0.60 : 0.24));
   const double hi = (t == 256) ? 1.0 : (t == 128 ? (f32 ? 0.90 : 0.75) : (f32 ? 0.80 : 0.33));
-  return occupancy_rate(wgs, slots, lo, hi);
+  return occupancy_rate(wgs, slots, lo, hi, (t == 64 && !f32) ? 2 : 0);
 }
 
 // C-tile edge for a contraction with an I x J result: the best-scoring of 256, 128, 64.
@@ -290,13 +294,16 @@ static inline WeightGradPlan plan_weight_grad(int M, int K, int N, int H, int BK
     const FoldPlan f = plan_fold(K, N, H, BK, BN, pl.splits);
     if (f.use) {
       // what the two ways cost beyond the contraction itself, in microseconds: the part of the
-      // K*N global atomics per slice that the contraction does not hide (about 2.8 ps each,
+      // K*N global atomics per slice that the contraction does not hide (2.8 to 5.2 ps each,
       // measured), against reading the tiles back (their stores overlap the contraction, unless
       // it is shorter than they are), writing and reading the images, and two more launches
       const double elems = (double)pl.splits * (double)K * (double)N;
       const double product_us = 2.0 * (double)M * K * N / (elem_bytes == 4 ? 110e6 : 900e6);
       const double store_us = elems * 4.0 / 4.0e6;
-      const double atomics_us = elems * 2.8e-6;
+      // (K*N atomics take about 5.2 ps each; a long contraction hides up to 2.4 ps of that — K = 2048,
+      //  N = 8192, bf16: M = 128 87 us in all against 57 us folded, M = 1024 108 against 79 us)
+      const double hidden = 0.45 * product_us < elems * 2.4e-6 ? 0.45 * product_us : elems * 2.4e-6;
+      const double atomics_us = elems * 5.2e-6 - hidden;
       // (a workgroup of the fold kernel reads some 15 GB/s: few workgroups cannot use the memory system)
       const double read_bytes = elems * 4.0 * (1.0 + (double)BK * BN / f.window);
       const double all_us = (read_bytes + 2.0 * (double)f.partial_bytes) / 4.5e6;

@@ -429,13 +429,14 @@ def test_cut_contraction_on_the_long_step_tile(oracle, shape, dtype):
     M, K, N, H, BK, BN = shape
     _say("cut contraction, long step", shape, dtype)
     code = _lib.dtype_code(torch.empty(0, dtype=dtype))
-    plans = [_lib.plan_query(op, M, K, N, H, BK, BN, code) for op in (0, 1)]
-    assert any(p["tile"] == 128 and p["slices"] > 1 for p in plans), plans
-    for p in plans:
-        assert p["slices"] == 1 or p["slice_len"] % p["step"] == 0, p
     (x, hw, dy), (x64, hw64, dy64) = make_inputs(M, K, N, H, dtype, seed=21)
-    y = rz_linear_forward_tl(x, hw, 1.0, M, K, N, H, *rargs(R1024), BLOCK_SIZE_K=BK, BLOCK_SIZE_N=BN)
-    dx = rz_linear_backward_input_grad_tl(dy, hw, 1.0, M, K, N, H, *rargs(R1024), BLOCK_SIZE_K=BK, BLOCK_SIZE_N=BN)
+    with _lib.tuning(tile=128):   # (the tile in question, whatever the plan would pick by itself; the cut stays the plan's)
+        plans = [_lib.plan_query(op, M, K, N, H, BK, BN, code) for op in (0, 1)]
+        assert any(p["tile"] == 128 and p["slices"] > 1 for p in plans), plans
+        for p in plans:
+            assert p["slices"] == 1 or p["slice_len"] % p["step"] == 0, p
+        y = rz_linear_forward_tl(x, hw, 1.0, M, K, N, H, *rargs(R1024), BLOCK_SIZE_K=BK, BLOCK_SIZE_N=BN)
+        dx = rz_linear_backward_input_grad_tl(dy, hw, 1.0, M, K, N, H, *rargs(R1024), BLOCK_SIZE_K=BK, BLOCK_SIZE_N=BN)
     torch.cuda.synchronize()
     assert_close(y.float().cpu().numpy(), oracle.forward(x64, hw64, N, BK, BN, R1024), dtype, "Y")
     assert_close(dx.float().cpu().numpy(), oracle.input_grad(dy64, hw64, K, BK, BN, R1024), dtype, "dX")

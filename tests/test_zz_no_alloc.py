@@ -23,7 +23,9 @@ def _say(*a):
 
 
 def _both(lib, shape, dtype, seed, oracle):
-    """dHW of one problem through both entry points; returns (static, workspace, oracle)."""
+    """dHW of one problem through both entry points; returns (static, workspace, oracle, whether
+    the workspace the plan asks for fits the static scratch: if not, the static entry point takes
+    the atomic scatter instead)."""
     from rzlinear_amd import _lib
     M, K, N, H, BK, BN = shape
     (x, _, dy), (x64, _, dy64) = make_inputs(M, K, N, H, dtype, seed=seed)
@@ -31,7 +33,6 @@ def _both(lib, shape, dtype, seed, oracle):
     R = (ctypes.c_int32 * 8)(*R1024)
     stream = torch.cuda.current_stream().cuda_stream
     need = lib.rz_weight_grad_workspace_bytes(M, K, N, H, BK, BN, code)
-    assert need <= SCRATCH_BYTES
     ws = torch.empty((max(need, 16),), dtype=torch.uint8, device="cuda")
     # poison the outputs: both entry points overwrite dHW completely
     a = torch.full((H,), float("nan"), dtype=dtype, device="cuda")
@@ -41,7 +42,7 @@ def _both(lib, shape, dtype, seed, oracle):
     _lib.check(lib.rz_weight_grad(x.data_ptr(), dy.data_ptr(), b.data_ptr(), ws.data_ptr(), need, M, K, N, H,
                                   BK, BN, R, 0.5, K, N, code, stream))
     torch.cuda.synchronize()
-    return a, b, oracle.weight_grad(x64, dy64, H, BK, BN, R1024, 0.5)
+    return a, b, oracle.weight_grad(x64, dy64, H, BK, BN, R1024, 0.5), need <= SCRATCH_BYTES
 
 
 # (first problem, smaller second problem, how the plan carries the first one out in bf16)
@@ -64,9 +65,10 @@ def test_static_scratch_matches_the_workspace_entry_point(oracle, pair, dtype):
         _say("static scratch", mode, "call", i, shape, dtype, plan)
         if dtype == torch.bfloat16 and i == 0:
             assert plan["mode"] == mode, plan      # the scratch layouts are all exercised
-        a, b, ref = _both(lib, shape, dtype, seed=50 + i, oracle=oracle)
+        a, b, ref, fits = _both(lib, shape, dtype, seed=50 + i, oracle=oracle)
+        assert fits or dtype != torch.bfloat16   # (the bf16 pairs exercise the scratch layouts named above)
         f = lambda t: t.float().cpu().numpy()
-        if plan["mode"] == "atomics":
+        if plan["mode"] == "atomics" or not fits:
             # global atomics: the summation order is not fixed, compare within the tolerance
             assert rel_err(f(a), f(b).astype(np.float64)) <= TOL[dtype]
         else:
