@@ -249,8 +249,8 @@ static inline WeightGradPlan plan_weight_grad(int M, int K, int N, int H, int BK
     pl.tile = pick_tile(K, N, elem_bytes, t);
     // fp32 with the tiles stored for the fold kernel: a 256 workgroup is alone on its compute unit
     // and its 256 KB of stores are exposed after a short loop over M; two 128 workgroups hide each
-    // other's (K = N = 10240: M = 128 455 -> 401 us, M = 1024 1938 -> 1797 us)
-    if (pl.tile == 256 && elem_bytes == 4 && M <= 2048 && t.fold != -1 && plan_fold(K, N, H, BK, BN, 1).use) pl.tile = 128;
+    // other's (K = N = 10240: M = 128 455 -> 401 us, M = 1024 1938 -> 1797 us, M = 4096 7002 -> 6449 us)
+    if (pl.tile == 256 && elem_bytes == 4 && M <= 8192 && t.fold != -1 && plan_fold(K, N, H, BK, BN, 1).use) pl.tile = 128;
   }
   const long long tiles = (long long)((K + pl.tile - 1) / pl.tile) * ((N + pl.tile - 1) / pl.tile);
   const int TR = slice_unit(pl.tile, elem_bytes);
