@@ -376,7 +376,13 @@ static inline WindowPlan plan_window(int M, int K, int N, int H, int BK, int BN,
   // (in units of 64-row tiles, i.e. of two strips: the figures below were fitted on those)
   const double per_wg = (double)tiles * ((double)w + (double)BK * BN) / (double)H * ((double)BK / 64.0);
   const double wg_rounds = (double)((pl.windows + kComputeUnits - 1) / kComputeUnits);
-  const double t_window = wg_rounds * per_wg * ((elem_bytes == 4 ? 0.43 + 0.63 * chunks : 0.31 + 0.18 * chunks)) + (planned ? 5.0 : 28.0);
+  double t_window = wg_rounds * per_wg * ((elem_bytes == 4 ? 0.43 + 0.63 * chunks : 0.31 + 0.18 * chunks)) + (planned ? 5.0 : 28.0);
+  // Every element of dHW receives K*N / H tiles, and the adds into one place of a window go in a
+  // fixed order, one after the other: with many tiles per element that chain is what takes the
+  // time, about 1.7 us a link (K = 2048, N = 8192, H = 200000: 84 links, 158 us at M = 32 — folded
+  // 57 us; K = N = 10240, H = 200000: 524 links, 1048 us).
+  const double chain_us = 1.7 * (double)K * (double)N / (double)H + 10.0;
+  if (t_window < chain_us) t_window = chain_us;
   // ... against what the contraction kernel's plan would take: the fold, or the atomic scatter
   const double t_scatter = 0.9 * (double)K * N / 184e3 + 2.0 * M * (double)K * N / 800e6;
   const double t_other = other.fold.use ? other.fold_us : t_scatter;
