@@ -204,6 +204,22 @@ static inline long long image_slices(long long tiles, long long r_steps) {
   return want < 1 ? 1 : want;
 }
 
+// How well C tiles fill their rounds of workgroups, relative to an ideal distribution.  256 tiles
+// go one to a compute unit in rounds of that many.  128 tiles go two to a compute unit; the
+// busiest compute unit gets c = ceil(tiles / CUs) of them and works through them in pairs, a
+// last odd one alone in about half the time of a pair.
+static inline double filled_256(long long tiles) {
+  return (double)tiles / (double)((tiles + kComputeUnits - 1) / kComputeUnits * kComputeUnits);
+}
+static inline double filled_128(long long tiles) {
+  const long long c = (tiles + kComputeUnits - 1) / kComputeUnits;
+  return ((double)tiles / (2.0 * kComputeUnits)) / ((double)(c / 2) + (c % 2 ? 0.52 : 0.0));
+}
+// fp32: the 128 tile in pairs runs at this fraction of the 256 tile's rate (weight-grad, measured:
+// 4096^2 1067 against 1012 us in one round each; K = N = 5120, M = 4096: 1831 against 2000 us,
+// 1600 tiles in seven half-rounds against 400 in two rounds)
+static constexpr double kPairRate128F32 = 0.955;
+
 static inline WeightGradPlan plan_weight_grad(int M, int K, int N, int H, int BK, int BN, int elem_bytes,
                                               const rz_tuning& t) {
   WeightGradPlan pl;
@@ -225,6 +241,19 @@ static inline WeightGradPlan plan_weight_grad(int M, int K, int N, int H, int BK
     if (pl.tile == 256 && elem_bytes == 4 && tiles256 < kComputeUnits &&
         (long long)((M + step256 - 1) / step256) * tiles256 < 4LL * kComputeUnits && cover128)
       pl.tile = 128;
+    // (two 128 workgroups fit a compute unit only while two images fit its LDS: K = N = 10240, M = 2048,
+    //  H = 36000: 3849 us against 3583 us with the 256 tile)
+    if (pl.tile == 256 && elem_bytes == 4 && cover128 && tiles256 >= kComputeUnits && (size_t)pitch * sizeof(float) <= 78 * 1024) {
+      // fp32, at least as many 256 tiles as compute units: the two tiles by how they fill their
+      // rounds (K = N = 10240 is six rounds and a quarter of the one, twelve and a half pairs of
+      // the other: M = 2048 3520 -> 3317 us, M = 4096 6972 -> 6486 us; K = N = 6000, M = 1024:
+      // 848 -> 698 us); the image stores of paired workgroups are half hidden behind each other
+      const long long tiles128 = tile_count(K, N, 128);
+      const double work_us = 2.0 * (double)M * K * N / 137e6, image_us = (double)pitch * 8.0 / 5e6;
+      const double t256 = work_us / filled_256(tiles256) + (double)tiles256 * image_us;
+      const double t128 = work_us / (kPairRate128F32 * filled_128(tiles128)) + 0.5 * (double)tiles128 * image_us;
+      if (t128 < t256 * 0.99) pl.tile = 128;
+    }
     if (pl.tile == 256 && elem_bytes == 2 && cover128) {
       // 16-bit: the two tiles by estimated time.  Fitted on MI355X (weight-grad, 256 workgroups):
       // a 256 workgroup pays about 5.5 steps of 64 rows for its fill, its image rounds and the
@@ -247,10 +276,15 @@ static inline WeightGradPlan plan_weight_grad(int M, int K, int N, int H, int BK
     }
   } else {
     pl.tile = pick_tile(K, N, elem_bytes, t);
-    // fp32 with the tiles stored for the fold kernel: a 256 workgroup is alone on its compute unit
-    // and its 256 KB of stores are exposed after a short loop over M; two 128 workgroups hide each
-    // other's (K = N = 10240: M = 128 455 -> 401 us, M = 1024 1938 -> 1797 us, M = 4096 7002 -> 6449 us)
-    if (pl.tile == 256 && elem_bytes == 4 && M <= 8192 && t.fold != -1 && plan_fold(K, N, H, BK, BN, 1).use) pl.tile = 128;
+    // fp32 with the tiles stored for the fold kernel: by how the two tiles fill their rounds when
+    // there are at least as many 256 tiles as compute units (K = N = 10240: M = 128 455 -> 401 us,
+    // M = 1024 1938 -> 1797 us, M = 4096 7002 -> 6449 us; K = N = 4096, one round exactly, stays
+    // with the 256 tile: 1043 against 1085 us); with fewer, a short M takes the 128 tile, whose
+    // paired workgroups hide each other's stores
+    if (pl.tile == 256 && elem_bytes == 4 && t.fold != -1 && plan_fold(K, N, H, BK, BN, 1).use) {
+      const long long t256 = tile_count(K, N, 256), t128 = tile_count(K, N, 128);
+      if (t256 >= kComputeUnits ? kPairRate128F32 * filled_128(t128) > filled_256(t256) * 1.01 : M <= 2048) pl.tile = 128;
+    }
   }
   const long long tiles = (long long)((K + pl.tile - 1) / pl.tile) * ((N + pl.tile - 1) / pl.tile);
   const int TR = slice_unit(pl.tile, elem_bytes);
