@@ -41,8 +41,6 @@ def weight_grad_hashed(input, output_grad, init_factor, M, K, N, H, R, BLOCK_SIZ
     if input.dtype != output_grad.dtype:
         raise TypeError("input is %s but output_grad is %s" % (input.dtype, output_grad.dtype))
     lib = _lib.load()
-    x, ldx = _lib.rows(input)
-    dy, lddy = _lib.rows(output_grad)
     code = _lib.dtype_code(output_grad)
     flags = 0
     if out is None:
@@ -59,11 +57,14 @@ def weight_grad_hashed(input, output_grad, init_factor, M, K, N, H, R, BLOCK_SIZ
             raise TypeError("out must be float32 or %s, got %s" % (output_grad.dtype, out.dtype))
         if accumulate:
             flags |= _lib.WG_ACCUMULATE
-    bias_grad = torch.empty((N,), device=output_grad.device, dtype=output_grad.dtype) if with_bias_grad else None
     if M == 0:   # an empty batch contributes a zero gradient (the reference returns its zeros(H))
         if not accumulate:
             out.zero_()
-        return out, (bias_grad.zero_() if with_bias_grad else None)
+        return out, (torch.zeros((N,), device=output_grad.device, dtype=output_grad.dtype) if with_bias_grad else None)
+    columns = N
+    x, ldx, K = _lib.whole_pieces(input, K)          # (K, N: the extents the call is made with)
+    dy, lddy, N = _lib.whole_pieces(output_grad, N)
+    bias_grad = torch.empty((N,), device=output_grad.device, dtype=output_grad.dtype) if with_bias_grad else None
     tuning = _lib.current_tuning()
     need = _lib.host_query("rz_weight_grad_hashed_workspace_bytes", M, K, N, H, BLOCK_SIZE_K, BLOCK_SIZE_N, code,
                            flags, int(with_bias_grad))
@@ -84,7 +85,7 @@ def weight_grad_hashed(input, output_grad, init_factor, M, K, N, H, R, BLOCK_SIZ
             x.data_ptr(), dy.data_ptr(), out.data_ptr(), bias_grad.data_ptr() if with_bias_grad else None,
             ws.data_ptr() if need else None, need, M, K, N, H, BLOCK_SIZE_K, BLOCK_SIZE_N, R, hash_levels,
             float(init_factor), ldx, lddy, code, flags, tuning, stream))
-    return out, bias_grad
+    return out, (bias_grad[:columns] if with_bias_grad else None)
 
 
 def rz_linear_backward_weight_grad_tl(input: torch.Tensor, output_grad: torch.Tensor, init_factor: float,
@@ -154,7 +155,7 @@ def input_grad_hashed(output_grad, hashed_weight, init_factor, M, K, N, H, R, BK
         raise TypeError("output_grad is %s but hashed_weight is %s" % (output_grad.dtype, hashed_weight.dtype))
     if M == 0:
         return torch.empty((0, K), device=output_grad.device, dtype=output_grad.dtype)
-    dy, lddy = _lib.rows(output_grad)
+    dy, lddy, N = _lib.whole_pieces(output_grad, N)   # (N: the extent the call is made with)
     hw = hashed_weight.contiguous()
     input_grad = torch.empty((M, K), device=output_grad.device, dtype=output_grad.dtype)
     lib = _lib.load()

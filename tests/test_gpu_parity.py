@@ -518,3 +518,35 @@ def test_random_shapes_16bit(oracle, shape):
     assert_close(f(dx), oracle.input_grad(dy64, hw64, K, BK, BN, R, 0.75), dtype, "dX")
     assert_close(f(dhw), oracle.weight_grad(x64, dy64, H, BK, BN, R, 0.75), dtype, "dHW")
     assert_close(f(dbias), dy64.sum(axis=0), dtype, "dbias")
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=lambda d: str(d).split(".")[-1])
+@pytest.mark.parametrize("shape", [(1100, 1023, 1001, 40000, 32, 64), (1030, 1025, 2047, 300000, 64, 64)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_large_16_bit_operands_with_odd_rows_are_padded_to_whole_pieces(oracle, shape, dtype):
+    """K and N that are not multiples of 8 would keep the 16-bit kernels off their direct-to-LDS
+    path; the launchers copy a large operand into zero-padded rows once and make the call with
+    the padded extent.  All three products and the bias gradient against the oracle; untouched
+    slots of dHW stay zero (the padding adds zeros to slots that the tiles cover anyway)."""
+    from rzlinear_amd import _lib
+    from rzlinear_amd.impl.RzLinearBackward import (rz_linear_backward_input_grad_tl,
+                                                    rz_linear_backward_weight_bias_grad_tl)
+    from rzlinear_amd.impl.RzLinearForward import rz_linear_forward_bias_tl
+    M, K, N, H, BK, BN = shape
+    _say("odd rows, padded", shape, dtype)
+    (x, hw, dy), (x64, hw64, dy64) = make_inputs(M, K, N, H, dtype, seed=31)
+    assert _lib.whole_pieces(x, K)[2] == (K + 7) // 8 * 8 and _lib.whole_pieces(dy, N)[2] == (N + 7) // 8 * 8
+    bias = torch.randn((N,), generator=torch.Generator().manual_seed(5)).to(dtype)
+    kw = dict(BLOCK_SIZE_K=BK, BLOCK_SIZE_N=BN)
+    y = rz_linear_forward_bias_tl(x, hw, bias.cuda(), 1.0, M, K, N, H, *rargs(R1024), **kw)
+    dx = rz_linear_backward_input_grad_tl(dy, hw, 1.0, M, K, N, H, *rargs(R1024), **kw)
+    dhw, dbias = rz_linear_backward_weight_bias_grad_tl(x, dy, 1.0, M, K, N, H, *rargs(R1024), **kw)
+    torch.cuda.synchronize()
+    assert y.shape == (M, N) and dx.shape == (M, K) and dhw.shape == (H,) and dbias.shape == (N,)
+    f = lambda t: t.float().cpu().numpy()
+    assert_close(f(y), oracle.forward(x64, hw64, N, BK, BN, R1024) + bias.double().numpy()[None, :], dtype, "Y")
+    assert_close(f(dx), oracle.input_grad(dy64, hw64, K, BK, BN, R1024), dtype, "dX")
+    ref = oracle.weight_grad(x64, dy64, H, BK, BN, R1024)
+    assert_close(f(dhw), ref, dtype, "dHW")
+    assert (f(dhw)[ref == 0] == 0).all()
+    assert rel_err(f(dbias), dy64.sum(axis=0)) <= TOL[dtype]
