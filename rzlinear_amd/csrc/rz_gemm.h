@@ -744,6 +744,12 @@ struct GemmKernel {
       // are issued into it; they have a whole step to land and are waited for just before the
       // barrier of step s+1.
       constexpr int NKS = TR / KS / WK;   // sub-steps of this wavefront's part of an R step
+      // fp32: left to itself the compiler moves a sub-step's fragment reads down to just before
+      // the MFMAs that use them (read, wait, four MFMAs).  Holding them a sub-step ahead, as
+      // written, is faster in the 64 tile (1024^3: 28.7 -> 27.4 us forward, 33.8 -> 31.4 us
+      // weight-grad) and in the 256 tile's input-grad (M = 32768, K = N = 2048: 2110 -> 2003 us),
+      // slower elsewhere (4096^3 forward 996 -> 1031 us; the 128 tile at 2048^3 154 -> 164 us).
+      constexpr bool kPinFrags = !kDirect && sizeof(T) == 4 && (TI == 64 || (TI == 256 && OP == kInputGrad));
       static_assert(NKS >= 3 && NKS * KS * WK == TR, "pipeline needs at least three sub-steps per R step");
       const int ks0 = wave_k * NKS;
       Frag fa[2][MI], fb[2][MJ];
@@ -775,6 +781,7 @@ struct GemmKernel {
         for (int ks = 0; ks < NKS; ks++) {
           if (ks + 1 < NKS) {
             frags(st, ks + 1, (ks + 1) & 1);
+            if constexpr (kPinFrags) __builtin_amdgcn_sched_barrier(0);
           } else {
             if constexpr (kDirect) {
               // the loads of step s+1 (the only ones in flight) must have landed
