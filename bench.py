@@ -67,22 +67,22 @@ TRAFFIC = {
     # (factors from the copy calibration in the same profile)
     ("square4096", "bf16"): {
         "profile": "profiles/rz_gemm_bf16_square4096.txt",
-        "bytes": {"forward": int((16682.2 * 2.0 + 32768.0) * 1024),       # algorithmic: 64.03 MiB
-                  "input_grad": int((16684.0 * 2.0 + 32768.0) * 1024),
-                  "weight_grad": int((98463.2 * 2.0 + 16784.5) * 1024)},  # X, dY re-read by the XCDs' tile groups; + partial images
+        "bytes": {"forward": int((16684.7 * 2.0 + 32768.0) * 1024),       # algorithmic: 64.03 MiB
+                  "input_grad": int((16687.2 * 2.0 + 32768.0) * 1024),
+                  "weight_grad": int((98460.5 * 2.0 + 16784.3) * 1024)},  # X, dY re-read by the XCDs' tile groups; + partial images
     },
     ("square4096", "fp32"): {
         "profile": "profiles/rz_gemm_fp32_square4096.txt",
-        "bytes": {"forward": int((34692.2 * 2.0 + 68352.0) * 1024),       # algorithmic: 128.06 MiB
-                  "input_grad": int((33275.6 * 2.0 + 65536.0) * 1024),
-                  "weight_grad": int((196817.3 * 2.0 + 16784.0) * 1024)},
+        "bytes": {"forward": int((34806.3 * 2.0 + 70144.0) * 1024),       # algorithmic: 128.06 MiB
+                  "input_grad": int((33265.9 * 2.0 + 67072.0) * 1024),
+                  "weight_grad": int((196838.4 * 2.0 + 17808.0) * 1024)},
     },
     ("ffn", "bf16"): {
         "profile": "profiles/rz_gemm_fold_bf16_ffn.txt",
-        "bytes": {"forward": int((71071.4 * 2.0 + 262144.0) * 1024),      # algorithmic: 320.1 MiB
-                  "input_grad": int((132344.1 * 2.0 + 65536.0) * 1024),
+        "bytes": {"forward": int((70906.4 * 2.0 + 262144.0) * 1024),      # algorithmic: 320.1 MiB
+                  "input_grad": int((132355.8 * 2.0 + 65536.0) * 1024),
                   # contraction (X, dY re-read by the XCDs' tile groups; X^T.dY written tile by tile: 256 MiB)
-                  "weight_grad": int((786592.1 * 2.0 + 262144.0) * 1024)},
+                  "weight_grad": int((786918.0 * 2.0 + 262144.0) * 1024)},
     },
 }
 
