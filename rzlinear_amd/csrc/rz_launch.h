@@ -97,14 +97,14 @@ static inline double tile_score(int I, int J, int t, int elem_bytes) {
 
 // Relative throughput of `wgs` workgroups of tile t (see tile_score_full, which this restates for
 // a workgroup count that includes the slices of a cut contraction).
-static inline double tile_rate(double wgs, int t, int elem_bytes) {
+static inline double tile_rate(double wgs, int t, int elem_bytes, double lo64_f32 = 0.60) {
   const bool f32 = elem_bytes == 4;
   // (32 x 64, four wavefronts: half a 64 workgroup's work in about its time, up to eight resident)
   if (t == 32) return occupancy_rate(wgs, 8, 0.40, 0.80);
   const int slots = (t == 256) ? 1 : (t == 128 ? 2 : 4);
   // (the 16-bit 64 tile: 0.24 with one workgroup per compute unit, 0.33 from two on — K = 2048, N = 8192:
   //  M = 128 14.9 us, M = 256 22.7 us; priced at 0.16 it lost to cut 128 tiles that take 21 and 30 us)
-  const double lo = (t == 256) ? 1.0 : (t == 128 ? (f32 ? 0.86 : 0.51) : (f32 ? 0.60 : 0.24));
+  const double lo = (t == 256) ? 1.0 : (t == 128 ? (f32 ? 0.86 : 0.51) : (f32 ? lo64_f32 : 0.24));
   const double hi = (t == 256) ? 1.0 : (t == 128 ? (f32 ? 0.90 : 0.75) : (f32 ? 0.80 : 0.33));
   return occupancy_rate(wgs, slots, lo, hi, (t == 64 && !f32) ? 2 : 0);
 }
@@ -492,6 +492,11 @@ static inline SplitPlan plan_split(int I, int J, int R, int elem_bytes, const rz
     const long long tiles = tile_count(I, J, tile);
     const int r_steps = (R + TR - 1) / TR;
     const double useful = (double)I * (double)J / ((double)tiles * tile * tile_cols(tile));
+    // (the fp32 64 tile of forward / input-grad, eight wavefronts: 0.67 of the 256 tile's rate with one
+    //  workgroup per compute unit when no tile or step is partial — K = 2048, N = 8192, M = 128: 45 us
+    //  whole against 52 us with the 128 tile cut in four; the bounds-checked form stays at 0.60)
+    const bool whole = I % tile == 0 && J % tile_cols(tile) == 0 && R % TR == 0;
+    const double lo64 = whole ? 0.67 : 0.60;
     for (int want = 1; want <= 16; want++) {
       if (want > 1 && t.split == -1) break;
       const int steps_per = (r_steps + want - 1) / want;
@@ -499,7 +504,7 @@ static inline SplitPlan plan_split(int I, int J, int R, int elem_bytes, const rz
       if (slices != want) continue;                           // (the same cut as a smaller `want`)
       if (slices > 1 && steps_per * (TR * elem_bytes / 128) < 4) break;   // slices of a few steps are all fill and drain
       const double steps = (double)steps_per * (TR * elem_bytes / 128);
-      const double rate = peak * tile_rate((double)tiles * slices, tile, elem_bytes) * useful * steps / (steps + 2.0);
+      const double rate = peak * tile_rate((double)tiles * slices, tile, elem_bytes, lo64) * useful * steps / (steps + 2.0);
       double us = 2.0 * (double)I * (double)J * (double)R / rate + 4.0;
       if (slices > 1) us += (2.0 * slices * (double)I * J * 4.0 + (double)I * J * elem_bytes) / 4.0e6 + 4.0;
       // (near ties go to the larger tile and the fewer slices, which come first)
