@@ -12,11 +12,14 @@ roofline of the slowest of the three kernels, the dense torch.matmul (hipBLASLt/
 the same GPU under the same warm-up / step counts, a short sweep over the other baseline
 configurations and the reference's CPU path timed on the host cores.
 
-Order of the GPU work (the GPU's clock governor needs some 30 ms of load to settle after an
-idle period, so what runs when is part of the protocol and is reported):
-  output check -> dense legs (W warm-up + K timed) -> rz legs (W warm-up + K timed: the headline)
-  -> dense legs again (W + K) -> sweep -> CPU baseline.
-The dense rate quoted against the headline is the mean of the two dense runs around it.
+Order of the GPU work (the GPU's clock governor needs tens of milliseconds of load to settle after
+an idle period, so what runs when is part of the protocol and is reported):
+  output check -> clock settling (untimed, independent of --warmup: dense and rz legs alternate
+  until three consecutive passes take the same time to within 2 %, at most 0.3 s) -> dense legs
+  (W warm-up + K timed) -> rz legs (W warm-up + K timed: the headline) -> dense legs again (W + K)
+  -> sweep (each row settles the same way first) -> practical MFMA ceiling -> CPU baseline.
+The dense rate quoted against the headline is the mean of the two dense runs around it;
+`rz_over_dense_settled` is against the faster of the two.
 """
 import argparse
 import ctypes
@@ -53,8 +56,11 @@ WORKLOADS = {
 }
 # the baseline configurations beside the headline one: (workload, dtype) rows of the sweep
 SWEEP = [("cpu_ref_1024", "fp32"), ("square1024", "fp32"), ("square1024", "bf16"), ("square2048", "fp32"),
-         ("square2048", "bf16"), ("square4096", "fp32"), ("square4096", "bf16"), ("rec_mlp", "bf16"),
-         ("ffn", "bf16"), ("collision", "fp32")]
+         ("square2048", "bf16"), ("square4096", "fp32"), ("square4096", "bf16"), ("square4096", "fp16"),
+         ("rec_mlp", "bf16"), ("ffn", "bf16"), ("collision", "fp32"),
+         # the reference's own benchmark grid at its large size (python/bench/bench.py:10-11 runs it in fp32)
+         ("grid_32_10240", "fp32"), ("grid_128_10240", "fp32"), ("grid_1024_10240", "fp32"),
+         ("grid_32_10240", "bf16"), ("grid_128_10240", "bf16"), ("grid_1024_10240", "bf16")]
 # dense MFMA peaks of MI355X, TFLOP/s
 PEAK = {"bf16": 2500.0, "fp16": 2500.0, "fp32": 157.3}
 # HBM bytes per launch of each leg, from rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE (KiB per
@@ -126,7 +132,7 @@ def make_workload(torch, _lib, name, dname, dev):
     # function of the layer's constants alone, built once like the hash constants themselves and
     # kept on the device) goes with every call, as the package's own launchers do it.
     plan = None
-    if _lib.plan_query(2, M, K, N, H, BK, BN, code)["mode"] in ("window", "fold"):
+    if _lib.plan_query(2, M, K, N, H, BK, BN, code, planned=True)["mode"] in ("window", "fold"):
         plan = _lib.layer_plan(K, N, H, BK, BN, R, 2, dev)
 
     def wgrad():
@@ -156,6 +162,34 @@ def make_workload(torch, _lib, name, dname, dev):
 
 
 EVENT_EVERY = 4   # steps between two steps whose legs are bracketed by HIP events
+
+
+def algorithmic_bytes(wl):
+    """Least HBM bytes of each leg: forward s(MK + MN + H), input-grad s(MN + MK + H), weight-grad
+    s(MK + MN) + 4H (the gradient is summed in fp32), s = bytes per element."""
+    M, K, N, H = (wl[k] for k in ("M", "K", "N", "H"))
+    s = 4 if wl["dname"] == "fp32" else 2
+    return {"forward": s * (M * K + M * N + H), "input_grad": s * (M * N + M * K + H),
+            "weight_grad": s * (M * K + M * N) + 4 * H}
+
+
+def settle(torch, leg_sets, cap_s=0.3, agree=0.02):
+    """Untimed: passes over every leg of `leg_sets` (dense and rz alternating, so that neither finds the
+    clocks as the other left them) until three consecutive passes take the same time to within
+    `agree`, for at most `cap_s` seconds.  Returns (passes, ms of the last pass)."""
+    legs = [f for legs in leg_sets for _, f in legs]
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    last, t_end, n = [], time.perf_counter() + cap_s, 0
+    while True:
+        a.record()
+        for f in legs:
+            f()
+        b.record()
+        b.synchronize()
+        n += 1
+        last = (last + [a.elapsed_time(b)])[-3:]
+        if (len(last) == 3 and max(last) <= min(last) * (1.0 + agree)) or time.perf_counter() >= t_end:
+            return n, last[-1]
 
 
 def run_legs(torch, legs, warmup, steps):
@@ -256,6 +290,45 @@ def api_level(torch, wl, warmup, steps):
             "rz_over_nn_linear": round(d_ms / rz_ms, 4)}
 
 
+def mfma_ceiling(torch, _lib, wl, launches=100):
+    """The MFMA rate this GPU sustains on the matrix work alone of one contraction of the headline
+    shape, with operands distributed like the workload's: rz_mfma_probe runs the inner loop's
+    MFMA stream (256 workgroups of eight wavefronts, 32 MFMA 32x32x16 per wavefront and step, as
+    many steps as make 2*M*N*K flop) without global loads, hashing or stores — mode 0 out of
+    registers, mode 1 with the fragment reads from LDS and the barrier per step.  The gap between
+    these figures and the data sheet's peak is the clock under matrix load (reported), not the
+    kernels'.  16-bit types only."""
+    if wl["dname"] == "fp32":
+        return None
+    lib = _lib.load()
+    dev = wl["x"].device
+    stream = torch.cuda.current_stream(dev).cuda_stream
+    operands = wl["x"].reshape(-1)[:32768].contiguous()           # 64 KB of the workload's own X
+    wgs = 256
+    steps = max(1, int(round(wl["flop_gemm"] / (wgs * 8 * 32 * 32768.0))))
+    out = torch.empty((wgs * 512,), dtype=torch.float32, device=dev)
+    ticks = torch.zeros((2 * wgs,), dtype=torch.int64, device=dev)
+    res = {"what": "rz_mfma_probe: %d workgroups x 8 wavefronts x %d steps x 32 MFMA 32x32x16 (%.1f GFLOP per launch), operands = "
+                   "the workload's X; %d launches after as many untimed" % (wgs, steps, wgs * 8 * steps * 32 * 32768 / 1e9, launches)}
+    for mode, key in ((0, "registers_only"), (1, "with_lds_fragments_and_barrier")):
+        def launch():
+            _lib.check(lib.rz_mfma_probe(operands.data_ptr(), out.data_ptr(), ticks.data_ptr(), wgs, steps, mode, wl["code"], stream))
+        for _ in range(launches):
+            launch()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        a.record()
+        for _ in range(launches):
+            launch()
+        b.record()
+        torch.cuda.synchronize()
+        ms = a.elapsed_time(b) / launches
+        t = ticks.view(wgs, 2).double().mean(0)
+        res[key] = {"us_per_launch": round(ms * 1e3, 2), "tflops": round(tflops(wgs * 8 * steps * 32 * 32768.0, ms), 1),
+                    "shader_clock_mhz": round(float(t[0] / (t[1] / 100.0)), 0)}
+    return res
+
+
 def tflops(flop, ms):
     return flop / (ms * 1e-3) / 1e12
 
@@ -272,6 +345,7 @@ def main():
     ap.add_argument("--no-sweep", action="store_true")
     ap.add_argument("--no-check", action="store_true")
     ap.add_argument("--no-api", action="store_true", help="skip the module-level (autograd) timing")
+    ap.add_argument("--no-ceiling", action="store_true", help="skip the MFMA-only probe (practical ceiling)")
     ap.add_argument("--cpu-budget", type=float, default=15.0, help="seconds of CPU-path timing")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MiB",
                     help="only run a plain device-to-device copy of this many MiB (five launches) and exit: "
@@ -307,6 +381,8 @@ def main():
     peak = PEAK[dname]
 
     check = None if args.no_check else output_check(torch, _lib, wl)
+
+    settled = settle(torch, [wl["legs"]] if args.no_dense else [wl["dense_legs"], wl["legs"]])
 
     dense_runs = []
     if not args.no_dense:
@@ -347,6 +423,7 @@ def main():
             "fwd_bwd_tflops": round(dense_step_tf, 2),
             "fwd_bwd_tflops_before_after": [round(tflops(3 * flop_gemm, r[0]), 2) for r in dense_runs],
             "rz_over_dense": round(value / dense_step_tf, 4),
+            "rz_over_dense_settled": round(value / max(tflops(3 * flop_gemm, r[0]) for r in dense_runs), 4),
             "rz_over_dense_per_kernel": {k: round(d_ms[k] / leg_ms[k], 4) for k in leg_ms},
         }
 
@@ -355,6 +432,7 @@ def main():
     if not args.no_sweep:
         sweep = []
         sw_warm, sw_steps = 5, 20
+        legs_of = ("forward", "input_grad", "weight_grad")
         for name, dn in SWEEP:
             if (name, dn) == (args.workload, dname):
                 row_rz, row_d = (ms_per_step, leg_ms), None
@@ -363,13 +441,22 @@ def main():
                 w2 = wl
             else:
                 w2 = make_workload(torch, _lib, name, dn, dev)
+                settle(torch, [w2["legs"]] if args.no_dense else [w2["dense_legs"], w2["legs"]], cap_s=0.15)
                 row_d = run_legs(torch, w2["dense_legs"], sw_warm, sw_steps) if not args.no_dense else None
                 row_rz = run_legs(torch, w2["legs"], sw_warm, sw_steps)
             fg = w2["flop_gemm"]
             row = {"workload": name, "dtype": dn, "M": w2["M"], "K": w2["K"], "N": w2["N"], "H": w2["H"],
                    "rz_tflops": {k: round(tflops(fg, v), 2) for k, v in row_rz[1].items()},
                    "rz_fwd_bwd_tflops": round(tflops(3 * fg, row_rz[0]), 2),
-                   "pct_mfma_peak": round(100.0 * tflops(3 * fg, row_rz[0]) / PEAK[dn], 2)}
+                   "pct_mfma_peak": round(100.0 * tflops(3 * fg, row_rz[0]) / PEAK[dn], 2),
+                   # roofline fraction of the row's slowest leg (weight_grad = every kernel of the call)
+                   "frac": round(min(tflops(fg, row_rz[1][k]) for k in legs_of) / PEAK[dn], 4),
+                   "slowest": max(legs_of, key=lambda k: row_rz[1][k])}
+            tr = TRAFFIC.get((name, dn))
+            if tr:   # measured HBM bytes of the contraction kernel of each leg over the least possible
+                alg = algorithmic_bytes(w2)
+                row["traffic_over_algorithmic"] = {k: round(tr["bytes"][k] / alg[k], 2) for k in legs_of}
+                row["traffic_source"] = tr["profile"]
             if row_d is not None:
                 row["dense_tflops"] = {k: round(tflops(fg, v), 2) for k, v in row_d[1].items()}
                 row["rz_over_dense"] = {k: round(row_d[1][k] / row_rz[1][k], 3) for k in row_rz[1]}
@@ -378,8 +465,10 @@ def main():
             if w2 is not wl:
                 del w2
                 torch.cuda.empty_cache()
-        sweep = {"protocol": "warm-up %d + %d timed steps per configuration (dense legs first, then rz); the headline "
-                             "configuration's row repeats the headline run" % (sw_warm, sw_steps), "rows": sweep}
+        sweep = {"protocol": "per configuration: clocks settled as for the headline (at most 0.15 s), then warm-up %d + %d "
+                             "timed steps (dense legs first, then rz); the headline configuration's row repeats the "
+                             "headline run; frac = slowest leg / MFMA peak of the dtype" % (sw_warm, sw_steps),
+                 "rows": sweep}
 
     # ---- the same step through the package's module and autograd (what a user of the reference
     # calls: python/bench/bench.py:44 times `rz(a)`), outputs allocated by the API, beside
@@ -387,6 +476,11 @@ def main():
     api = None
     if not args.no_api:
         api = api_level(torch, wl, 5, 20)
+
+    ceiling = None if args.no_ceiling else mfma_ceiling(torch, _lib, wl)
+    if ceiling is not None:
+        roofline["practical_ceiling"] = ceiling
+        roofline["frac_of_practical_ceiling"] = round(leg_tflops[slowest] / ceiling["registers_only"]["tflops"], 4)
 
     cpu_baseline = None
     if not args.no_cpu_baseline:
@@ -429,6 +523,8 @@ def main():
                    "weight_grad_layer_plan": bool(wl["layer_plan"])},
         "pct_mfma_peak": round(100.0 * value / peak, 2),
         "output_check": check,
+        "clock_settling": {"passes": settled[0], "last_pass_ms": round(settled[1], 4),
+                           "rule": "untimed passes over dense + rz legs until three in a row agree within 2 %, at most 0.3 s"},
         "roofline": roofline,
         "dense_gemm": dense,
         "api_level": api,

@@ -81,8 +81,12 @@ typedef struct rz_tuning {
   int split;      /* forward / input-grad: 0 = automatic, -1 = never split the contraction */
   int clamp;      /* ragged 16-bit shapes: 0 = automatic, -1 = always the bounds-checked kernels */
   int fold;       /* weight-grad with a hashed_weight too large for LDS: 0 = automatic, 1 = X^T.dY stored
-                     tile by tile and folded into dHW by a second kernel whenever possible, -1 = never */
-  int reserved;   /* must be 0 */
+                     tile by tile and folded into dHW by a second kernel whenever possible, 2 = the same
+                     with the windowed fold kernel even for the few tiles that have a kernel of their own,
+                     -1 = never */
+  int poll_limit; /* weight-grad by windows: 0 = default; > 0 = how often a wavefront looks at the flags of the
+                     earlier strips it waits for before it gives up and the window is stored as NaN (a bounded
+                     wait; tests set a tiny value to see every wavefront leave the kernel all the same) */
 } rz_tuning;
 
 /* Library / ABI version (major*10000 + minor*100 + patch). */
@@ -195,7 +199,9 @@ int rz_weight_grad(const void* X, const void* dY, void* dHW, void* workspace,
  * for which rz_weight_grad would store X^T.dY tile by tile in more than 32 MiB takes the scatter
  * kernel with global atomics instead; a problem that needs more than 32 MiB even so is refused
  * with RZ_ERR_SCRATCH_LIMIT (at M = N = K = 4096, H = 16778 the need is 17 MB).  The first call on a device looks the array's
- * address up (make that call outside a graph capture).  All calls on one GPU share the one array:
+ * address up (make that call outside a graph capture).  The array used is that of the CURRENT device, which must be
+ * the device that holds dHW (and the other operands, and the stream): a call whose dHW lives on another device, or is
+ * not device memory at all, is refused with RZ_ERR_BAD_ARGUMENT.  All calls on one GPU share the one array:
  * calls that overlap in time on the same GPU — different streams, or different host threads —
  * race on it and must be serialised by the caller; calls on one stream are ordered and safe.
  * Nothing in the array needs to survive between calls, and each call writes what it reads.
@@ -272,7 +278,9 @@ int rz_weight_grad_hashed(const void* X, const void* dY, void* dHW, void* dbias,
  *   rz_weight_grad_planned  rz_weight_grad_hashed with that device copy; the workspace is asked
  *                         for as for rz_weight_grad_hashed (never more is needed).  The plan must
  *                         have been built for the same K, N, H, BK, BN, R and hash_levels: the
- *                         size is checked, the contents cannot be from the host.
+ *                         size is checked on the host; the plan's header (shapes, tile, hash and a
+ *                         checksum of R) is checked by the kernels that read it, which store NaN
+ *                         into dHW instead of following a plan of another layer.
  * No counterpart in the reference, whose kernels hash every tile offset on every call
  * (impl/RzLinearBackward.py:369).
  */
@@ -289,13 +297,17 @@ int rz_weight_grad_planned(const void* X, const void* dY, void* dHW, void* dbias
  * How a call would be carried out (host-side, touches no device): which C tile, how many
  * slices of the contracted dimension and how long each, which kernel form.  op: 0 = forward,
  * 1 = input-grad, 2 = weight-grad (flags / with_dbias as for rz_weight_grad_hashed, else 0).
+ * RZ_PLAN_WITH_LAYER_PLAN in flags: answer for a call that carries a layer plan (rz_weight_grad_planned), which
+ * changes what the window kernel costs and hence when it is taken.
  * Fills out[8] = { C-tile edge, slices, contracted elements per slice, contracted elements per
- * kernel step, mode, workgroups, 0, 0 } with mode 0 = plain store, 1 = split contraction with
+ * kernel step, mode, workgroups, workgroups per window of the fold kernel (mode 5, else 0), windows of dHW
+ * (modes 4 and 5, else 0) } with mode 0 = plain store, 1 = split contraction with
  * fp32 partial planes, 2 = weight-grad through LDS images of dHW, 3 = weight-grad by global
  * atomics, 4 = weight-grad by windows of dHW, 5 = weight-grad stored tile by tile and folded
  * into dHW by a second kernel.  For tests of the planning logic and for tuning; no counterpart in the
  * reference.
  */
+#define RZ_PLAN_WITH_LAYER_PLAN 0x100u
 int rz_plan_query(int op, int M, int K, int N, int H, int BK, int BN, int dtype, unsigned flags,
                   int with_dbias, const rz_tuning* tuning, int32_t out[8]);
 
@@ -334,6 +346,23 @@ int rz_sgd_step(void* param, const void* grad, float* momentum_buf, float* maste
 int rz_adam_step(void* param, const void* grad, float* exp_avg, float* exp_avg_sq, float* master, int64_t n,
                  int param_dtype, int grad_dtype, float lr, float beta1, float beta2, float eps,
                  float weight_decay, int decoupled, int step, float grad_scale, void* stream);
+
+/*
+ * Measurement aid, no counterpart in the reference: the MFMA rate this GPU sustains on the
+ * matrix work of the contraction kernels' inner loop when nothing else is in the way.  Launches
+ * `workgroups` workgroups of eight wavefronts (one per compute unit fits); every wavefront issues
+ * steps * 32 MFMA 32x32x16 on eight accumulator blocks, i.e. a launch is
+ * workgroups * 8 * steps * 32 * 32768 flop.  mode 0: operands stay in registers; mode 1: fragments
+ * come out of LDS (six 1 KB reads per eight MFMA, one barrier per step), as in the real loop.
+ * operands: 64 KB of 16-bit values of `dtype` (RZ_BF16 or RZ_F16) in device memory — the clock
+ * under matrix load depends on how much the operand bits toggle, so pass values like the real
+ * data's.  out: workgroups * 512 floats (written, meaningless).  ticks: 2 * workgroups uint64:
+ * shader clocks and ticks of the constant 100 MHz clock that the first wavefront of each
+ * workgroup spent in the loop, which gives the shader clock under this load.  bench.py times
+ * the launches and reports the result next to the roofline of the data sheet's peak.
+ */
+int rz_mfma_probe(const void* operands, void* out, void* ticks, int workgroups, int steps, int mode,
+                  int dtype, void* stream);
 
 #ifdef __cplusplus
 }

@@ -24,7 +24,7 @@ EXPORTS = (
     "rz_forward_hashed_workspace_bytes", "rz_input_grad_hashed_workspace_bytes",
     "rz_weight_grad_hashed_workspace_bytes", "rz_plan_query", "rz_weight_grad_static",
     "rz_layer_plan_bytes", "rz_layer_plan_build", "rz_weight_grad_planned",
-    "rz_sgd_step", "rz_adam_step",
+    "rz_sgd_step", "rz_adam_step", "rz_mfma_probe",
 )
 
 
@@ -33,7 +33,7 @@ class Tuning(ctypes.Structure):
     automatic).  Only tests and benchmarks set any of it."""
     _fields_ = [("tile", ctypes.c_int), ("stages", ctypes.c_int), ("lds_image", ctypes.c_int),
                 ("window", ctypes.c_int), ("split", ctypes.c_int), ("clamp", ctypes.c_int),
-                ("fold", ctypes.c_int), ("reserved", ctypes.c_int)]
+                ("fold", ctypes.c_int), ("poll_limit", ctypes.c_int)]
 
 
 # What the launchers of this package pass as `tuning` (None = automatic).  The C library keeps no
@@ -173,6 +173,8 @@ def load():
     lib.rz_adam_step.restype = c_int
     lib.rz_adam_step.argtypes = [c_vp, c_vp, f32p, f32p, f32p, c_i64, c_int, c_int, c_f, c_f, c_f, c_f, c_f, c_int,
                                  c_int, c_f, c_vp]
+    lib.rz_mfma_probe.restype = c_int
+    lib.rz_mfma_probe.argtypes = [c_vp, c_vp, c_vp, c_int, c_int, c_int, c_int, c_vp]
     lib.rz_materialize.restype = c_int
     lib.rz_materialize.argtypes = [c_vp, c_vp, c_int, c_int, c_int, c_int, c_int, i32p, c_int, c_i64,
                                    c_int, c_vp]
@@ -290,10 +292,16 @@ def layer_plan(K, N, H, BK, BN, R, hash_levels, device):
 PLAN_MODES = {0: "store", 1: "split", 2: "lds_image", 3: "atomics", 4: "window", 5: "fold"}
 
 
-def plan_query(op, M, K, N, H, BK, BN, dtype_code_, flags=0, with_dbias=False):
+PLAN_WITH_LAYER_PLAN = 0x100
+
+
+def plan_query(op, M, K, N, H, BK, BN, dtype_code_, flags=0, with_dbias=False, planned=False):
     """How the library would carry out a call (rz_plan_query), under the current tuning:
-    dict(tile, slices, slice_len, step, mode, workgroups).  op: 0 forward, 1 input-grad, 2 weight-grad."""
+    dict(tile, slices, slice_len, step, mode, workgroups, shares, windows).  op: 0 forward, 1 input-grad,
+    2 weight-grad; planned: the call will carry a layer plan (rz_weight_grad_planned)."""
     t = _tuning
+    if planned:
+        flags |= PLAN_WITH_LAYER_PLAN
     key = ("rz_plan_query", (op, M, K, N, H, BK, BN, dtype_code_, flags, int(with_dbias)),
            None if t is None else tuple(getattr(t, f) for f, _ in Tuning._fields_))
     ans = _host_answers.get(key)
@@ -301,5 +309,5 @@ def plan_query(op, M, K, N, H, BK, BN, dtype_code_, flags=0, with_dbias=False):
         out = (ctypes.c_int32 * 8)()
         check(load().rz_plan_query(op, M, K, N, H, BK, BN, dtype_code_, flags, int(with_dbias), current_tuning(), out))
         ans = _host_answers[key] = dict(tile=out[0], slices=out[1], slice_len=out[2], step=out[3],
-                                        mode=PLAN_MODES[out[4]], workgroups=out[5])
+                                        mode=PLAN_MODES[out[4]], workgroups=out[5], shares=out[6], windows=out[7])
     return dict(ans)

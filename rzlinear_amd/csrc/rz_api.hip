@@ -293,6 +293,15 @@ static void launch_reduce_partials(int out_dtype, const float* part, void* out, 
     hipLaunchKernelGGL((reduce_partials_kernel<f16_t, ACC, GROUPS>), grid, block, 0, s, part, (f16_t*)out, H, pitch, nparts);
 }
 
+static hipError_t launch_fold_small(const FoldParams& fp, hipStream_t s) {
+  const long long tiles = (long long)fp.tiles_k * fp.tiles_n;
+  if (fp.partial != nullptr || fp.out == nullptr || fp.shares != 1 || tiles > kFoldSmallTiles ||
+      fp.window != kFoldSmallThreads || (long long)fp.windows * fp.window < fp.H)
+    return hipErrorInvalidValue;
+  hipLaunchKernelGGL(fold_small_kernel<1>, dim3((unsigned)fp.windows), dim3(kFoldSmallThreads), 0, s, fp);
+  return hipGetLastError();
+}
+
 static hipError_t launch_fold(const FoldParams& fp, hipStream_t s) {
   static std::atomic<uint64_t> raised{0};
   const size_t lds = fold_lds_bytes(fp.window);
@@ -420,6 +429,7 @@ static int weight_grad_impl(const void* X, const void* dY, void* dHW, void* dbia
       w.tiles_n = (N + BN - 1) / BN;
       w.accumulate = accumulate ? 1 : 0;
       w.out_f32 = dhw_dtype == RZ_F32 ? 1 : 0;
+      w.poll_limit = tuning.poll_limit > 0 ? tuning.poll_limit : kWindowPollLimit;
       hipError_t e = dtype == RZ_F32 ? launch_window_f32(w, wp.windows, s)
                      : dtype == RZ_BF16 ? launch_window_bf16(w, wp.windows, s)
                                         : launch_window_f16(w, wp.windows, s);
@@ -443,8 +453,12 @@ static int weight_grad_impl(const void* X, const void* dY, void* dHW, void* dbia
     if (launch_gemm(dtype, kWeightGrad, p, &plan, nullptr, tuning, s) != hipSuccess) return RZ_ERR_LAUNCH;
     FoldParams fp;
     fp.tiles = p.tiles_out;
+    fp.plan_header = nullptr;
     if (planned) {
       fp.offsets = layer_plan + lay.offsets_at;
+      fp.plan_header = layer_plan;
+    } else if (f.small) {
+      fp.offsets = nullptr;   // (the kernel hashes the few offsets it needs)
     } else {
       int32_t* offsets = (int32_t*)((char*)workspace + f.tiles_bytes + f.partial_bytes);
       hipLaunchKernelGGL(tile_offsets_kernel, dim3((p.out_tiles_k * p.out_tiles_n + 255) / 256), dim3(256), 0, s, offsets,
@@ -467,7 +481,7 @@ static int weight_grad_impl(const void* X, const void* dY, void* dHW, void* dbia
     fp.window = f.window;
     fp.windows = f.windows;
     fp.shares = f.shares;
-    if (launch_fold(fp, s) != hipSuccess) return RZ_ERR_LAUNCH;
+    if ((f.small ? launch_fold_small(fp, s) : launch_fold(fp, s)) != hipSuccess) return RZ_ERR_LAUNCH;
     if (f.shares > 1) {
       if (accumulate) launch_reduce_partials<true>(dhw_dtype, fp.partial, dHW, H, fp.pitch, f.shares, s);
       else launch_reduce_partials<false>(dhw_dtype, fp.partial, dHW, H, fp.pitch, f.shares, s);
@@ -515,11 +529,19 @@ static __device__ __align__(256) unsigned char scratch[kScratchBytes];
 static constexpr int kMaxDevices = 64;
 static std::atomic<void*> scratch_ptr[kMaxDevices];
 
-// Device address of this device's scratch array, or null (status in *st) if it cannot be had.
-static void* scratch_of_current_device(int* st) {
+// Device address of the current device's scratch array, or null (status in *st) if it cannot be
+// had.  `owned` is memory of the call (its dHW): the kernels will run where it lives, so it must be
+// device memory of the current device, or they would be handed another GPU's array.
+static void* scratch_of_current_device(const void* owned, int* st) {
   int dev = -1;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
     *st = RZ_ERR_LAUNCH;
+    return nullptr;
+  }
+  hipPointerAttribute_t attr;
+  if (hipPointerGetAttributes(&attr, owned) != hipSuccess || attr.type != hipMemoryTypeDevice || attr.device != dev) {
+    (void)hipGetLastError();   // (a pointer HIP does not know leaves an error behind: it is reported here, not later)
+    *st = RZ_ERR_BAD_ARGUMENT;
     return nullptr;
   }
   void* p = scratch_ptr[dev].load(std::memory_order_acquire);
@@ -721,8 +743,14 @@ RZ_API int rz_weight_grad_static(const void* X, const void* dY, void* dHW, int M
         return RZ_ERR_SCRATCH_LIMIT;
     }
   }
-  int st = RZ_OK;
-  void* ws = scratch_of_current_device(&st);
+  // (argument errors are reported as rz_weight_grad reports them, before the device is looked at)
+  if (X == nullptr || dY == nullptr || dHW == nullptr) return RZ_ERR_NULL_POINTER;
+  if (dtype_bytes(dtype) == 0) return RZ_ERR_BAD_DTYPE;
+  if (M < 1 || ldx < K || lddy < N) return RZ_ERR_BAD_SHAPE;
+  HashParams h;
+  int st = make_hash(&h, K, N, H, BK, BN, R, RZ_HASH_TWO_LEVEL);
+  if (st != RZ_OK) return st;
+  void* ws = scratch_of_current_device(dHW, &st);
   if (ws == nullptr) return st;
   return weight_grad_impl(X, dY, dHW, nullptr, ws, kScratchBytes, M, K, N, H, BK, BN, R, init_factor, ldx, lddy,
                           dtype, 0u, stream, RZ_HASH_TWO_LEVEL, &tuning);
@@ -827,7 +855,8 @@ RZ_API int rz_layer_plan_build(void* plan_host, size_t plan_bytes, int K, int N,
     start[0] = 0;
   }
   const int32_t header[kLayerPlanHeader] = {kLayerPlanMagic, kLayerPlanVersion, K, N, H, BK, BN, hash_levels, l.tiles,
-                                            l.windows, l.window, (int32_t)entries, l.strips_per_tile, 0, 0, 0};
+                                            l.windows, l.window, (int32_t)entries, l.strips_per_tile,
+                                            layer_plan_hash_sum(h), 0, 0};
   for (int i = 0; i < kLayerPlanHeader; i++) w[i] = header[i];
   return RZ_OK;
 }
@@ -845,8 +874,9 @@ RZ_API int rz_weight_grad_planned(const void* X, const void* dY, void* dHW, void
 
 RZ_API int rz_plan_query(int op, int M, int K, int N, int H, int BK, int BN, int dtype, unsigned flags,
                          int with_dbias, const rz_tuning* tuning, int32_t out[8]) {
-  (void)flags; (void)with_dbias;
+  (void)with_dbias;
   if (out == nullptr) return RZ_ERR_NULL_POINTER;
+  const bool planned = (flags & RZ_PLAN_WITH_LAYER_PLAN) != 0;
   const int eb = dtype_bytes(dtype);
   if (eb == 0) return RZ_ERR_BAD_DTYPE;
   if (M < 1 || K < 1 || N < 1 || H < 1) return RZ_ERR_BAD_SHAPE;
@@ -858,15 +888,20 @@ RZ_API int rz_plan_query(int op, int M, int K, int N, int H, int BK, int BN, int
   if (op == kWeightGrad) {
     const WeightGradPlan plan = plan_weight_grad(M, K, N, H, BK, BN, eb, t);
     WindowPlan wp = {};
-    if (!plan.lds_image()) wp = plan_window(M, K, N, H, BK, BN, eb, t, plan);
+    if (!plan.lds_image())
+      wp = plan_window(M, K, N, H, BK, BN, eb, t, plan, planned && layer_plan_layout(K, N, H, BK, BN).windows > 0);
     if (wp.use) {
-      out[0] = 0; out[1] = 1; out[2] = M; out[3] = 32; out[4] = 4; out[5] = wp.windows;
+      out[0] = 0; out[1] = 1; out[2] = M; out[3] = 32; out[4] = 4; out[5] = wp.windows; out[7] = wp.windows;
       return RZ_OK;
     }
     const KernelForm f = kernel_form(op, K, N, M, plan.r_chunk, plan.tile, plan.workgroups, eb, t);
     out[0] = plan.tile; out[1] = plan.splits; out[2] = plan.r_chunk; out[3] = f.step;
     out[4] = plan.fold.use ? 5 : plan.image_pitch > 0 ? 2 : 3;
     out[5] = (int32_t)plan.workgroups;
+    if (plan.fold.use) {
+      out[6] = plan.fold.shares;
+      out[7] = plan.fold.windows;
+    }
     return RZ_OK;
   }
   if (op != kForward && op != kInputGrad) return RZ_ERR_BAD_ARGUMENT;

@@ -33,12 +33,15 @@
 
 #include "../../include/rzlinear.h"
 #include "rz_common.h"
+#include "rz_launch.h"
 
 namespace rz {
 
 struct FoldParams {
   const float* tiles;   // [slices][tiles_k * tiles_n][BK * BN]
-  const int32_t* offsets;   // [tiles_k * tiles_n] where every tile starts in hashed_weight (hashed once, by another kernel)
+  const int32_t* offsets;   // [tiles_k * tiles_n] where every tile starts in hashed_weight (hashed once, by another kernel;
+                            // null for the few-tiles kernel: it hashes them itself)
+  const int32_t* plan_header;   // `offsets` belongs to a layer plan (else null): its header, checked against this call's
   float* partial;       // [shares][pitch]: every workgroup writes its window of its share's image ...
   void* out;            // ... or, with a single share (partial == null), its window of dHW itself:
   int out_dtype;        //     an rz_dtype code,
@@ -84,7 +87,10 @@ __global__ __launch_bounds__(kFoldThreads) void fold_tiles_kernel(const FoldPara
   const int run = E < kFoldRun ? E : kFoldRun, runs = E / run;   // (E is a power of two)
   const int per_tile = p.slices * runs;                          // list entries of a tile
   const int full_lim = (p.h.BK - 1) | (p.h.BN - 1) << 14;
-  for (int q = tid; q < p.window; q += kFoldThreads) img[q] = 0.f;   // (own positions only)
+  // Offsets from a plan that was built for another layer, tile or hash would be in range and
+  // wrong: then the image is NaN and nothing is added (what the output paths below store).
+  const bool plan_ok = p.plan_header == nullptr || layer_plan_matches(p.plan_header, p.K, p.N, p.H, p.h);   // (uniform)
+  for (int q = tid; q < p.window; q += kFoldThreads) img[q] = plan_ok ? 0.f : __builtin_nanf("");   // (own positions only)
 
   // bit j: tile first + i + 1024 j (below `stop`) lands in the window.  The offsets are fetched
   // sixteen at a time, by loads that depend on no condition (one load under a branch per index
@@ -133,9 +139,11 @@ __global__ __launch_bounds__(kFoldThreads) void fold_tiles_kernel(const FoldPara
     return incl;
   };
 
-  // The window's tiles are numbered in a fixed order (pass by pass, thread by thread); the share
-  // takes an equal part of the numbers: the workgroups of a window then have the same work to
-  // within a tile, whatever the hash does.
+  // The window's tiles are numbered in a fixed order that depends on nothing but the table of
+  // offsets: pass by pass of kFoldScan * kFoldThreads tile indices, and inside a pass wavefront by
+  // wavefront, thread by thread, bit by bit of the thread's mask.  A share takes an equal part of
+  // the numbers, so the workgroups of a window have the same work to within a tile whatever the
+  // hash does, and — every share numbering alike — their parts are a partition of the window's tiles.
   int rank_lo = 0, rank_hi = 0x7fffffff;
   if (p.shares > 1) {
     int mine = 0, before;
@@ -144,139 +152,142 @@ __global__ __launch_bounds__(kFoldThreads) void fold_tiles_kernel(const FoldPara
     rank_lo = (int)((long long)share * all / p.shares);
     rank_hi = (int)((long long)(share + 1) * all / p.shares);
   }
-  int lo = 0, seen = 0;                    // tiles [0, lo) hold `seen` tiles of the window
-  int span = kFoldScan * kFoldThreads;
+  const int cap = kFoldList / per_tile;    // tiles whose runs the list holds at a time (at least four)
+  int lo = plan_ok ? 0 : ntiles, seen = 0;   // tiles [0, lo) hold `seen` tiles of the window
   while (lo < ntiles && seen < rank_hi) {   // (uniform: every thread of the workgroup goes round together)
-    if (span > ntiles - lo) span = ntiles - lo;
-    // --- list the share's tiles among [lo, lo + span) ---------------------------------------------
-    unsigned long long mask = scan(lo, lo + span);
-    const int mine = __popcll(mask);
+    const int span = (ntiles - lo) < kFoldScan * kFoldThreads ? (ntiles - lo) : kFoldScan * kFoldThreads;
+    const unsigned long long pass_mask = scan(lo, lo + span);
+    const int mine = __popcll(pass_mask);
     const int incl = wave_scan(mine);
     int before;
     const int found = total_of(incl, &before);
+    const int first_rank = seen + before + incl - mine;   // of this thread's first tile
     const int want_lo = rank_lo > seen ? rank_lo : seen;
     const int want_hi = rank_hi < seen + found ? rank_hi : seen + found;
-    const int total = (want_hi > want_lo ? want_hi - want_lo : 0) * per_tile;
-    if (total > kFoldList) {   // does not fit: look at half the range (a range of kFoldList / per_tile >= 4 tiles always fits)
-      span = (span + 1) / 2;
-      continue;
-    }
-    int rank = seen + before + incl - mine;   // of this thread's first tile
-    while (mask != 0ull) {
-      const int j = __ffsll((long long)mask) - 1;
-      mask &= mask - 1ull;
-      if (rank >= want_lo && rank < want_hi) {
-        const int id = lo + tid + j * kFoldThreads;
-        const int rel = p.offsets[id] - w0;
-        const int tk = id / p.tiles_n, tn = id - tk * p.tiles_n;
-        const int rows = (p.K - tk * p.h.BK) < p.h.BK ? (p.K - tk * p.h.BK) : p.h.BK;
-        const int cols = (p.N - tn * p.h.BN) < p.h.BN ? (p.N - tn * p.h.BN) : p.h.BN;
-        for (int s = 0; s < p.slices; s++)
-          for (int c = 0; c < runs; c++) {
-            const int slot = ((rank - want_lo) * p.slices + s) * runs + c;
-            list_at[slot] = ((s * ntiles + id) << eshift) + c * run;
-            list_rel[slot] = rel + c * run;
-            list_lim[slot] = (rows - 1) | (cols - 1) << 14 | c << 28;
-          }
-      }
-      rank++;
-    }
     seen += found;
-    __syncthreads();
-    // --- add the listed runs into the window ---------------------------------------------------
-    // Every wavefront on its own: lane u holds entry u of a chunk of 64 list entries; the entries
-    // that meet one of the wavefront's blocks are taken in list order, in rounds of kFoldRound;
-    // the next round's loads are in flight while this round's values are added.  What describes
-    // an entry to the wavefront is uniform (scalar registers).
-    struct Round {
-      fold_f4 v[kFoldRound];
-      int pos[kFoldRound];   // window position of the block
-      int e0[kFoldRound];    // float of the run that falls on the block's first position (-255 .. run - 1)
-      int lim[kFoldRound];   // the entry's, -1: no entry
-    };
-    unsigned long long todo = 0ull;   // entries of the chunk that this wavefront still has to add
-    int next = 0;                     // first list entry behind the chunk
-    int c_pos = 0, c_e0 = 0, c_off = 0, c_lim = 0;
-    auto refill = [&]() {
-      while (todo == 0ull && next < total) {   // (uniform)
-        const int t = next + lane;
-        const bool have = t < total;
-        const int rel = have ? list_rel[t] : 0, at = have ? list_at[t] : 0;
-        c_lim = have ? list_lim[t] : 0;
-        const int first = rel >> 8;                    // (arithmetic shift: the block of the run's first float)
-        const int b = first + ((wave - first) & 15);   // the wavefront's only block among the sixteen from there on
-        c_pos = b * kFoldBlock;
-        c_e0 = c_pos - rel;
-        c_off = at + c_e0;
-        todo = __ballot(have && b >= 0 && c_pos < wlen && c_e0 < run);
-        next += 64;
-      }
-    };
-    auto issue = [&](Round& r) {
-#pragma unroll
-      for (int u = 0; u < kFoldRound; u++) {
-        const bool any = todo != 0ull;
-        const int src = any ? (int)__builtin_ctzll(todo) : 0;
-        todo &= todo - 1ull;
-        const int off = __builtin_amdgcn_readlane(c_off, src), lim = __builtin_amdgcn_readlane(c_lim, src);
-        r.pos[u] = __builtin_amdgcn_readlane(c_pos, src);
-        r.e0[u] = __builtin_amdgcn_readlane(c_e0, src);
-        r.lim[u] = any ? lim : -1;
-        // (every slot loads, an empty one the buffer's first floats: with no branch around the
-        //  loads their number is fixed, and the wait for this round's values can leave the next
-        //  round's in flight)
-        const long long first = any ? (long long)off : 0ll;
-        unsigned mine = lane16;   // byte offset of the lane's four floats from the block's first
-        if (any && (r.e0[u] < 0 || r.e0[u] + kFoldBlock > run)) {   // (uniform) an end of the run:
-          // lanes that lie wholly outside the run fetch floats of the run that other lanes fetch
-          // anyway (their values count as zero below) instead of a neighbouring tile's
-          const int e = r.e0[u] + lane4;
-          const int inside = e <= -4 ? 0 : (e >= run ? max(run - 4, r.e0[u]) : e);
-          mine = (unsigned)(inside - r.e0[u]) * 4u;
+    lo += span;
+    // The share's tiles of this pass, `cap` numbers at a time (the numbering does not depend on
+    // how many fit the list, so a share that needs several chunks still takes exactly its part).
+    for (int chunk_lo = want_lo; chunk_lo < want_hi; chunk_lo += cap) {   // (uniform)
+      const int chunk_hi = (chunk_lo + cap) < want_hi ? (chunk_lo + cap) : want_hi;
+      const int total = (chunk_hi - chunk_lo) * per_tile;
+      if (chunk_lo != want_lo) __syncthreads();   // (the wavefronts are done reading the previous chunk's list)
+      unsigned long long mask = pass_mask;
+      int rank = first_rank;
+      while (mask != 0ull) {
+        const int j = __ffsll((long long)mask) - 1;
+        mask &= mask - 1ull;
+        if (rank >= chunk_lo && rank < chunk_hi) {
+          const int id = lo - span + tid + j * kFoldThreads;
+          const int rel = p.offsets[id] - w0;
+          const int tk = id / p.tiles_n, tn = id - tk * p.tiles_n;
+          const int rows = (p.K - tk * p.h.BK) < p.h.BK ? (p.K - tk * p.h.BK) : p.h.BK;
+          const int cols = (p.N - tn * p.h.BN) < p.h.BN ? (p.N - tn * p.h.BN) : p.h.BN;
+          for (int s = 0; s < p.slices; s++)
+            for (int c = 0; c < runs; c++) {
+              const int slot = ((rank - chunk_lo) * p.slices + s) * runs + c;
+              list_at[slot] = ((s * ntiles + id) << eshift) + c * run;
+              list_rel[slot] = rel + c * run;
+              list_lim[slot] = (rows - 1) | (cols - 1) << 14 | c << 28;
+            }
         }
-        // (read once and never again: a load that leaves the caches to the offsets and to the
-        //  contraction's stores still on their way to memory — K = N = 10240: 129 -> 111 us)
-        r.v[u] = __builtin_nontemporal_load(
-            reinterpret_cast<const fold_f4u*>(reinterpret_cast<const char*>(p.tiles) + first * 4 + mine));
+        rank++;
       }
-    };
-    // (plain read-add-write: LDS float atomics are several times slower, and nobody else touches
-    //  this lane's words; runs that overlap are added one after the other, in list order)
-    auto add = [&](const Round& r) {
-#pragma unroll
-      for (int u = 0; u < kFoldRound; u++) {
-        if (r.lim[u] == -1) continue;   // (uniform)
-        fold_f4 v = r.v[u];
-        const int lim = r.lim[u];
-        if (r.e0[u] < 0 || r.e0[u] + kFoldBlock > run || (lim & 0x0fffffff) != full_lim) {
-          // an end of the run, or a tile that sticks out of K x N: what is not the run's counts as zero
-          asm volatile("" ::: "memory");   // (keeps this arithmetic out of the common path)
-          const int rows = (lim & 0x3fff) + 1, cols = ((lim >> 14) & 0x3fff) + 1, base = (lim >> 28) * run;
-#pragma unroll
-          for (int f = 0; f < 4; f++) {
-            const int e = r.e0[u] + lane4 + f, in_tile = base + e;
-            const bool ok = e >= 0 && e < run && (in_tile >> p.h.bn_shift) < rows && (in_tile & (p.h.BN - 1)) < cols;
-            v[f] = ok ? v[f] : 0.f;
+      __syncthreads();
+      // --- add the listed runs into the window ---------------------------------------------------
+      // Every wavefront on its own: lane u holds entry u of a chunk of 64 list entries; the entries
+      // that meet one of the wavefront's blocks are taken in list order, in rounds of kFoldRound;
+      // the next round's loads are in flight while this round's values are added.  What describes
+      // an entry to the wavefront is uniform (scalar registers).
+      struct Round {
+        fold_f4 v[kFoldRound];
+        int pos[kFoldRound];   // window position of the block
+        int e0[kFoldRound];    // float of the run that falls on the block's first position (-255 .. run - 1)
+        int lim[kFoldRound];   // the entry's, -1: no entry
+      };
+      unsigned long long todo = 0ull;   // entries of the chunk that this wavefront still has to add
+      int next = 0;                     // first list entry behind the chunk
+      int c_pos = 0, c_e0 = 0, c_off = 0, c_lim = 0;
+      auto refill = [&]() {
+        while (todo == 0ull && next < total) {   // (uniform)
+          const int t = next + lane;
+          const bool have = t < total;
+          const int rel = have ? list_rel[t] : 0, at = have ? list_at[t] : 0;
+          c_lim = have ? list_lim[t] : 0;
+          const int first = rel >> 8;                    // (arithmetic shift: the block of the run's first float)
+          const int b = first + ((wave - first) & 15);   // the wavefront's only block among the sixteen from there on
+          c_pos = b * kFoldBlock;
+          c_e0 = c_pos - rel;
+          c_off = at + c_e0;
+          todo = __ballot(have && b >= 0 && c_pos < wlen && c_e0 < run);
+          next += 64;
+        }
+      };
+      auto issue = [&](Round& r) {
+  #pragma unroll
+        for (int u = 0; u < kFoldRound; u++) {
+          const bool any = todo != 0ull;
+          const int src = any ? (int)__builtin_ctzll(todo) : 0;
+          todo &= todo - 1ull;
+          const int off = __builtin_amdgcn_readlane(c_off, src), lim = __builtin_amdgcn_readlane(c_lim, src);
+          r.pos[u] = __builtin_amdgcn_readlane(c_pos, src);
+          r.e0[u] = __builtin_amdgcn_readlane(c_e0, src);
+          r.lim[u] = any ? lim : -1;
+          // (every slot loads, an empty one the buffer's first floats: with no branch around the
+          //  loads their number is fixed, and the wait for this round's values can leave the next
+          //  round's in flight)
+          const long long first = any ? (long long)off : 0ll;
+          unsigned mine = lane16;   // byte offset of the lane's four floats from the block's first
+          if (any && (r.e0[u] < 0 || r.e0[u] + kFoldBlock > run)) {   // (uniform) an end of the run:
+            // lanes that lie wholly outside the run fetch floats of the run that other lanes fetch
+            // anyway (their values count as zero below) instead of a neighbouring tile's
+            const int e = r.e0[u] + lane4;
+            const int inside = e <= -4 ? 0 : (e >= run ? max(run - 4, r.e0[u]) : e);
+            mine = (unsigned)(inside - r.e0[u]) * 4u;
           }
+          // (read once and never again: a load that leaves the caches to the offsets and to the
+          //  contraction's stores still on their way to memory — K = N = 10240: 129 -> 111 us)
+          r.v[u] = __builtin_nontemporal_load(
+              reinterpret_cast<const fold_f4u*>(reinterpret_cast<const char*>(p.tiles) + first * 4 + mine));
         }
-        fold_f4* at = reinterpret_cast<fold_f4*>(img + r.pos[u] + lane4);
-        *at = *at + v;
-      }
-    };
-    Round r0, r1;
-    refill();
-    issue(r0);
-    while (true) {   // (uniform per wavefront; no barrier inside)
-      refill();
-      issue(r1);
-      add(r0);
-      if (r1.lim[0] == -1) break;   // (entries fill a round from its first slot)
+      };
+      // (plain read-add-write: LDS float atomics are several times slower, and nobody else touches
+      //  this lane's words; runs that overlap are added one after the other, in list order)
+      auto add = [&](const Round& r) {
+  #pragma unroll
+        for (int u = 0; u < kFoldRound; u++) {
+          if (r.lim[u] == -1) continue;   // (uniform)
+          fold_f4 v = r.v[u];
+          const int lim = r.lim[u];
+          if (r.e0[u] < 0 || r.e0[u] + kFoldBlock > run || (lim & 0x0fffffff) != full_lim) {
+            // an end of the run, or a tile that sticks out of K x N: what is not the run's counts as zero
+            asm volatile("" ::: "memory");   // (keeps this arithmetic out of the common path)
+            const int rows = (lim & 0x3fff) + 1, cols = ((lim >> 14) & 0x3fff) + 1, base = (lim >> 28) * run;
+  #pragma unroll
+            for (int f = 0; f < 4; f++) {
+              const int e = r.e0[u] + lane4 + f, in_tile = base + e;
+              const bool ok = e >= 0 && e < run && (in_tile >> p.h.bn_shift) < rows && (in_tile & (p.h.BN - 1)) < cols;
+              v[f] = ok ? v[f] : 0.f;
+            }
+          }
+          fold_f4* at = reinterpret_cast<fold_f4*>(img + r.pos[u] + lane4);
+          *at = *at + v;
+        }
+      };
+      Round r0, r1;
       refill();
       issue(r0);
-      add(r1);
-      if (r0.lim[0] == -1) break;
+      while (true) {   // (uniform per wavefront; no barrier inside)
+        refill();
+        issue(r1);
+        add(r0);
+        if (r1.lim[0] == -1) break;   // (entries fill a round from its first slot)
+        refill();
+        issue(r0);
+        add(r1);
+        if (r0.lim[0] == -1) break;
+      }
     }
-    lo += span;
   }
   // --- the window of this share's image ---------------------------------------------------------
   __syncthreads();   // (the words below were added up by other threads)
@@ -294,6 +305,128 @@ __global__ __launch_bounds__(kFoldThreads) void fold_tiles_kernel(const FoldPara
     f16_t* out = reinterpret_cast<f16_t*>(p.out) + w0;
     for (int q = tid; q < wlen; q += kFoldThreads)
       out[q] = ElemTraits<f16_t>::from_float(img[q] + (p.accumulate ? ElemTraits<f16_t>::to_float(out[q]) : 0.f));
+  }
+}
+
+// ---- the same sum for a layer of few tiles ------------------------------------------------------
+// With a few thousand tiles at most, every workgroup can afford to look at every tile offset, and
+// the machinery above (windows in LDS, shares, run lists walked by wavefronts) costs more than it
+// saves: a 1024 x 1024 layer has 256 tiles and a hashed_weight of 65536 elements, and its whole
+// gradient is a few microseconds of reading.  Here a workgroup of 256 threads owns 256 * PER
+// consecutive elements of dHW, thread t the elements t, t + 256, ...; it lists the tiles whose
+// slice meets its elements (ascending tile index: one ballot and two barriers per 1024 tiles) and
+// every thread then walks down the list and adds what each tile holds for its elements — loads of
+// 256 consecutive floats per wavefront-row, fixed order of additions (tile by tile, slice by slice),
+// no atomics, every element of dHW written once.
+static constexpr int kFoldSmallThreads = 256;
+static constexpr int kFoldSmallTiles = 4096;   // tiles at most: the list in LDS can hold every one of them
+
+template <int PER>
+__global__ __launch_bounds__(kFoldSmallThreads) void fold_small_kernel(const FoldParams p) {
+  __shared__ int list_id[kFoldSmallTiles];     // tiles that meet this workgroup's elements, ascending
+  __shared__ int list_rel[kFoldSmallTiles];    // ... and where each starts, relative to the first element
+  __shared__ int wave_count[kFoldSmallThreads / 64];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  constexpr int kSpan = kFoldSmallThreads * PER;
+  const int h0 = blockIdx.x * kSpan;
+  const int span = (p.H - h0) < kSpan ? (p.H - h0) : kSpan;
+  const int E = p.h.BK * p.h.BN, eshift = p.h.bk_shift + p.h.bn_shift;
+  const int ntiles = p.tiles_k * p.tiles_n;
+  const bool plan_ok = p.plan_header == nullptr || layer_plan_matches(p.plan_header, p.K, p.N, p.H, p.h);   // (uniform)
+  int listed = 0;
+  for (int first = 0; first < ntiles && plan_ok; first += 4 * kFoldSmallThreads) {
+    // thread t looks at the tiles first + 4 t .. first + 4 t + 3 (ascending over the threads)
+    int rel[4];
+    unsigned hit = 0u;
+#pragma unroll
+    for (int u = 0; u < 4; u++) {
+      const int id = first + 4 * tid + u;
+      const int idc = id < ntiles ? id : ntiles - 1;
+      // (without a table, the few offsets a thread needs are hashed on the spot)
+      rel[u] = (p.offsets != nullptr ? p.offsets[idc] : (int)tile_offset(p.h, (uint32_t)(idc / p.tiles_n), (uint32_t)(idc % p.tiles_n))) - h0;
+      hit |= (unsigned)((id < ntiles) & (rel[u] > -E) & (rel[u] < span)) << u;
+    }
+    const int mine = __popc(hit);
+    int incl = mine;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const int up = __shfl_up(incl, d, 64);
+      if (lane >= d) incl += up;
+    }
+    __syncthreads();   // (the counts of the previous round have been read)
+    if (lane == 63) wave_count[wave] = incl;
+    __syncthreads();
+    int at = listed + incl - mine;
+    for (int w = 0; w < kFoldSmallThreads / 64; w++) {
+      const int c = wave_count[w];
+      if (w < wave) at += c;
+      listed += c;
+    }
+#pragma unroll
+    for (int u = 0; u < 4; u++)
+      if ((hit >> u) & 1u) {
+        list_id[at] = first + 4 * tid + u;
+        list_rel[at] = rel[u];
+        at++;
+      }
+  }
+  __syncthreads();
+  float acc[PER];
+#pragma unroll
+  for (int j = 0; j < PER; j++) acc[j] = plan_ok ? 0.f : __builtin_nanf("");
+  // The list is taken 32 / PER tiles at a time: all loads of a batch are issued before the first value is
+  // used (a load per tile under its own branch would wait out one memory latency after the other: 17
+  // tiles took 10 us that way), and the values are added in list order.  A thread that a tile does not
+  // reach loads the tile buffer's first float instead and adds zero.
+  constexpr int kBatch = 32 / PER;
+  for (int e0 = 0; e0 < listed; e0 += kBatch) {   // (uniform)
+    unsigned off[kBatch][PER];
+    bool ok[kBatch][PER];
+#pragma unroll
+    for (int u = 0; u < kBatch; u++) {
+      const int e = e0 + u < listed ? e0 + u : listed - 1;
+      const int id = list_id[e], rel = list_rel[e];
+      const int tk = id / p.tiles_n, tn = id - tk * p.tiles_n;
+      // rows and columns of the tile inside K x N (what lies beyond was never written)
+      const int rows = (p.K - tk * p.h.BK) < p.h.BK ? (p.K - tk * p.h.BK) : p.h.BK;
+      const int cols = (p.N - tn * p.h.BN) < p.h.BN ? (p.N - tn * p.h.BN) : p.h.BN;
+      const bool whole = rows == p.h.BK && cols == p.h.BN;
+#pragma unroll
+      for (int j = 0; j < PER; j++) {
+        const int x = tid + j * kFoldSmallThreads - rel;   // element of the tile that lands on this thread's j-th element
+        ok[u][j] = e0 + u < listed && x >= 0 && x < E && tid + j * kFoldSmallThreads < span &&
+                   (whole || ((x >> p.h.bn_shift) < rows && (x & (p.h.BN - 1)) < cols));
+        off[u][j] = ok[u][j] ? ((unsigned)id << eshift) + (unsigned)x : 0u;
+      }
+    }
+    for (int sl = 0; sl < p.slices; sl++) {
+      const float* base = p.tiles + (((size_t)sl * ntiles) << eshift);
+      float v[kBatch][PER];
+#pragma unroll
+      for (int u = 0; u < kBatch; u++)
+#pragma unroll
+        for (int j = 0; j < PER; j++) v[u][j] = base[off[u][j]];
+#pragma unroll
+      for (int u = 0; u < kBatch; u++)
+#pragma unroll
+        for (int j = 0; j < PER; j++) acc[j] += ok[u][j] ? v[u][j] : 0.f;
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < PER; j++) {
+    const int pos = tid + j * kFoldSmallThreads;
+    if (pos >= span) continue;
+    const int q = h0 + pos;
+    if (p.out_dtype == RZ_F32) {
+      float* out = reinterpret_cast<float*>(p.out);
+      out[q] = acc[j] + (p.accumulate ? out[q] : 0.f);
+    } else if (p.out_dtype == RZ_BF16) {
+      bf16_t* out = reinterpret_cast<bf16_t*>(p.out);
+      out[q] = ElemTraits<bf16_t>::from_float(acc[j] + (p.accumulate ? ElemTraits<bf16_t>::to_float(out[q]) : 0.f));
+    } else {
+      f16_t* out = reinterpret_cast<f16_t*>(p.out);
+      out[q] = ElemTraits<f16_t>::from_float(acc[j] + (p.accumulate ? ElemTraits<f16_t>::to_float(out[q]) : 0.f));
+    }
   }
 }
 

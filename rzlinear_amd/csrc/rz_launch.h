@@ -19,7 +19,7 @@ static inline bool tuning_valid(const rz_tuning& t) {
   return (t.tile == 0 || t.tile == 32 || t.tile == 64 || t.tile == 128 || t.tile == 256) && (t.stages == 0 || t.stages == 1) &&
          (t.lds_image == 0 || t.lds_image == -1) && (t.window >= -1 && t.window <= 1) &&
          (t.split == 0 || t.split == -1) && (t.clamp == 0 || t.clamp == -1) &&
-         (t.fold >= -1 && t.fold <= 1) && t.reserved == 0;
+         (t.fold >= -1 && t.fold <= 2) && t.poll_limit >= 0;
 }
 
 // Kernels that use more than the default 64 KB of LDS need their limit raised once per kernel
@@ -132,6 +132,7 @@ static constexpr size_t kFoldMarginBytes = 2048;
 
 struct FoldPlan {
   int use;
+  int small;             // few tiles: the kernel whose workgroups each look at every tile (no windows in LDS, no shares)
   int window, windows;   // floats per window (a multiple of 1024, at most 32768) and their number
   int shares;            // workgroups per window, each with an equal part of the window's tiles and an image of its own
   size_t tiles_bytes;    // the tile-by-tile X^T.dY: slices * tiles * BK*BN floats, with a margin before and after
@@ -139,13 +140,28 @@ struct FoldPlan {
   size_t offsets_bytes;  // where every tile starts in hashed_weight, one int32 per tile
 };
 
-static inline FoldPlan plan_fold(int K, int N, int H, int BK, int BN, int slices) {
+static inline FoldPlan plan_fold(int K, int N, int H, int BK, int BN, int slices, bool windowed = false) {
   FoldPlan f = {};
   const long long E = (long long)BK * BN;
   const long long tiles = (long long)((K + BK - 1) / BK) * ((N + BN - 1) / BN);
   // (element indices of the buffer are 32-bit in the kernels; the fold lists slices entries per tile)
   if (E > 16384 || slices > 64 || (long long)slices * tiles * E >= (1LL << 31)) return f;
   const int kWindowMax = 32768, kThreads = 1024;
+  // (few tiles over a hashed_weight of up to 2^18 elements: measured 5 to 8 us; with a larger one every
+  //  workgroup would still look at every tile for the handful that reach it, and the windowed kernel or
+  //  the window kernel do better — K = 2048, N = 4096, H = 2^20: 20 us against the window kernel's 25 in all)
+  if (tiles <= 4096 && H <= (1 << 18) && !windowed) {
+    // every workgroup of 256 threads owns 256 elements of dHW
+    f.small = 1;
+    f.window = 256;
+    f.windows = (H + f.window - 1) / f.window;
+    f.shares = 1;
+    f.tiles_bytes = (((size_t)slices * tiles * E * sizeof(float) + 255) & ~(size_t)255) + 2 * kFoldMarginBytes;
+    f.partial_bytes = 0;
+    f.offsets_bytes = ((size_t)tiles * sizeof(int32_t) + 255) & ~(size_t)255;
+    f.use = 1;
+    return f;
+  }
   f.windows = (H + kWindowMax - 1) / kWindowMax;
   // from half a window per compute unit on, the windows are cut so that whole rounds of workgroups
   // come out, and every workgroup writes its window of dHW itself (no shares, no images)
@@ -325,7 +341,7 @@ static inline WeightGradPlan plan_weight_grad(int M, int K, int N, int H, int BK
   pl.fold = FoldPlan{};
   pl.fold_us = 0.0;
   if (!image && t.fold != -1) {
-    const FoldPlan f = plan_fold(K, N, H, BK, BN, pl.splits);
+    const FoldPlan f = plan_fold(K, N, H, BK, BN, pl.splits, t.fold == 2);
     if (f.use) {
       // what the two ways cost beyond the contraction itself, in microseconds: the part of the
       // K*N global atomics per slice that the contraction does not hide (2.8 to 5.2 ps each,
@@ -342,8 +358,12 @@ static inline WeightGradPlan plan_weight_grad(int M, int K, int N, int H, int BK
       const double read_bytes = elems * 4.0 * (1.0 + (double)BK * BN / f.window);
       const double all_us = (read_bytes + 2.0 * (double)f.partial_bytes) / 4.5e6;
       const double one_us = read_bytes / ((double)f.windows * f.shares) / 15e3;
-      const double fold_us = (store_us > product_us ? store_us - product_us : 0.0) + (all_us > one_us ? all_us : one_us) + 10.0;
-      if (t.fold == 1 || fold_us < atomics_us) {
+      // (few tiles: every element is read once, by a kernel of a few microseconds; it is taken even where
+      //  the atomics would be a little faster — K = N = 1024: 5 us against 3 us on top of the contraction —
+      //  because it adds in a fixed order: the same bits on every call)
+      const double fold_us = f.small ? (store_us > product_us ? store_us - product_us : 0.0) + elems * 4.0 / 4.5e6 + 5.0
+                                     : (store_us > product_us ? store_us - product_us : 0.0) + (all_us > one_us ? all_us : one_us) + 10.0;
+      if (t.fold >= 1 || f.small || fold_us < atomics_us) {
         pl.fold = f;
         // (for the comparison with the window kernel: every round of workgroups of the contraction
         //  kernel also pays its fill, drain and store — about 5 us for a round of 256 tiles, 10 us
@@ -428,7 +448,7 @@ static inline WindowPlan plan_window(int M, int K, int N, int H, int BK, int BN,
 // K, N, H, the tile and the hash constants, not on M, the element type or the data), computed once
 // on the host and kept by the caller in device memory.  int32 words:
 //   [0, 16)   header: magic, version, K, N, H, BK, BN, hash_levels, tiles, windows, window,
-//             entries, strips per tile, 0, 0, 0
+//             entries, strips per tile, checksum of the hash constants (layer_plan_hash_sum), 0, 0
 //   offsets   [tiles]           where every W tile starts in hashed_weight (index tk * tiles_n + tn)
 //   start     [windows + 1]     first entry of every window of the window kernel (window_geometry)
 //   list      [capacity]        the strips (tile * strips per tile + strip) that meet the window, ascending
@@ -436,6 +456,19 @@ static inline WindowPlan plan_window(int M, int K, int N, int H, int BK, int BN,
 // The lists exist for the tiles the window kernel supports (windows = 0 otherwise).
 static constexpr int32_t kLayerPlanMagic = 0x525a4c50, kLayerPlanVersion = 1;
 static constexpr int kLayerPlanHeader = 16;
+// What a plan's header says of the hash constants that its offsets were computed with (the kernels
+// that read a plan compare it with their own call's constants).
+__host__ __device__ static inline int32_t layer_plan_hash_sum(const HashParams& h) {
+  uint32_t s = 2166136261u;
+  const uint32_t v[8] = {h.R0, h.R1, h.R2, h.R3, h.R4, h.R5, h.R7, (uint32_t)h.levels};
+  for (int i = 0; i < 8; i++) s = (s ^ v[i]) * 16777619u;
+  return (int32_t)(s & 0x7fffffffu);
+}
+// header words 2..7 and 13 against a call (K, N, H, BK, BN, hash_levels, constants)
+__host__ __device__ static inline bool layer_plan_matches(const int32_t* hd, int K, int N, int H, const HashParams& h) {
+  return hd[0] == kLayerPlanMagic && hd[2] == K && hd[3] == N && hd[4] == H && hd[5] == h.BK && hd[6] == h.BN &&
+         hd[7] == h.levels && hd[13] == layer_plan_hash_sum(h);
+}
 struct LayerPlanLayout {
   bool ok;
   int tiles, windows, window, strips_per_tile, strip_elems;

@@ -24,6 +24,7 @@
 #include <type_traits>
 
 #include "rz_gemm.h"
+#include "rz_launch.h"
 
 namespace rz {
 
@@ -38,7 +39,7 @@ struct WindowParams {
   const int32_t* plan_start;
   const int32_t* plan_list;
   const int32_t* plan_offs;
-  const int32_t* plan_header;   // K, N, H, BK, BN, window at words 2..6 and 10: checked against this call's
+  const int32_t* plan_header;   // shapes, tile, hash (words 2..7, 13) and window (10): checked against this call's
   int M, K, N, H;
   int64_t ldx, lddy;
   float scale;
@@ -47,7 +48,13 @@ struct WindowParams {
   int tiles_k, tiles_n;
   int accumulate;    // dHW += gradient instead of dHW = gradient
   int out_f32;       // dHW is fp32 whatever T is
+  int poll_limit;    // looks at the flags of earlier strips before a wavefront gives up (kWindowPollLimit)
 };
+
+// How often a wavefront looks at the flags of the earlier strips it must wait for before it gives
+// up.  A look takes at least 64 clocks (the sleep between two), so the limit is some seconds —
+// far beyond any real wait (a strip's product takes microseconds) and still an end.
+static constexpr int kWindowPollLimit = 1 << 24;
 
 // TBK x TBN is the hashed tile (compile time).  The unit of work is a strip of 32 rows of a tile
 // (its slice of hashed_weight is the 32 * TBN elements from off + 32 * TBN * strip on): a
@@ -88,6 +95,7 @@ struct WindowKernel {
     int offs[kList];              // ... their offsets in hashed_weight
     int done[kList];              // ... and whether they have been added to the window
     int count[2][kWaves];
+    int spoilt;                   // a wavefront gave up waiting for an earlier strip: the window is stored as NaN
     alignas(16) T stage[kWaves][kStageElems];
     alignas(16) float window[4];  // the image of dHW[w0, w0 + window) starts here, then 64
                                   // dump slots
@@ -145,6 +153,7 @@ struct WindowKernel {
       const float4 z = {0.f, 0.f, 0.f, 0.f};
       *reinterpret_cast<float4*>(win + i) = z;
     }
+    if (tid == 0) sm.spoilt = 0;   // (read after the barriers of the rounds below)
 
     const int total = p.tiles_k * p.tiles_n;
     const int ngroups = (p.M + kGroupRows - 1) / kGroupRows;
@@ -189,7 +198,7 @@ struct WindowKernel {
       // A plan built for another layer would send the loads below anywhere: refuse it, loudly
       // (the window of dHW becomes NaN), instead of reading outside X and dY.
       const int32_t* hd = p.plan_header;
-      if (hd[2] != p.K || hd[3] != p.N || hd[4] != p.H || hd[5] != TBK || hd[6] != TBN || hd[10] != p.window ||
+      if (!layer_plan_matches(hd, p.K, p.N, p.H, p.h) || hd[5] != TBK || hd[6] != TBN || hd[10] != p.window ||
           hd[12] != kStrips) {
         const float nan = __builtin_nanf("");
         if (p.out_f32 || sizeof(T) == 4) {
@@ -394,8 +403,12 @@ struct WindowKernel {
       // slices meet its own, and raise its flag
       auto add_tile = [&](int e) {
         const int tile_off = __builtin_amdgcn_readfirstlane(sm.offs[e]);
-        // lane l looks at the earlier entries l, l + 64, ...: straight-line LDS reads, no branches
-        for (;;) {
+        // lane l looks at the earlier entries l, l + 64, ...: straight-line LDS reads, no branches.
+        // The wait is bounded: an entry only waits for earlier ones, whose owners wait for still
+        // earlier ones, so it ends by itself; should a flag never come all the same (a list that
+        // is not what this kernel expects), the wavefront gives up after kPollLimit looks, marks
+        // the window as spoilt and goes on, so that every wavefront reaches the end of the kernel.
+        for (int polls = 0;; polls++) {
           bool pending = false;
           for (int f = lane; f < e; f += 64) {
             const int d = sm.offs[f] - tile_off;
@@ -403,6 +416,10 @@ struct WindowKernel {
             pending |= (d < kStripElems) & (d > -kStripElems) & (dn == 0);
           }
           if (!__any(pending)) break;
+          if (polls >= p.poll_limit) {   // (uniform)
+            if (lane == 0) __hip_atomic_store(&sm.spoilt, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            break;
+          }
           __builtin_amdgcn_s_sleep(1);
         }
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
@@ -589,6 +606,12 @@ struct WindowKernel {
     }
 
     // store the window: dHW[w0 + i] (+)= image[i], each element exactly once
+    __syncthreads();   // (a window that no strip meets has passed no barrier since it was cleared)
+    if (sm.spoilt) {   // (uniform) the order of the adds was not kept: say so in the result
+      const float nan = __builtin_nanf("");
+      for (int i = tid; i < wlen; i += kThreads) win[i] = nan;
+      __syncthreads();
+    }
     if (p.out_f32 || sizeof(T) == 4) {
       float* out = static_cast<float*>(p.dHW) + w0;
       for (int i = tid; i < wlen; i += kThreads) out[i] = win[i] + (p.accumulate ? out[i] : 0.f);

@@ -73,7 +73,7 @@ def weight_grad_hashed(input, output_grad, init_factor, M, K, N, H, R, BLOCK_SIZ
     if use_layer_plan is None:
         use_layer_plan = _lib.use_layer_plans
     if use_layer_plan and _lib.plan_query(2, M, K, N, H, BLOCK_SIZE_K, BLOCK_SIZE_N, code, flags,
-                                          with_bias_grad)["mode"] in ("window", "fold"):
+                                          with_bias_grad, planned=True)["mode"] in ("window", "fold"):
         plan = _lib.layer_plan(K, N, H, BLOCK_SIZE_K, BLOCK_SIZE_N, R, hash_levels, output_grad.device)
     if plan is not None:
         _lib.check(lib.rz_weight_grad_planned(

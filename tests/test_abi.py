@@ -98,7 +98,7 @@ def test_status_codes(lib):
     assert lib.rz_forward(one, one, one, 8, 128, 128, 65536, 64, 64, _R(R1024), 1.0, 64, 128, 0, None) == -2
     assert lib.rz_input_grad(one, one, one, 8, 128, 128, 4096, 64, 64, _R(R1024), 1.0, 128, 128, 0, None) == -4
     assert lib.rz_weight_grad(one, one, one, None, 0, 8, 128, 128, 65536, 64, 64, _R(R1024), 1.0, 128, 128, 1,
-                              None) == -7                         # bf16 needs the fp32 workspace
+                              None) == -7                         # a hashed_weight beyond LDS needs a workspace
     assert lib.rz_materialize(one, one, 128, 128, 65536, 64, 64, _R(R1024), 2, 64, 0, None) == -2
     # a skinny problem splits its contraction and then needs the workspace
     need = lib.rz_forward_workspace_bytes(32, 10240, 1024, 65536, 64, 64, 0)
@@ -108,12 +108,18 @@ def test_status_codes(lib):
                              10240, 1024, 0, None) == -7
     assert lib.rz_input_grad_ws(one, one, one, None, 0, 32, 1024, 10240, 65536, 64, 64, _R(R1024), 1.0,
                                 10240, 1024, 0, None) == -7
-    assert lib.rz_weight_grad_workspace_bytes(8, 128, 128, 65536, 64, 64, 0) == 0
-    assert lib.rz_weight_grad_workspace_bytes(8, 128, 128, 65536, 64, 64, 1) == 65536 * 4
+    # a hashed_weight too large for LDS and few tiles: X^T.dY tile by tile (4 tiles of 16 KB between two margins
+    # of 2 KB) and the table of tile offsets; with the fold switched off, the atomic scatter: nothing for an
+    # fp32 gradient, its fp32 image for a 16-bit one
+    from rzlinear_amd import _lib
+    for code in (0, 1):
+        assert lib.rz_weight_grad_workspace_bytes(8, 128, 128, 65536, 64, 64, code) == 4 * 16384 + 2 * 2048 + 256
+    no_fold = _lib.Tuning(fold=-1)
+    assert lib.rz_weight_grad_hashed_workspace_bytes(8, 128, 128, 65536, 64, 64, 0, 0, 0, ctypes.byref(no_fold)) == 0
+    assert lib.rz_weight_grad_hashed_workspace_bytes(8, 128, 128, 65536, 64, 64, 1, 0, 0, ctypes.byref(no_fold)) == 65536 * 4
     assert lib.rz_forward_hashed(one, one, None, one, None, 0, 8, 128, 128, 65536, 64, 64, _R(R1024), 5, 1.0,
                                  128, 128, 0, None, None) == -9
     # tuning overrides are validated
-    from rzlinear_amd import _lib
     bad = _lib.Tuning(tile=96)
     assert lib.rz_forward_hashed(one, one, None, one, None, 0, 8, 128, 128, 65536, 64, 64, _R(R1024), 2, 1.0,
                                  128, 128, 0, ctypes.byref(bad), None) == -9

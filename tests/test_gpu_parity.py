@@ -122,7 +122,7 @@ TILE_CASES = [
     # (M, K, N, H, BK, BN): complete tiles for every C-tile size, ragged, and both scatter paths
     (512, 512, 512, 9000, 64, 64),
     (300, 200, 330, 9000, 32, 64),
-    (256, 256, 512, 70000, 64, 64),      # H too large for the LDS image: global atomics
+    (256, 256, 512, 70000, 64, 64),      # H too large for the LDS image: tiles stored and folded (fold = -1: global atomics)
     (130, 70, 90, 2000, 16, 16),         # 16-wide tiles: LDS atomics inside the image
     (2688, 192, 2432, 30000, 64, 64),    # > 384 tiles of 128: the four-wavefront 128 form
 ]
@@ -130,7 +130,7 @@ TILE_CASES = [
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=lambda d: str(d).split(".")[-1])
 @pytest.mark.parametrize("env", [{"tile": 32}, {"tile": 64}, {"tile": 128}, {"tile": 256}, {"tile": 128, "stages": 1},
-                                 {"tile": 256, "lds_image": -1}],
+                                 {"tile": 256, "lds_image": -1}, {"lds_image": -1, "fold": -1, "window": -1}],
                          ids=lambda e: "-".join("%s=%s" % (k, v) for k, v in e.items()))
 @pytest.mark.parametrize("shape", TILE_CASES, ids=lambda s: "x".join(map(str, s)))
 def test_every_tile_shape_and_scatter_mode(oracle, shape, env, dtype):

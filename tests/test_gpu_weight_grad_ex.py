@@ -17,12 +17,13 @@ R1024 = SEED_CONSTANTS[1024]
 CASES = [
     (512, 512, 512, 9000, 64, 64),       # complete tiles, LDS image
     (300, 200, 330, 9000, 32, 64),       # ragged
-    (256, 256, 512, 70000, 64, 64),      # H too large for the LDS image: global atomics
+    (256, 256, 512, 70000, 64, 64),      # H too large for the LDS image: tiles stored and folded (fold = -1: global atomics)
     (130, 70, 90, 2000, 16, 16),         # 16-wide tiles
     (4100, 192, 160, 30000, 64, 64),     # long M: the reduction is cut into slices
     (40, 1500, 140, 9000, 64, 64),       # more tile rows than R steps: some workgroups never sum
 ]
-ENVS = [{}, {"tile": 64}, {"tile": 128}, {"tile": 256}, {"tile": 128, "stages": 1}, {"lds_image": -1}]   # rz_tuning overrides
+ENVS = [{}, {"tile": 64}, {"tile": 128}, {"tile": 256}, {"tile": 128, "stages": 1}, {"lds_image": -1},
+        {"lds_image": -1, "fold": -1}]   # rz_tuning overrides
 _env_id = lambda e: "-".join("%s=%s" % (k, v) for k, v in e.items()) or "auto"
 _dt_id = lambda d: str(d).split(".")[-1]
 _shape_id = lambda s: "x".join(map(str, s))
@@ -55,7 +56,7 @@ def test_bias_grad_from_the_weight_grad_pass(oracle, shape, env, dtype):
 
 @pytest.mark.parametrize("out_dtype", ["same", "f32"])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=_dt_id)
-@pytest.mark.parametrize("env", [{}, {"lds_image": -1}], ids=_env_id)
+@pytest.mark.parametrize("env", [{}, {"lds_image": -1}, {"lds_image": -1, "fold": -1}], ids=_env_id)
 @pytest.mark.parametrize("shape", CASES[:4], ids=_shape_id)
 def test_accumulate_into_an_existing_gradient(oracle, tuned, shape, env, dtype, out_dtype):
     from rzlinear_amd.impl.RzLinearBackward import (rz_linear_backward_weight_bias_grad_tl,
@@ -141,8 +142,9 @@ FOLD_CASES = [
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16], ids=_dt_id)
+@pytest.mark.parametrize("kernel", [1, 2], ids=["auto", "windowed"])
 @pytest.mark.parametrize("shape", FOLD_CASES, ids=_shape_id)
-def test_tiles_stored_plainly_and_folded_into_the_gradient(oracle, tuned, shape, dtype):
+def test_tiles_stored_plainly_and_folded_into_the_gradient(oracle, tuned, shape, kernel, dtype):
     """hashed_weight too large for an LDS image: the contraction kernel stores X^T.dY tile by tile
     and scatters nothing; the fold kernel's workgroups own windows of hashed_weight and add up the
     tiles that land there.  No atomics, a fixed order of additions: the same bits on every call.
@@ -151,7 +153,9 @@ def test_tiles_stored_plainly_and_folded_into_the_gradient(oracle, tuned, shape,
     from rzlinear_amd.impl.RzLinearBackward import (rz_linear_backward_weight_bias_grad_tl,
                                                     rz_linear_backward_weight_grad_tl)
     M, K, N, H, BK, BN, tile = shape
-    tuned(fold=1, window=-1, lds_image=-1, tile=tile)
+    # (fold = 1 leaves layers of at most 4096 tiles to the kernel for few tiles, fold = 2 sends them through
+    #  the windowed kernel as well)
+    tuned(fold=kernel, window=-1, lds_image=-1, tile=tile)
     code = _lib.dtype_code(torch.empty(0, dtype=dtype))
     plan = _lib.plan_query(2, M, K, N, H, BK, BN, code)
     _say("fold", shape, dtype, plan)
@@ -179,3 +183,82 @@ def test_tiles_stored_plainly_and_folded_into_the_gradient(oracle, tuned, shape,
     c = rz_linear_backward_weight_grad_tl(x, dy, 0.5, M, K, N, H, *rargs(R1024), **kw)
     torch.cuda.synchronize()
     assert rel_err(f(c), ref) <= TOL[dtype]
+
+
+def test_fold_shares_take_a_partition_of_a_window_even_when_their_lists_overflow(oracle):
+    """768 x 768 hashed tiles of 16 x 16 over a hashed_weight of 500 000: sixteen windows, sixteen
+    workgroups to a window, and every one of them has more tiles (about 2 400) than its list holds
+    (2 048 runs), so each works through its part in several chunks.  The parts must still be a
+    partition of the window's tiles: a tile taken twice or dropped shows as an error of the size of
+    the gradient itself.  Reference as in test_gpu_full_size.py (index map checked against the
+    oracle, float64 product and index_add_ on the GPU)."""
+    from rzlinear_amd import _lib
+    from rzlinear_amd.impl.RzLinearBackward import rz_linear_backward_weight_grad_tl
+    from rzlinear_amd.impl.RzLinearIdx import rz_linear_weight_tl
+    M, K, N, H, BK, BN = 32, 12288, 12288, 500000, 16, 16
+    dtype = torch.bfloat16
+    code = _lib.dtype_code(torch.empty(0, dtype=dtype))
+    plan = _lib.plan_query(2, M, K, N, H, BK, BN, code, planned=True)
+    _say("fold, lists that overflow", plan)
+    assert plan["mode"] == "fold" and plan["shares"] > 1
+    tiles_per_share = (K // BK) * (N // BN) * (H / plan["windows"] + BK * BN) / H / plan["shares"]
+    assert tiles_per_share * plan["slices"] > 2048          # more than a list holds
+    g = torch.Generator().manual_seed(91)
+    x = torch.randn((M, K), generator=g).to(dtype).cuda()
+    dy = torch.randn((M, N), generator=g).to(dtype).cuda()
+    kw = dict(BLOCK_SIZE_K=BK, BLOCK_SIZE_N=BN)
+    idx = rz_linear_weight_tl(torch.arange(H, dtype=torch.float32, device="cuda"), K, N, H, *rargs(R1024), **kw).long()
+    assert np.array_equal(idx.cpu().numpy(), oracle.index_map(K, N, H, BK, BN, R1024))
+    a = rz_linear_backward_weight_grad_tl(x, dy, 1.0, M, K, N, H, *rargs(R1024), **kw)
+    b = rz_linear_backward_weight_grad_tl(x, dy, 1.0, M, K, N, H, *rargs(R1024), **kw)
+    torch.cuda.synchronize()
+    dW = x.double().t() @ dy.double()
+    ref = torch.zeros((H,), dtype=torch.float64, device="cuda").index_add_(0, idx.reshape(-1), dW.reshape(-1))
+    err = float((a.double() - ref).abs().max() / ref.abs().max())
+    assert err <= TOL[dtype], err
+    assert abs(float(a.double().sum() - dW.sum())) <= TOL[dtype] * float(dW.abs().sum()) / 10   # every tile exactly once
+    assert torch.equal(a, b)
+
+
+SMALL_LAYERS = [
+    # (M, K, N, H, BK, BN): a hashed_weight beyond an LDS image, at most 4096 tiles
+    (1024, 1024, 1024, 65536, 64, 64),     # the reference's CPU-runnable configuration
+    (128, 1024, 1024, 65536, 32, 64),      # its benchmark grid at K = N = 1024, the launchers' default tile
+    (300, 200, 330, 250000, 32, 64),       # ragged; a thousand workgroups, most of them with no tile at all
+    (4100, 192, 160, 50000, 64, 64),       # M in slices
+    (77, 520, 264, 40000, 128, 128),       # tiles that reach beyond K x N
+    (64, 4096, 4096, 1 << 18, 64, 64),     # 4096 tiles over 2^18 elements: the most this kernel takes
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=_dt_id)
+@pytest.mark.parametrize("shape", SMALL_LAYERS, ids=_shape_id)
+def test_small_layers_with_a_large_hashed_weight_are_folded_without_atomics(oracle, shape, dtype):
+    """No tuning: a layer of few tiles whose hashed_weight does not fit an LDS image stores X^T.dY tile
+    by tile and a second, small kernel adds the tiles up in a fixed order — the same bits on every call,
+    where the atomic scatter it replaces left the order of the additions open.  With a layer plan's
+    offsets and with the kernel's own hashing; accumulating; against the oracle."""
+    from rzlinear_amd import _lib
+    from rzlinear_amd.impl.RzLinearBackward import rz_linear_backward_weight_grad_tl, weight_grad_hashed
+    M, K, N, H, BK, BN = shape
+    code = _lib.dtype_code(torch.empty(0, dtype=dtype))
+    plan = _lib.plan_query(2, M, K, N, H, BK, BN, code)
+    _say("small fold", shape, dtype, plan)
+    assert plan["mode"] == "fold" and plan["shares"] == 1
+    (x, _, dy), (x64, _, dy64) = make_inputs(M, K, N, H, dtype, seed=68)
+    kw = dict(BLOCK_SIZE_K=BK, BLOCK_SIZE_N=BN)
+    ref = oracle.weight_grad(x64, dy64, H, BK, BN, R1024, 0.5)
+    a = rz_linear_backward_weight_grad_tl(x, dy, 0.5, M, K, N, H, *rargs(R1024), **kw)
+    b = rz_linear_backward_weight_grad_tl(x, dy, 0.5, M, K, N, H, *rargs(R1024), **kw)
+    R = _lib.hash_constants(*rargs(R1024))
+    c, _ = weight_grad_hashed(x, dy, 0.5, M, K, N, H, R, BK, BN, use_layer_plan=False)
+    torch.cuda.synchronize()
+    f = lambda t: t.float().cpu().numpy()
+    assert rel_err(f(a), ref) <= TOL[dtype]
+    assert (f(a)[ref == 0] == 0).all()
+    assert torch.equal(a, b) and torch.equal(a, c)
+    start = torch.linspace(-1, 1, H).cuda()
+    buf = start.clone()
+    rz_linear_backward_weight_grad_tl(x, dy, 0.5, M, K, N, H, *rargs(R1024), out=buf, accumulate=True, **kw)
+    torch.cuda.synchronize()
+    assert rel_err(buf.cpu().numpy(), start.double().cpu().numpy() + ref) <= TOL[dtype]

@@ -173,6 +173,65 @@ def test_a_plan_of_another_layer_is_refused_on_the_device(tuned):
     assert torch.isnan(out).all()
 
 
+@pytest.mark.parametrize("mode", ["window", "fold"])
+def test_a_plan_built_with_other_hash_constants_is_refused_on_the_device(tuned, mode):
+    """Same K, N, H and tile, other constants: every offset of the plan is in range and wrong.  The
+    header carries a checksum of the constants; the window kernel and the fold kernel compare it
+    with their call's and store NaN instead of a wrong gradient."""
+    from rzlinear_amd import _lib
+    tuned(window=1) if mode == "window" else tuned(fold=1, window=-1)
+    M, K, N, H, BK, BN = 32, 512, 512, 300000, 64, 64
+    _say("layer plan of other constants", mode)
+    (x, _, dy), _ = make_inputs(M, K, N, H, torch.float32, seed=42)
+    lib = _lib.load()
+    R = _lib.hash_constants(*rargs(R1024))
+    other = _lib.hash_constants(*rargs(SEED_CONSTANTS[0]))
+    assert _lib.plan_query(2, M, K, N, H, BK, BN, _lib.RZ_F32, planned=True)["mode"] == mode
+    need = lib.rz_weight_grad_hashed_workspace_bytes(M, K, N, H, BK, BN, _lib.RZ_F32, 0, 0, _lib.current_tuning())
+    ws = torch.empty((max(need, 16),), dtype=torch.uint8, device=x.device)
+    out = {}
+    for name, consts in (("own", R), ("other", other)):
+        plan = _lib.layer_plan(K, N, H, BK, BN, consts, 2, x.device)
+        out[name] = torch.zeros((H,), device=x.device)
+        _lib.check(lib.rz_weight_grad_planned(x.data_ptr(), dy.data_ptr(), out[name].data_ptr(), None, ws.data_ptr(), need,
+                                              plan.data_ptr(), plan.numel() * 4, M, K, N, H, BK, BN, R, 2, 1.0, K, N,
+                                              _lib.RZ_F32, 0, _lib.current_tuning(), torch.cuda.current_stream().cuda_stream))
+    torch.cuda.synchronize()
+    assert torch.isfinite(out["own"]).all() and float(out["own"].abs().max()) > 0
+    assert torch.isnan(out["other"]).all()
+
+
+def test_a_wavefront_that_gives_up_waiting_spoils_its_window_and_leaves(oracle, tuned):
+    """The wait for earlier strips is bounded.  With the bound set to one look (from the host, through
+    rz_tuning) wavefronts give up where they would have waited: the kernel still ends, and every
+    window of dHW is either exactly what the unbounded run gives or NaN throughout."""
+    from rzlinear_amd import _lib
+    from rzlinear_amd.impl.RzLinearBackward import rz_linear_backward_weight_grad_tl
+    M, K, N, H, BK, BN = 64, 1024, 1024, 200000, 64, 64
+    _say("bounded wait of the window kernel")
+    (x, _, dy), (x64, _, dy64) = make_inputs(M, K, N, H, torch.bfloat16, seed=44)
+    code = _lib.dtype_code(x)
+    tuned(window=1)
+    q = _lib.plan_query(2, M, K, N, H, BK, BN, code, planned=True)
+    assert q["mode"] == "window"
+    good = rz_linear_backward_weight_grad_tl(x, dy, 1.0, M, K, N, H, *rargs(R1024), BLOCK_SIZE_K=BK, BLOCK_SIZE_N=BN)
+    tuned(window=1, poll_limit=1)
+    hasty = rz_linear_backward_weight_grad_tl(x, dy, 1.0, M, K, N, H, *rargs(R1024), BLOCK_SIZE_K=BK, BLOCK_SIZE_N=BN)
+    torch.cuda.synchronize()
+    assert rel_err(good.float().cpu().numpy(), oracle.weight_grad(x64, dy64, H, BK, BN, R1024, 1.0)) <= TOL[torch.bfloat16]
+    window = -(-H // q["windows"])
+    window = (window + 3) // 4 * 4
+    spoilt = 0
+    for w0 in range(0, H, window):
+        a, b = hasty[w0:w0 + window], good[w0:w0 + window]
+        if torch.isnan(a).any():
+            assert torch.isnan(a).all()
+            spoilt += 1
+        else:
+            assert torch.equal(a, b)
+    _say("  windows stored as NaN: %d of %d" % (spoilt, q["windows"]))
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=_dt_id)
 def test_fold_path_takes_its_tile_offsets_from_the_plan(oracle, tuned, monkeypatch, dtype):
     from rzlinear_amd import _lib

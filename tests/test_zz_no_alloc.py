@@ -48,8 +48,9 @@ def _both(lib, shape, dtype, seed, oracle):
 # (first problem, smaller second problem, how the plan carries the first one out in bf16)
 PAIRS = [
     ((768, 512, 640, 9000, 64, 64), (200, 256, 192, 5000, 64, 64), "lds_image"),
-    ((512, 384, 512, 70000, 64, 64), (96, 128, 192, 40000, 32, 64), "atomics"),
-    ((32, 2048, 4096, 1 << 20, 64, 64), (16, 2048, 4096, 1 << 20, 64, 64), "window"),
+    ((512, 384, 512, 70000, 64, 64), (96, 128, 192, 40000, 32, 64), "fold"),
+    ((512, 512, 768, 200000, 256, 256), (96, 256, 256, 100000, 256, 128), "atomics"),   # tiles too large to fold
+    ((32, 4096, 8192, 1 << 21, 64, 64), (16, 4096, 8192, 1 << 21, 64, 64), "window"),
 ]
 
 
@@ -108,3 +109,22 @@ def test_static_scratch_refuses_what_does_not_fit():
     # argument errors come back as from rz_weight_grad
     assert lib.rz_weight_grad_static(None, one, one, 64, 64, 64, 5000, 64, 64, R, 1.0, 64, 64, 0, None) == -1
     assert lib.rz_weight_grad_static(one, one, one, 64, 64, 64, 4096, 64, 64, R, 1.0, 64, 64, 0, None) == -4
+
+
+def test_static_scratch_is_that_of_the_device_that_holds_the_gradient():
+    """The scratch array used is the current device's; a dHW that is not memory of that device (here:
+    host memory) would make the kernels work in another address space, and is refused."""
+    from rzlinear_amd import _lib
+    lib = _lib.load()
+    M, K, N, H = 64, 64, 64, 5000
+    x = torch.zeros((M, K), device="cuda")
+    dy = torch.zeros((M, N), device="cuda")
+    host = torch.zeros((H,))
+    R = (ctypes.c_int32 * 8)(*R1024)
+    st = lib.rz_weight_grad_static(x.data_ptr(), dy.data_ptr(), host.data_ptr(), M, K, N, H, 64, 64, R, 1.0, K, N,
+                                   _lib.RZ_F32, torch.cuda.current_stream().cuda_stream)
+    assert st == -9
+    dev = torch.zeros((H,), device="cuda")
+    _lib.check(lib.rz_weight_grad_static(x.data_ptr(), dy.data_ptr(), dev.data_ptr(), M, K, N, H, 64, 64, R, 1.0, K, N,
+                                         _lib.RZ_F32, torch.cuda.current_stream().cuda_stream))
+    torch.cuda.synchronize()
