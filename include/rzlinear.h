@@ -38,7 +38,7 @@ extern "C" {
 typedef enum rz_status {
   RZ_OK = 0,
   RZ_ERR_NULL_POINTER = -1,
-  RZ_ERR_BAD_SHAPE = -2,       /* M, K, N < 1, ld too small, sizes beyond int32 tiling */
+  RZ_ERR_BAD_SHAPE = -2,       /* M, K, N < 1, ld too small (or 256 rows of it beyond 4 GB), sizes beyond int32 tiling */
   RZ_ERR_BAD_TILE = -3,        /* BK/BN not a power of two in [16,256] */
   RZ_ERR_HASH_RANGE = -4,      /* H <= BK*BN  (reference: assert H > BLOCK_SIZE_K*BLOCK_SIZE_N) */
   RZ_ERR_BAD_DTYPE = -5,

@@ -234,22 +234,6 @@ def rows(t):
     return t, ld
 
 
-def whole_pieces(t, cols):
-    """rows(t) for an operand whose `cols` columns are contracted (or, for the weight gradient, tiled)
-    16 bytes at a time.  The 16-bit kernels stage an operand straight into LDS only if its rows
-    are whole 16-byte pieces; K or N that is not a multiple of 8 sends them through the
-    bounds-checked kernels instead (bf16 4096^3 with K = 4095: forward 224 us instead of 117,
-    weight-grad 427 instead of 123).  A large operand is therefore copied once into rows padded
-    with zeros up to the next multiple of 8 — zeros add nothing to any of the three products (as
-    long as the other operand is finite there: 0 * inf is not 0) — and the call is made with the
-    padded extent, which names the same hashed tiles.  Returns (tensor, row pitch, extent)."""
-    t, ld = rows(t)
-    if t.element_size() == 2 and cols % 8 and t.shape[0] * cols >= (1 << 20):
-        t = torch.nn.functional.pad(t, (0, 8 - cols % 8))
-        return t, t.stride(0), t.shape[1]
-    return t, ld, cols
-
-
 def workspace(nbytes, device):
     """A scratch buffer of nbytes on `device` (None when nbytes is 0)."""
     return torch.empty((nbytes,), device=device, dtype=torch.uint8) if nbytes else None
@@ -272,13 +256,25 @@ _layer_plans = {}
 use_layer_plans = True
 
 
+def clear_layer_plans():
+    """Forget every layer plan built so far (they are kept per layer geometry and device until this
+    is called; a process that goes through many geometries can release them here)."""
+    _layer_plans.clear()
+
+
 def layer_plan(K, N, H, BK, BN, R, hash_levels, device):
     """The layer plan (rz_layer_plan_build) for these layer constants as an int32 tensor on `device`,
-    built on the host the first time it is asked for and kept for the life of the process (it depends
-    on the layer alone: shapes, tile and hash constants; about 10 bytes per W tile strip)."""
+    built on the host the first time it is asked for and kept until clear_layer_plans() (it depends
+    on the layer alone: shapes, tile and hash constants; about 10 bytes per W tile strip).  The
+    first request copies the plan to the device with an ordinary, synchronous copy: make it outside
+    a stream capture (one warm-up call of the layer, or this function itself, does)."""
     key = (K, N, H, BK, BN, tuple(int(v) for v in R), int(hash_levels), str(device))
     plan = _layer_plans.get(key)
     if plan is None:
+        if torch.cuda.is_current_stream_capturing():
+            raise RuntimeError("rzlinear_amd: the layer plan for K=%d N=%d H=%d tile %dx%d has to be built (a host-to-device "
+                               "copy) but the current stream is being captured; call the layer once, or "
+                               "_lib.layer_plan(...), before the capture" % (K, N, H, BK, BN))
         lib = load()
         nbytes = lib.rz_layer_plan_bytes(K, N, H, BK, BN)
         if nbytes == 0:

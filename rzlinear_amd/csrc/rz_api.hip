@@ -64,6 +64,10 @@ static int make_hash(HashParams* h, int K, int N, int H, int BK, int BN, const i
   return RZ_OK;
 }
 
+// Row pitches are limited so that a tile's rows stay within the 32-bit byte offsets of the kernels'
+// load addresses (256 rows of 2^23 four-byte elements are 2^33 bytes: the limit is per element type below).
+static bool pitch_ok(int64_t ld, int elem_bytes) { return ld > 0 && ld * elem_bytes * 256 < (1LL << 32); }
+
 static int dtype_bytes(int dtype) {
   switch (dtype) {
     case RZ_F32: return 4;
@@ -368,6 +372,7 @@ static int weight_grad_impl(const void* X, const void* dY, void* dHW, void* dbia
   if (X == nullptr || dY == nullptr || dHW == nullptr) return RZ_ERR_NULL_POINTER;
   if (dtype_bytes(dtype) == 0) return RZ_ERR_BAD_DTYPE;
   if (M < 1 || ldx < K || lddy < N) return RZ_ERR_BAD_SHAPE;
+  if (!pitch_ok(ldx, dtype_bytes(dtype)) || !pitch_ok(lddy, dtype_bytes(dtype))) return RZ_ERR_BAD_SHAPE;
   if (flags & ~(unsigned)(RZ_WG_ACCUMULATE | RZ_WG_DHW_F32 | RZ_WG_DBIAS_F32)) return RZ_ERR_BAD_ARGUMENT;
   const rz_tuning tuning = tuning_or_default(tuning_arg);
   if (!tuning_valid(tuning)) return RZ_ERR_BAD_ARGUMENT;
@@ -611,7 +616,7 @@ static int forward_impl(const void* X, const void* HW, const void* bias, void* Y
                         void* stream, int hash_levels = RZ_HASH_TWO_LEVEL, const rz_tuning* tuning_arg = nullptr) {
   if (X == nullptr || HW == nullptr || Y == nullptr) return RZ_ERR_NULL_POINTER;
   if (dtype_bytes(dtype) == 0) return RZ_ERR_BAD_DTYPE;
-  if (M < 1 || ldx < K || ldy < N) return RZ_ERR_BAD_SHAPE;
+  if (M < 1 || ldx < K || ldy < N || !pitch_ok(ldx, dtype_bytes(dtype)) || !pitch_ok(ldy, dtype_bytes(dtype))) return RZ_ERR_BAD_SHAPE;
   const rz_tuning tuning = tuning_or_default(tuning_arg);
   if (!tuning_valid(tuning)) return RZ_ERR_BAD_ARGUMENT;
   GemmParams p = {};
@@ -635,7 +640,7 @@ static int input_grad_impl(const void* dY, const void* HW, void* dX, void* works
                            int hash_levels = RZ_HASH_TWO_LEVEL, const rz_tuning* tuning_arg = nullptr) {
   if (dY == nullptr || HW == nullptr || dX == nullptr) return RZ_ERR_NULL_POINTER;
   if (dtype_bytes(dtype) == 0) return RZ_ERR_BAD_DTYPE;
-  if (M < 1 || lddy < N || lddx < K) return RZ_ERR_BAD_SHAPE;
+  if (M < 1 || lddy < N || lddx < K || !pitch_ok(lddy, dtype_bytes(dtype)) || !pitch_ok(lddx, dtype_bytes(dtype))) return RZ_ERR_BAD_SHAPE;
   const rz_tuning tuning = tuning_or_default(tuning_arg);
   if (!tuning_valid(tuning)) return RZ_ERR_BAD_ARGUMENT;
   GemmParams p = {};
@@ -836,7 +841,7 @@ RZ_API int rz_layer_plan_build(void* plan_host, size_t plan_bytes, int K, int N,
     auto for_each_pair = [&](auto&& f) {
       for (int id = 0; id < l.tiles; id++)
         for (int sidx = 0; sidx < l.strips_per_tile; sidx++) {
-          const long long so = (long long)offsets[id] + (long long)sidx * l.strip_elems;
+          const long long so = (long long)offsets[id] + window_unit_start(BN, sidx);
           const long long first = so / l.window, last = (so + l.strip_elems - 1) / l.window;
           for (long long b = first; b <= last && b < l.windows; b++) f((int)b, id * l.strips_per_tile + sidx, (int32_t)so);
         }

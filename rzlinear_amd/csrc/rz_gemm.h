@@ -115,13 +115,28 @@ __device__ __forceinline__ u32x4_t mask_tail(u32x4_t v, int col, int col_lim) {
   return v;
 }
 
+// The 16-bit elements sh .. 7 of a 16-byte piece moved down to positions 0 .. 7 - sh, zeros above (1 <= sh <= 7).
+__device__ __forceinline__ u32x4_t shift_down_16(u32x4_t v, int sh) {
+  const uint64_t lo = (uint64_t)v[0] | (uint64_t)v[1] << 32, hi = (uint64_t)v[2] | (uint64_t)v[3] << 32;
+  const int bits = sh * 16;
+  const uint64_t olo = bits >= 64 ? hi >> (bits - 64) : (lo >> bits) | (hi << (64 - bits));
+  const uint64_t ohi = bits >= 64 ? 0ull : hi >> bits;
+  u32x4_t r = {(uint32_t)olo, (uint32_t)(olo >> 32), (uint32_t)ohi, (uint32_t)(ohi >> 32)};
+  return r;
+}
+
 // COLSUM (weight-grad only): also sum the columns of B (dY) for the bias gradient.
 // CLAMP (with FULL = false): ragged shapes.  The last R step may be partial (its excess is
-// cleared in LDS; where R is contiguous in an operand it must be a multiple of the 16-byte
-// piece) and the C tile grid may have ragged edges.  Tiles are then still staged directly: a piece that
+// cleared in LDS) and the C tile grid may have ragged edges.  Tiles are then still staged directly: a piece that
 // would start outside the operand is fetched from the nearest row / piece inside it (hashed
 // pieces need nothing: every tile index hashes to a valid slice).  What such a piece holds
 // only reaches rows or columns of C that the bounds-checked epilogue never stores.
+// Rows of a plain operand need not be whole 16-byte pieces either (any K, N >= 8): the piece that
+// straddles the end of a row is fetched as it lies, reaching into the next row — except in the
+// operand's LAST row, where that would read beyond the operand: there the piece is fetched so that
+// it ends with the row, and one thread puts it right in LDS afterwards (a second, guarded load,
+// shifted into place).  Where R is the contiguous dimension the excess elements of the straddling
+// piece are cleared in LDS in every row, like the pieces wholly beyond R.
 // WK (forward / input-grad): WK groups of WI x WJ wavefronts share a C tile; group g multiplies
 // the g-th part of every R step and the groups' accumulators are added through LDS at the end.
 // For a tile with one wavefront per SIMD (fp32, 64 x 64) this puts a second wavefront on every
@@ -327,6 +342,13 @@ struct GemmKernel {
     u32x4_t ra[LA::kPieces], rb[LB::kPieces];
     // elements of the last R step that lie beyond R (ragged contraction, direct staging)
     const int tail = CLAMP ? steps * TR - (r_end - r_begin) : 0;
+    // elements of the piece that straddles the end of an operand's rows (0: rows are whole pieces):
+    // along R in forward / input-grad, along I (X) and J (dY) in weight-grad
+    const int rag_r = (CLAMP && OP != kWeightGrad) ? (p.R & (VEC - 1)) : 0;
+    const int rag_i = (CLAMP && OP == kWeightGrad) ? (p.I & (VEC - 1)) : 0;
+    const int rag_j = (CLAMP && OP == kWeightGrad) ? (p.J & (VEC - 1)) : 0;
+    // the step that holds the operands' last row is issued piece by piece and put right in LDS
+    const bool slow_last = CLAMP && (tail > 0 || ((rag_i | rag_j) != 0 && r_end == p.R));
 
     // Bias gradient (COLSUM): the tiles_i workgroups of one tile column and slice stage the same
     // rows of dY, so they take turns: the workgroup whose turn it is adds the rows of that R
@@ -536,9 +558,15 @@ struct GemmKernel {
         // (CLAMP forward / input-grad: pieces of the last, partial R step beyond R come from the
         //  last piece inside and are cleared in LDS as well)
         const int gc = r0 + col;
-        const int cc = (CLAMP && gc >= p.R) ? p.R - VEC : gc;
+        int cc = (CLAMP && gc >= p.R) ? p.R - VEC : gc;
+        int ca = ci;
+        if constexpr (CLAMP) {
+          // the piece that straddles the end of the operand's last row ends with the row (see clear_tail)
+          if (A_LAYOUT == kRContig && rag_r && ci == p.I - 1 && gc < p.R && gc + VEC > p.R) cc = p.R - VEC;
+          if (A_LAYOUT == kRStrided && rag_i && cr == p.R - 1 && gi < p.I && gi + VEC > p.I) ca = p.I - VEC;
+        }
         const T* src = (A_LAYOUT == kRContig) ? gA + (int64_t)ci * p.lda + cc
-                                              : gA + (int64_t)cr * p.lda + ci;
+                                              : gA + (int64_t)cr * p.lda + ca;
         direct_load(src, sm.a[st], q, LA::kPieces);
       }
       if constexpr (OP == kWeightGrad) {
@@ -547,9 +575,10 @@ struct GemmKernel {
           int row, col;
           direct_src(LB{}, B_LAYOUT, q, row, col);
           const int gj = j0 + col;
-          const int cj = (!CLAMP || gj < p.J) ? gj : p.J - VEC;
+          int cj = (!CLAMP || gj < p.J) ? gj : p.J - VEC;
           const int gr = r0 + row;
           const int cr = (CLAMP && gr >= p.R) ? p.R - 1 : gr;
+          if (CLAMP && rag_j && cr == p.R - 1 && gj < p.J && gj + VEC > p.J) cj = p.J - VEC;
           direct_load(gB + (int64_t)cr * p.ldb + cj, sm.b[st], q, LB::kPieces);
         }
       }
@@ -576,7 +605,9 @@ struct GemmKernel {
           a_voff[q] = (uint32_t)(((int64_t)ci * p.lda + col) * (int64_t)sizeof(T));
         } else {
           const int gi = i0 + col;
-          const int ci = (!CLAMP || gi < p.I) ? col : p.I - VEC - i0;
+          // (an offset is unsigned: a tile with fewer than VEC columns inside I has no whole piece of its
+          //  own to repeat and repeats its first, straddling one)
+          const int ci = (!CLAMP || gi < p.I) ? col : (p.I - VEC - i0 > 0 ? p.I - VEC - i0 : 0);
           a_voff[q] = (uint32_t)(((int64_t)row * p.lda + ci) * (int64_t)sizeof(T));
         }
       }
@@ -586,7 +617,7 @@ struct GemmKernel {
         direct_src(LB{}, B_LAYOUT, q, row, col);
         if constexpr (OP == kWeightGrad) {
           const int gj = j0 + col;
-          const int cj = (!CLAMP || gj < p.J) ? col : p.J - VEC - j0;
+          const int cj = (!CLAMP || gj < p.J) ? col : (p.J - VEC - j0 > 0 ? p.J - VEC - j0 : 0);
           b_voff[q] = (uint32_t)(((int64_t)row * p.ldb + cj) * (int64_t)sizeof(T));
           b_tab[q] = 0;
         } else {
@@ -614,7 +645,7 @@ struct GemmKernel {
     // all tiles of R step `step` -> LDS stage `st`
     auto direct_issue = [&](int step, int st) {
       const int r0 = r_begin + step * TR;
-      if (CLAMP && tail > 0 && step == steps - 1) {   // (uniform) the partial last step
+      if (CLAMP && slow_last && step == steps - 1) {   // (uniform) the partial last step, or the one with the operands' last row
         direct_issue_plain_slow(step, st);
       } else {
         // first element of the A tile of this step (uniform)
@@ -638,32 +669,58 @@ struct GemmKernel {
           direct_load_so(hw_base, off[q] * (uint32_t)sizeof(T) + b_voff[q], sm.b[st], q, LB::kPieces);
       }
     };
-    // CLAMP, last R step with fewer than TR elements of R: once every wavefront's loads of that
-    // step have landed (the caller has just passed a barrier), the part of both stages beyond R
-    // — fetched from inside the operands, or from tiles beyond the tile grid — is set to zero:
-    // whole rows where X is contiguous, the trailing 16-byte pieces of every row where R is
-    // (R is then a multiple of the piece width).  A second barrier makes that visible.  Happens
-    // at most once per workgroup.
+    // CLAMP, last R step: once every wavefront's loads of that step have landed (the caller has just
+    // passed a barrier), the part of both stages beyond R — fetched from inside the operands, or
+    // from tiles beyond the tile grid — is set to zero: whole rows where X is contiguous; where R is,
+    // the trailing 16-byte pieces of every row and the excess elements of a piece that straddles R.
+    // The straddling piece of an operand's last row (fetched so that it ends with the row, lest the
+    // load reach beyond the operand) is fetched again here, through registers, and shifted into
+    // place.  A second barrier makes all that visible.  Happens at most once per workgroup.
     auto clear_tail = [&](int st) {
       if constexpr (CLAMP) {
-        if (tail > 0) {
+        if (slow_last) {
           const u32x4_t z = {0u, 0u, 0u, 0u};
-          auto clear = [&](auto L, int layout, T* stage) {
+          // `plain`: the operand's rows lie in memory as they are (not hashed); g, ld: the operand;
+          // x0, ext: the tile's first index and the operand's extent along X
+          auto clear = [&](auto L, int layout, T* stage, bool plain, const T* g, int64_t ld, int x0, int ext, int rag_x) {
             typedef decltype(L) LL;
             if (layout == kRStrided) {
               const int first = TR - tail;
               for (int i = tid; i < tail * (LL::kPitch / VEC); i += kThreads)
                 *reinterpret_cast<u32x4_t*>(stage + first * LL::kPitch + i * VEC) = z;
+              // the operand's last row (the last one before `first`), the piece that straddles its end
+              const int c = ext - rag_x - x0;
+              if (plain && rag_x && r_end == p.R && c >= 0 && c < LL::kPitch && tid == 0) {
+                const int row = first - 1;
+                u32x4_t v;
+                __builtin_memcpy(&v, g + (int64_t)(p.R - 1) * ld + (ext - VEC), 16);
+                *reinterpret_cast<u32x4_t*>(stage + row * LL::kPitch + ((((c >> 5) ^ (row & 3)) << 5) | (c & 31))) =
+                    shift_down_16(v, VEC - rag_x);
+              }
             } else {
               const int pieces = tail / VEC, first = TR / VEC - pieces;
               for (int i = tid; i < LL::kRows * pieces; i += kThreads) {
                 const int row = i / pieces, pz = first + i % pieces;
                 *reinterpret_cast<u32x4_t*>(stage + row * LL::kPitch + ((pz ^ row_swizzle(row)) << 3)) = z;
               }
+              if (rag_r) {
+                const int pz = first - 1;   // the piece that straddles R
+                for (int row = tid; row < LL::kRows; row += kThreads) {
+                  u32x4_t* at = reinterpret_cast<u32x4_t*>(stage + row * LL::kPitch + ((pz ^ row_swizzle(row)) << 3));
+                  u32x4_t v;
+                  if (plain && x0 + row >= ext - 1) {   // the operand's last row, and the rows beyond that repeat it
+                    __builtin_memcpy(&v, g + (int64_t)(ext - 1) * ld + (p.R - VEC), 16);
+                    v = shift_down_16(v, VEC - rag_r);
+                  } else {
+                    v = mask_tail<T>(*at, 0, rag_r);
+                  }
+                  *at = v;
+                }
+              }
             }
           };
-          clear(LA{}, A_LAYOUT, sm.a[st]);
-          clear(LB{}, B_LAYOUT, sm.b[st]);
+          clear(LA{}, A_LAYOUT, sm.a[st], true, gA, p.lda, i0, p.I, rag_i);
+          clear(LB{}, B_LAYOUT, sm.b[st], OP == kWeightGrad, gB, p.ldb, j0, p.J, rag_j);
           __syncthreads();
         }
       }

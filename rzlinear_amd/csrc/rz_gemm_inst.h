@@ -141,13 +141,14 @@ static hipError_t launch_gemm_t(int op, GemmParams p, const WeightGradPlan* plan
   }
 }
 
-template <typename T, int TBK, int TBN, bool STAGED>
+template <typename T, int TBN, bool STAGED>
 static hipError_t launch_window_form(const WindowParams& p, int windows, hipStream_t stream) {
-  typedef WindowKernel<T, TBK, TBN, STAGED> K;
+  typedef WindowKernel<T, TBN, STAGED> K;
   static_assert(K::kFixedBytes + sizeof(float) * kWindowFloats <= 160 * 1024, "window does not fit the LDS");
   if (p.window < 4 || p.window > kWindowFloats || (p.window & 3) || windows < 1) return hipErrorInvalidValue;
   if ((long long)windows * p.window < p.H) return hipErrorInvalidValue;
-  auto kernel = rz_window_kernel<T, TBK, TBN, STAGED>;
+  if (p.h.BN != TBN || !window_tile_supported(p.h.BK, p.h.BN)) return hipErrorInvalidValue;
+  auto kernel = rz_window_kernel<T, TBN, STAGED>;
   const size_t smem = K::kFixedBytes + sizeof(float) * (size_t)p.window;
   static std::atomic<uint64_t> lds_limit_raised{0};
   if (smem > 64 * 1024) {
@@ -159,19 +160,20 @@ static hipError_t launch_window_form(const WindowParams& p, int windows, hipStre
 }
 
 // Operands whose rows hold whole 16-byte pieces go through the staged form.
-template <typename T, int TBK, int TBN>
+template <typename T, int TBN>
 static hipError_t launch_window_one(const WindowParams& p, int windows, hipStream_t stream) {
   constexpr int kVec = 16 / (int)sizeof(T);
   // (the staged form keeps a lane's piece offsets, up to sixteen rows, in 32-bit registers)
   if (p.K % kVec == 0 && p.N % kVec == 0 && p.ldx < (1 << 26) && p.lddy < (1 << 26))
-    return launch_window_form<T, TBK, TBN, true>(p, windows, stream);
-  return launch_window_form<T, TBK, TBN, false>(p, windows, stream);
+    return launch_window_form<T, TBN, true>(p, windows, stream);
+  return launch_window_form<T, TBN, false>(p, windows, stream);
 }
 
 template <typename T>
 static hipError_t launch_window_t(const WindowParams& p, int windows, hipStream_t stream) {
-  if (p.h.BK == 64 && p.h.BN == 64) return launch_window_one<T, 64, 64>(p, windows, stream);
-  if (p.h.BK == 32 && p.h.BN == 64) return launch_window_one<T, 32, 64>(p, windows, stream);
+  if (p.h.BN == 64) return launch_window_one<T, 64>(p, windows, stream);
+  if (p.h.BN == 32) return launch_window_one<T, 32>(p, windows, stream);
+  if (p.h.BN == 128) return launch_window_one<T, 128>(p, windows, stream);
   return hipErrorInvalidValue;
 }
 

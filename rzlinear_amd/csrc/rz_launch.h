@@ -395,7 +395,19 @@ struct WindowPlan {
 };
 static constexpr int kWindowFloats = 25600;   // LDS floats a workgroup can hold next to its staging
 
-static inline bool window_tile_supported(int BK, int BN) { return BN == 64 && (BK == 64 || BK == 32); }
+// Hashed tiles that the window kernel serves: 32 to 256 rows, 32 to 128 columns.  Its unit of work is 32
+// rows by min(BN, 64) columns of a tile; a tile has window_units of them, unit u = strip * parts + part
+// starting at off + window_unit_start and spanning window_unit_span elements of hashed_weight.
+static inline bool window_tile_supported(int BK, int BN) {
+  return (BN == 32 || BN == 64 || BN == 128) && (BK == 32 || BK == 64 || BK == 128 || BK == 256);
+}
+static inline int window_unit_cols(int BN) { return BN < 64 ? BN : 64; }
+static inline int window_units(int BK, int BN) { return (BK / 32) * (BN / window_unit_cols(BN)); }
+static inline int window_unit_span(int BN) { return 31 * BN + window_unit_cols(BN); }
+static inline long long window_unit_start(int BN, int u) {
+  const int parts = BN / window_unit_cols(BN);
+  return (long long)(u / parts) * (32 * BN) + (long long)(u % parts) * window_unit_cols(BN);
+}
 
 // Size and number of the windows for a hashed_weight of H elements (a function of H alone: a
 // layer plan built once per layer holds the strip lists of exactly these windows).
@@ -427,10 +439,15 @@ static inline WindowPlan plan_window(int M, int K, int N, int H, int BK, int BN,
   // operands of every tile come out of L2 again: tiles that share a window share no rows or
   // columns of W; a wavefront has three groups of rows in flight, which is what its registers hold).
   const double chunks = (double)((M + 31) / 32);
-  // (in units of 64-row tiles, i.e. of two strips: the figures below were fitted on those)
-  const double per_wg = (double)tiles * ((double)w + (double)BK * BN) / (double)H * ((double)BK / 64.0);
+  // (in units of 64 x 64 tiles, i.e. of two strips of 64 columns: the figures below were fitted on those;
+  //  32-column tiles take the time of 64-column ones — their units are half empty)
+  const double per_wg = (double)tiles * ((double)w + (double)BK * BN) / (double)H * ((double)BK / 64.0) * (BN > 64 ? BN / 64.0 : 1.0);
   const double wg_rounds = (double)((pl.windows + kComputeUnits - 1) / kComputeUnits);
-  double t_window = wg_rounds * per_wg * ((elem_bytes == 4 ? 0.43 + 0.63 * chunks : 0.31 + 0.18 * chunks)) + (planned ? 5.0 : 28.0);
+  // (rows of X or dY that are not whole 16-byte pieces are fetched element by element: about 2.2 times the
+  //  time per tile — M = 256, K = 10239, N = 10240, bf16: 411 us against 190 us with K = 10240)
+  const int vec = 16 / elem_bytes;
+  const double by_elements = (K % vec == 0 && N % vec == 0) ? 1.0 : 2.2;
+  double t_window = wg_rounds * per_wg * by_elements * ((elem_bytes == 4 ? 0.43 + 0.63 * chunks : 0.31 + 0.18 * chunks)) + (planned ? 5.0 : 28.0);
   // Every element of dHW receives K*N / H tiles, and the adds into one place of a window go in a
   // fixed order, one after the other: with many tiles per element that chain is what takes the
   // time, about 1.7 us a link (K = 2048, N = 8192, H = 200000: 84 links, 158 us at M = 32 — folded
@@ -451,7 +468,8 @@ static inline WindowPlan plan_window(int M, int K, int N, int H, int BK, int BN,
 //             entries, strips per tile, checksum of the hash constants (layer_plan_hash_sum), 0, 0
 //   offsets   [tiles]           where every W tile starts in hashed_weight (index tk * tiles_n + tn)
 //   start     [windows + 1]     first entry of every window of the window kernel (window_geometry)
-//   list      [capacity]        the strips (tile * strips per tile + strip) that meet the window, ascending
+//   list      [capacity]        the units of work (tile * units per tile + unit: 32 rows by up to 64 columns of
+//                               a tile, see window_units) that meet the window, ascending
 //   offs      [capacity]        ... and where each starts in hashed_weight
 // The lists exist for the tiles the window kernel supports (windows = 0 otherwise).
 static constexpr int32_t kLayerPlanMagic = 0x525a4c50, kLayerPlanVersion = 1;
@@ -471,7 +489,7 @@ __host__ __device__ static inline bool layer_plan_matches(const int32_t* hd, int
 }
 struct LayerPlanLayout {
   bool ok;
-  int tiles, windows, window, strips_per_tile, strip_elems;
+  int tiles, windows, window, strips_per_tile, strip_elems;   // (units per tile, elements a unit spans)
   long long capacity;                 // list entries reserved (an upper bound of those used)
   size_t offsets_at, start_at, list_at, offs_at, words;
 };
@@ -485,9 +503,9 @@ static inline LayerPlanLayout layer_plan_layout(int K, int N, int H, int BK, int
   l.start_at = round16(l.offsets_at + (size_t)tiles);
   if (window_tile_supported(BK, BN) && tiles <= (1 << 20)) {
     window_geometry(H, &l.window, &l.windows);
-    l.strips_per_tile = BK / 32;
-    l.strip_elems = 32 * BN;
-    // a strip of strip_elems consecutive elements meets at most ceil(strip_elems / window) + 1 windows
+    l.strips_per_tile = window_units(BK, BN);
+    l.strip_elems = window_unit_span(BN);
+    // a unit that spans strip_elems consecutive elements meets at most ceil(strip_elems / window) + 1 windows
     l.capacity = tiles * l.strips_per_tile * ((l.strip_elems + l.window - 1) / l.window + 1);
   }
   l.list_at = round16(l.start_at + (size_t)l.windows + 1);
@@ -582,11 +600,10 @@ static inline KernelForm kernel_form(int op, int I, int J, int R, int chunk, int
   const int step_plain = 128 / elem_bytes;
   const int step_direct = (direct_capable && tile == 128 && f.waves == 8) ? 256 / elem_bytes : step_plain;
   f.full = (I % tile == 0) && (J % tile_cols(tile) == 0) && (R % step_direct == 0) && (chunk % step_direct == 0);
-  // a plain operand's 16-byte pieces must not straddle the end of its rows: forward / input-grad
-  // need R, weight-grad needs I and J, to be multiples of the piece
+  // a plain operand's rows must hold at least one 16-byte piece (a piece that straddles the end of a
+  // row is handled in the kernel; a row shorter than a piece is not)
   const int vec = 16 / elem_bytes;
-  const bool pieces_ok = op == kWeightGrad ? (I % vec == 0 && J % vec == 0 && I >= vec && J >= vec)
-                                           : (R % vec == 0 && R >= vec);
+  const bool pieces_ok = op == kWeightGrad ? (I >= vec && J >= vec) : R >= vec;
   f.clamp = !f.full && direct_capable && pieces_ok && t.clamp != -1;
   f.step = (f.full || f.clamp) ? step_direct : step_plain;
   return f;

@@ -56,22 +56,28 @@ struct WindowParams {
 // far beyond any real wait (a strip's product takes microseconds) and still an end.
 static constexpr int kWindowPollLimit = 1 << 24;
 
-// TBK x TBN is the hashed tile (compile time).  The unit of work is a strip of 32 rows of a tile
-// (its slice of hashed_weight is the 32 * TBN elements from off + 32 * TBN * strip on): a
-// wavefront holds the strip's 32x32 blocks in registers.
+// The hashed tile is BK x TBN: TBN (32, 64 or 128) at compile time — it is the row pitch of a tile's
+// slice of hashed_weight — BK (a multiple of 32) at run time.  The unit of work is 32 rows by UC =
+// min(TBN, 64) columns of a tile: strip s (rows 32 s .. 32 s + 31) of a 128-column tile is two
+// units side by side.  Unit u = s * parts + part of a tile at `off` starts at off + 32 * TBN * s +
+// UC * part and its rows are TBN apart: from its first to its last element it spans kUnitSpan =
+// 31 * TBN + UC elements (all of them its own when the tile is no wider than 64).  A wavefront
+// holds the unit's 32x32 blocks in registers.
 // STAGED (K and N multiples of the 16-byte piece): operands travel as 16-byte pieces through the
 // wavefront's staging area (a quarter of the load instructions per byte for fp32, an eighth for the
 // 16-bit types); otherwise fragments are loaded element by element.
-template <typename T, int TBK, int TBN, bool STAGED>
+template <typename T, int TBN, bool STAGED>
 struct WindowKernel {
-  static_assert(TBK % 32 == 0 && TBN % 32 == 0, "a tile is whole 32x32 blocks");
+  static_assert(TBN == 32 || TBN == 64 || TBN == 128, "tiles of 32, 64 or 128 columns");
   typedef ElemTraits<T> Tr;
   typedef typename Mfma<T>::Frag Frag;
   static constexpr int kThreads = 1024;
   static constexpr int kWaves = kThreads / 64;
-  static constexpr int kStrips = TBK / 32;               // strips of a tile
-  static constexpr int kStripElems = 32 * TBN;           // elements of hashed_weight under a strip
-  static constexpr int BI = 1, BJ = TBN / 32;            // blocks of a strip
+  static constexpr int UC = TBN < 64 ? TBN : 64;         // columns of a unit
+  static constexpr int kParts = TBN / UC;                // units side by side in a strip of a tile
+  static constexpr int kUnitSpan = 31 * TBN + UC;        // elements of hashed_weight from a unit's first to its last
+  static constexpr int kMaxUnits = 16;                   // units of a tile at most (BK <= 256)
+  static constexpr int BI = 1, BJ = UC / 32;             // blocks of a unit
   static constexpr int KS = Tr::kMfmaK;                  // rows of M one MFMA contracts (16 or 2)
   // rows of M loaded ahead as one group (16 wavefronts per compute unit leave 128 registers each)
   static constexpr int kGroupRows = sizeof(T) == 4 ? 8 : 16;
@@ -85,13 +91,12 @@ struct WindowKernel {
   // staged: a wavefront's own staging area, one group of rows of X (32 columns) and of dY (TBN
   // columns), 3 KB; the list is kept shorter to make room for it next to the window
   static constexpr int VEC = Tr::kVec;                   // elements of a 16-byte piece
-  static constexpr int kStageX = kGroupRows * 32, kStageElems = STAGED ? kStageX + kGroupRows * TBN : 8;
-  static constexpr int kList = STAGED ? 960 : kThreads * kStrips;   // capacity of the list of strips found
-  static_assert(!STAGED || TBN == 64, "the staged dY rows are swizzled as two halves");
-  static_assert(!STAGED || (64 * VEC == kGroupRows * 32), "one piece of X and two of dY per lane and group");
+  static constexpr int kStageX = kGroupRows * 32, kStageElems = STAGED ? kStageX + kGroupRows * UC : 8;
+  static constexpr int kList = 960;   // capacity of the list of units found
+  static_assert(!STAGED || (64 * VEC == kGroupRows * 32), "one piece of X and BJ of dY per lane and group");
 
   struct Smem {
-    int list[kList];              // strips found in this pass (tile id * kStrips + strip), ascending
+    int list[kList];              // units found in this pass (tile id * units per tile + unit), ascending
     int offs[kList];              // ... their offsets in hashed_weight
     int done[kList];              // ... and whether they have been added to the window
     int count[2][kWaves];
@@ -157,6 +162,8 @@ struct WindowKernel {
 
     const int total = p.tiles_k * p.tiles_n;
     const int ngroups = (p.M + kGroupRows - 1) / kGroupRows;
+    const int units = (p.h.BK >> 5) * kParts;               // units of a tile (a power of two, at most kMaxUnits)
+    const int ushift = __builtin_ctz(units);
 
     f32x16_t acc[BI][BJ];
 #pragma unroll
@@ -168,38 +175,45 @@ struct WindowKernel {
     // kDepth register sets: the fragments of the next groups are loaded while this one is multiplied
     Frag fa[kDepth][GS][BI], fb[kDepth][GS][BJ];
     // 16-bit staged path: the raw 16-byte pieces instead (one of X, two of dY per lane and group)
-    u32x4_t px[kDepth], py[kDepth][2];
-    // element offset of this lane's piece of X, and of its two pieces of dY, from the first row of a group
+    u32x4_t px[kDepth], py[kDepth][BJ];
+    // element offset of this lane's piece of X, and of its BJ pieces of dY, from the first row of a group
     const int lane_x = STAGED ? (lane / (32 / VEC)) * (int)p.ldx + (lane % (32 / VEC)) * VEC : 0;
-    const int lane_y[2] = {STAGED ? (lane / (TBN / VEC)) * (int)p.lddy + (lane % (TBN / VEC)) * VEC : 0,
-                           STAGED ? (lane / (TBN / VEC) + 64 / (TBN / VEC)) * (int)p.lddy + (lane % (TBN / VEC)) * VEC : 0};
+    int lane_y[BJ];
+#pragma unroll
+    for (int q = 0; q < BJ; q++)
+      lane_y[q] = STAGED ? (lane / (UC / VEC) + q * (64 / (UC / VEC))) * (int)p.lddy + (lane % (UC / VEC)) * VEC : 0;
 
-    // Listing the strips that meet the window, in ascending (tile, strip) order.  The tile ids of
+    // Listing the units that meet the window, in ascending (tile, unit) order.  The tile ids of
     // a range [lo, hi) are dealt to the wavefronts in contiguous chunks; every wavefront first
-    // counts the strips of its chunk that meet the window, the counts are added up (one
-    // barrier), then it examines its chunk again and writes its strips behind those of the
+    // counts the units of its chunk that meet the window, the counts are added up (one
+    // barrier), then it examines its chunk again and writes its units behind those of the
     // wavefronts before it.  Normally the range is the whole table and the list (kList entries)
     // takes every hit; if it would overflow, the range is halved until its hits fit, and the
-    // rest of the table follows in further rounds.  (A range of one tile has at most kStrips
+    // rest of the table follows in further rounds.  (A range of one tile has at most kMaxUnits
     // hits, so the halving ends.)
-    auto strips_of = [&](int id, int off, unsigned long long* mask) -> int {
-      // ballots of "strip s of tile id meets the window" over the wavefront; returns their total
-      int n = 0;
-#pragma unroll
-      for (int s = 0; s < kStrips; s++) {
-        const long long so = (long long)off + (long long)s * kStripElems;
-        mask[s] = __ballot(id >= 0 && so < w0 + wlen && so + kStripElems > w0);
-        n += __popcll(mask[s]);
+    auto unit_start = [&](int off, int u) -> long long {
+      return (long long)off + (long long)(u / kParts) * (32 * TBN) + (u % kParts) * UC;
+    };
+    auto units_of = [&](int id, int off) -> unsigned {
+      // bit u: unit u of tile id meets the window (id < 0: no tile)
+      unsigned hits = 0u;
+      for (int u = 0; u < units; u++) {   // (uniform)
+        const long long so = unit_start(off, u);
+        hits |= (unsigned)(id >= 0 && so < w0 + wlen && so + kUnitSpan > w0) << u;
       }
-      return n;
+      return hits;
+    };
+    auto wave_sum = [&](int v) -> int {
+#pragma unroll
+      for (int d = 32; d >= 1; d >>= 1) v += __shfl_xor(v, d, 64);
+      return v;
     };
     const bool planned = p.plan_start != nullptr;   // (uniform)
     if (planned) {
       // A plan built for another layer would send the loads below anywhere: refuse it, loudly
       // (the window of dHW becomes NaN), instead of reading outside X and dY.
       const int32_t* hd = p.plan_header;
-      if (!layer_plan_matches(hd, p.K, p.N, p.H, p.h) || hd[5] != TBK || hd[6] != TBN || hd[10] != p.window ||
-          hd[12] != kStrips) {
+      if (!layer_plan_matches(hd, p.K, p.N, p.H, p.h) || hd[6] != TBN || hd[10] != p.window || hd[12] != units) {
         const float nan = __builtin_nanf("");
         if (p.out_f32 || sizeof(T) == 4) {
           for (int i = tid; i < wlen; i += kThreads) (static_cast<float*>(p.dHW) + w0)[i] = nan;
@@ -241,10 +255,10 @@ struct WindowKernel {
   #pragma unroll
             for (int u = 0; u < kBatch; u++) {
               const int id = id0 + u * 64 + lane;
-              unsigned long long mask[kStrips];
-              mine += strips_of(id < end ? id : -1, offv[u], mask);
+              mine += __popc(units_of(id < end ? id : -1, offv[u]));
             }
           }
+          mine = wave_sum(mine);
           __syncthreads();   // (the counts of the previous attempt or round have been read)
           if (lane == 0) sm.count[0][wave] = mine;
           __syncthreads();
@@ -252,7 +266,7 @@ struct WindowKernel {
   #pragma unroll
           for (int w = 0; w < kWaves; w++) found += __builtin_amdgcn_readfirstlane(sm.count[0][w]);
           if (found <= kList) break;
-          hi = lo + (hi - lo) / 2;   // (found > kList >= kStrips, so the range holds at least two tiles)
+          hi = lo + (hi - lo) / 2;   // (found > kList >= kMaxUnits, so the range holds at least two tiles)
         }
         {
           int at = 0;
@@ -269,22 +283,25 @@ struct WindowKernel {
   #pragma unroll
             for (int u = 0; u < kBatch; u++) {
               const int id = id0 + u * 64 + lane;
-              unsigned long long mask[kStrips];
-              const int n = strips_of(id < end ? id : -1, offv[u], mask);
-              // the strips of the lanes below me, then my own in order
-              int mine = at;
+              unsigned hits = units_of(id < end ? id : -1, offv[u]);
+              // the units of the lanes below me (tiles with smaller ids), then my own in order
+              const int c = __popc(hits);
+              int incl = c;
   #pragma unroll
-              for (int s = 0; s < kStrips; s++) mine += __popcll(mask[s] & ((1ull << lane) - 1ull));
-  #pragma unroll
-              for (int s = 0; s < kStrips; s++) {
-                if ((mask[s] >> lane) & 1ull) {
-                  sm.list[mine] = id * kStrips + s;
-                  sm.offs[mine] = offv[u] + s * kStripElems;
-                  sm.done[mine] = 0;
-                  mine++;
-                }
+              for (int d = 1; d < 64; d <<= 1) {
+                const int up = __shfl_up(incl, d, 64);
+                if (lane >= d) incl += up;
               }
-              at += n;
+              int mine = at + incl - c;
+              while (hits != 0u) {
+                const int un = __builtin_ctz(hits);
+                hits &= hits - 1u;
+                sm.list[mine] = (id << ushift) + un;
+                sm.offs[mine] = (int)unit_start(offv[u], un);
+                sm.done[mine] = 0;
+                mine++;
+              }
+              at += __shfl(incl, 63, 64);
             }
           }
         }
@@ -313,13 +330,13 @@ struct WindowKernel {
       //  and turn the loads into flat ones, which also count as LDS traffic)
       int strip_x = 0, strip_k0 = 0, strip_n0 = 0;
       bool strip_whole = false;
-      // which of a lane's three pieces of the group at row m0 of strip (k0, n0) lie inside the matrices
-      auto pieces_inside = [&](int m0, int k0, int n0, bool& okx, bool& oky0, bool& oky1) {
-        constexpr int PX = 32 / VEC, PY = TBN / VEC;
+      // which of a lane's pieces of the group at row m0 of the unit at (k0, n0) lie inside the matrices
+      auto pieces_inside = [&](int m0, int k0, int n0, bool& okx, bool (&oky)[BJ]) {
+        constexpr int PX = 32 / VEC, PY = UC / VEC;
         okx = m0 + lane / PX < p.M && k0 + (lane % PX) * VEC < p.K;
         const bool col_ok = n0 + (lane % PY) * VEC < p.N;
-        oky0 = m0 + lane / PY < p.M && col_ok;
-        oky1 = m0 + lane / PY + 64 / PY < p.M && col_ok;
+#pragma unroll
+        for (int q = 0; q < BJ; q++) oky[q] = m0 + lane / PY + q * (64 / PY) < p.M && col_ok;
       };
       // ... and the same for the strip being multiplied
       int mult_k0 = 0, mult_n0 = 0;
@@ -330,11 +347,11 @@ struct WindowKernel {
           if (fg == 0) {   // (uniform) a new strip
             const int ftc = ft < my_tiles ? ft : my_tiles - 1;
             const int v = __builtin_amdgcn_readfirstlane(sm.list[wave + ftc * kWaves]);
-            const int id = v / kStrips, strip = v % kStrips;
+            const int id = v >> ushift, un = v & (units - 1);
             const int tk = id / p.tiles_n, tn = id - tk * p.tiles_n;
-            strip_k0 = tk * TBK + strip * 32;              // the strip's first row of W
-            strip_n0 = tn * TBN;
-            strip_whole = strip_k0 + 32 <= p.K && strip_n0 + TBN <= p.N;
+            strip_k0 = tk * p.h.BK + (un / kParts) * 32;   // the unit's first row of W
+            strip_n0 = tn * TBN + (un % kParts) * UC;      // ... and first column
+            strip_whole = strip_k0 + 32 <= p.K && strip_n0 + UC <= p.N;
             // (a strip that begins beyond K contributes nothing; its base is kept inside the matrix)
             strip_x = strip_k0 < p.K ? strip_k0 : p.K - 1;
           }
@@ -342,8 +359,9 @@ struct WindowKernel {
           const T* rows_x = gX + ((int64_t)m0 * p.ldx + strip_x);
           const T* rows_y = gdY + ((int64_t)m0 * p.lddy + strip_n0);
           const T* src_x = rows_x + lane_x;
-          const T* src_y0 = rows_y + lane_y[0];
-          const T* src_y1 = rows_y + lane_y[1];
+          const T* src_y[BJ];
+#pragma unroll
+          for (int q = 0; q < BJ; q++) src_y[q] = rows_y + lane_y[q];
           if (!(strip_whole && m0 + kGroupRows <= p.M)) {   // (uniform, rare)
             // a piece outside the matrix is fetched from inside it (and replaced by zero when the
             // item is multiplied, where the same checks are made again: nothing about a set is
@@ -351,15 +369,15 @@ struct WindowKernel {
             // (the empty statement keeps this block out of the usual path: its arithmetic would
             //  otherwise be carried out for every item and thrown away)
             asm volatile("" ::: "memory");
-            bool okx, oky0, oky1;
-            pieces_inside(m0, strip_k0, strip_n0, okx, oky0, oky1);
+            bool okx, oky[BJ];
+            pieces_inside(m0, strip_k0, strip_n0, okx, oky);
             src_x = okx ? src_x : gX + (int64_t)m0 * p.ldx;
-            src_y0 = oky0 ? src_y0 : gdY + (int64_t)m0 * p.lddy;
-            src_y1 = oky1 ? src_y1 : gdY + (int64_t)m0 * p.lddy;
+#pragma unroll
+            for (int q = 0; q < BJ; q++) src_y[q] = oky[q] ? src_y[q] : gdY + (int64_t)m0 * p.lddy;
           }
           __builtin_memcpy(&px[S], src_x, 16);
-          __builtin_memcpy(&py[S][0], src_y0, 16);
-          __builtin_memcpy(&py[S][1], src_y1, 16);
+#pragma unroll
+          for (int q = 0; q < BJ; q++) __builtin_memcpy(&py[S][q], src_y[q], 16);
           if (++fg == ngroups) {
             fg = 0;
             ft++;
@@ -369,14 +387,15 @@ struct WindowKernel {
         {
           const int ftc = ft < my_tiles ? ft : my_tiles - 1;
           const int v = __builtin_amdgcn_readfirstlane(sm.list[wave + ftc * kWaves]);
-          const int id = v / kStrips, strip = v % kStrips;
+          const int id = v >> ushift, un = v & (units - 1);
           const int tk = id / p.tiles_n, tn = id - tk * p.tiles_n;
-          const int k0 = tk * TBK + strip * 32;              // the strip's first row of W
+          const int k0 = tk * p.h.BK + (un / kParts) * 32;   // the unit's first row of W
+          const int n0 = tn * TBN + (un % kParts) * UC;      // ... and first column
           const int m0 = fg * kGroupRows;
           const bool whole = m0 + kGroupRows <= p.M;
           // (a strip that begins beyond K contributes nothing; its base is kept inside the matrix)
           const T* rows_x = gX + (int64_t)m0 * p.ldx + (int64_t)(k0 < p.K ? k0 : p.K - 1);
-          const T* rows_y = gdY + (int64_t)m0 * p.lddy + (int64_t)tn * TBN;
+          const T* rows_y = gdY + (int64_t)m0 * p.lddy + (int64_t)(n0 < p.N ? n0 : p.N - 1);
 #pragma unroll
           for (int a = 0; a < BI; a++) {
             const int col = a * 32 + (lane & 31);
@@ -388,7 +407,7 @@ struct WindowKernel {
 #pragma unroll
           for (int b = 0; b < BJ; b++) {
             const int col = b * 32 + (lane & 31);
-            const bool ok = tn * TBN + col < p.N;
+            const bool ok = n0 + col < p.N;
 #pragma unroll
             for (int s = 0; s < GS; s++)
               fb[S][s][b] = load_frag(rows_y, p.lddy, s * KS, m0, p.M, lane, ok ? col : 0, ok, whole);
@@ -413,7 +432,7 @@ struct WindowKernel {
           for (int f = lane; f < e; f += 64) {
             const int d = sm.offs[f] - tile_off;
             const int dn = __hip_atomic_load(&sm.done[f], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-            pending |= (d < kStripElems) & (d > -kStripElems) & (dn == 0);
+            pending |= (d < kUnitSpan) & (d > -kUnitSpan) & (dn == 0);
           }
           if (!__any(pending)) break;
           if (polls >= p.poll_limit) {   // (uniform)
@@ -424,8 +443,8 @@ struct WindowKernel {
         }
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
         const int rel = (int)((long long)tile_off - w0);   // (offsets and window starts are below 2^31)
-        if (rel >= 0 && rel + kStripElems <= wlen) {
-          // the whole strip lies inside the window (the usual case): no checks, constant offsets
+        if (rel >= 0 && rel + kUnitSpan <= wlen) {
+          // the whole unit lies inside the window (the usual case): no checks, constant offsets
 #pragma unroll
           for (int b = 0; b < BJ; b++) {
             float* at = win + rel + ((lane >> 5) * 4) * TBN + b * 32 + (lane & 31);
@@ -488,34 +507,38 @@ struct WindowKernel {
             // out in order, so neither the reads below nor the next group's writes need a barrier)
             T* st = sm.stage[wave];
             const u32x4_t z = {0u, 0u, 0u, 0u};
-            constexpr int PX = 32 / VEC, PY = TBN / VEC;
+            constexpr int PX = 32 / VEC, PY = UC / VEC;
             // (pieces outside the matrix become zero; the usual set has none: a uniform branch, no selects)
-            u32x4_t wx = px[S], wy[2] = {py[S][0], py[S][1]};
-            if (pg == 0) {   // (uniform) a new strip
+            u32x4_t wx = px[S], wy[BJ];
+#pragma unroll
+            for (int q = 0; q < BJ; q++) wy[q] = py[S][q];
+            if (pg == 0) {   // (uniform) a new unit
               const int ptc = pt < my_tiles ? pt : my_tiles - 1;
               const int v = __builtin_amdgcn_readfirstlane(sm.list[wave + ptc * kWaves]);
-              const int id = v / kStrips, tk = id / p.tiles_n;
-              mult_k0 = tk * TBK + (v % kStrips) * 32;
-              mult_n0 = (id - tk * p.tiles_n) * TBN;
-              mult_whole = mult_k0 + 32 <= p.K && mult_n0 + TBN <= p.N;
+              const int id = v >> ushift, un = v & (units - 1), tk = id / p.tiles_n;
+              mult_k0 = tk * p.h.BK + (un / kParts) * 32;
+              mult_n0 = (id - tk * p.tiles_n) * TBN + (un % kParts) * UC;
+              mult_whole = mult_k0 + 32 <= p.K && mult_n0 + UC <= p.N;
             }
             if (!(mult_whole && (pg + 1) * kGroupRows <= p.M)) {
               asm volatile("" ::: "memory");
-              bool okx, oky0, oky1;
-              pieces_inside(pg * kGroupRows, mult_k0, mult_n0, okx, oky0, oky1);
+              bool okx, oky[BJ];
+              pieces_inside(pg * kGroupRows, mult_k0, mult_n0, okx, oky);
               wx = okx ? wx : z;
-              wy[0] = oky0 ? wy[0] : z;
-              wy[1] = oky1 ? wy[1] : z;
+#pragma unroll
+              for (int q = 0; q < BJ; q++) wy[q] = oky[q] ? wy[q] : z;
             }
             *reinterpret_cast<u32x4_t*>(st + (lane / PX) * 32 + (lane % PX) * VEC) = wx;
             if constexpr (k16) {
 #pragma unroll
-              for (int q = 0; q < 2; q++) {
-                const int r = (lane >> 3) + 8 * q, pc = lane & 7;
-                // dY rows are two 64-byte chunks, swapped in every other pair of rows, so that the four
-                // rows of a transpose read fall on different banks
-                *reinterpret_cast<u32x4_t*>(st + kStageX + r * TBN + ((((pc >> 2) ^ ((r >> 1) & 1)) << 5) | ((pc & 3) << 3))) =
-                    wy[q];
+              for (int q = 0; q < BJ; q++) {
+                const int r = lane / PY + (64 / PY) * q, pc = lane % PY;
+                // 64-column units: dY rows are two 64-byte chunks, swapped in every other pair of rows, so
+                // that the four rows of a transpose read fall on different banks; 32-column units lie as X does
+                if constexpr (UC == 64)
+                  *reinterpret_cast<u32x4_t*>(st + kStageX + r * UC + ((((pc >> 2) ^ ((r >> 1) & 1)) << 5) | ((pc & 3) << 3))) = wy[q];
+                else
+                  *reinterpret_cast<u32x4_t*>(st + kStageX + r * UC + pc * VEC) = wy[q];
               }
               // fragments by the LDS transpose read: within 16 lanes, lane c receives column c of a
               // 4 x 16 block whose rows the lanes address four-per-row
@@ -533,16 +556,17 @@ struct WindowKernel {
               Frag b[BJ];
 #pragma unroll
               for (int j = 0; j < BJ; j++)
-                b[j] = tr_frag(st + kStageX + row * TBN + (((j ^ ((row >> 1) & 1)) << 5) | col), TBN);
+                b[j] = UC == 64 ? tr_frag(st + kStageX + row * UC + (((j ^ ((row >> 1) & 1)) << 5) | col), UC)
+                                : tr_frag(st + kStageX + row * UC + col, UC);
 #pragma unroll
               for (int j = 0; j < BJ; j++) acc[0][j] = Mfma<T>::run(a, b[j], acc[0][j]);
             } else {
               // fp32: the two 128-byte halves of a dY row are swapped in every other row, so that the
               // two rows of an MFMA step (lanes 0-31 and 32-63) lie on different banks
 #pragma unroll
-              for (int q = 0; q < 2; q++) {
+              for (int q = 0; q < BJ; q++) {
                 const int r = lane / PY + (64 / PY) * q, c = (lane % PY) * VEC;
-                *reinterpret_cast<u32x4_t*>(st + kStageX + r * TBN + (c ^ ((r & 1) << 5))) = wy[q];
+                *reinterpret_cast<u32x4_t*>(st + kStageX + r * UC + (UC == 64 ? (c ^ ((r & 1) << 5)) : c)) = wy[q];
               }
               // fragments: lane l holds row 2 s + (l >> 5), column l & 31 of the block
               const int mg = lane >> 5, cl = lane & 31;
@@ -551,7 +575,7 @@ struct WindowKernel {
               for (int g = 0; g < GS; g++) {
                 a[g] = st[(2 * g + mg) * 32 + cl];
 #pragma unroll
-                for (int j = 0; j < BJ; j++) b[g][j] = st[kStageX + (2 * g + mg) * TBN + (((j ^ mg) << 5) | cl)];
+                for (int j = 0; j < BJ; j++) b[g][j] = st[kStageX + (2 * g + mg) * UC + (UC == 64 ? (((j ^ mg) << 5) | cl) : cl)];
               }
 #pragma unroll
               for (int g = 0; g < GS; g++)
@@ -623,9 +647,9 @@ struct WindowKernel {
   }
 };
 
-template <typename T, int TBK, int TBN, bool STAGED>
-__global__ __launch_bounds__((WindowKernel<T, TBK, TBN, STAGED>::kThreads)) void rz_window_kernel(WindowParams p) {
-  typedef WindowKernel<T, TBK, TBN, STAGED> K;
+template <typename T, int TBN, bool STAGED>
+__global__ __launch_bounds__((WindowKernel<T, TBN, STAGED>::kThreads)) void rz_window_kernel(WindowParams p) {
+  typedef WindowKernel<T, TBN, STAGED> K;
   extern __shared__ __attribute__((aligned(16))) unsigned char rz_window_smem[];
   K::run(p, *reinterpret_cast<typename K::Smem*>(rz_window_smem));
 }

@@ -61,9 +61,8 @@ def weight_grad_hashed(input, output_grad, init_factor, M, K, N, H, R, BLOCK_SIZ
         if not accumulate:
             out.zero_()
         return out, (torch.zeros((N,), device=output_grad.device, dtype=output_grad.dtype) if with_bias_grad else None)
-    columns = N
-    x, ldx, K = _lib.whole_pieces(input, K)          # (K, N: the extents the call is made with)
-    dy, lddy, N = _lib.whole_pieces(output_grad, N)
+    x, ldx = _lib.rows(input)
+    dy, lddy = _lib.rows(output_grad)
     bias_grad = torch.empty((N,), device=output_grad.device, dtype=output_grad.dtype) if with_bias_grad else None
     tuning = _lib.current_tuning()
     need = _lib.host_query("rz_weight_grad_hashed_workspace_bytes", M, K, N, H, BLOCK_SIZE_K, BLOCK_SIZE_N, code,
@@ -85,7 +84,7 @@ def weight_grad_hashed(input, output_grad, init_factor, M, K, N, H, R, BLOCK_SIZ
             x.data_ptr(), dy.data_ptr(), out.data_ptr(), bias_grad.data_ptr() if with_bias_grad else None,
             ws.data_ptr() if need else None, need, M, K, N, H, BLOCK_SIZE_K, BLOCK_SIZE_N, R, hash_levels,
             float(init_factor), ldx, lddy, code, flags, tuning, stream))
-    return out, (bias_grad[:columns] if with_bias_grad else None)
+    return out, bias_grad
 
 
 def rz_linear_backward_weight_grad_tl(input: torch.Tensor, output_grad: torch.Tensor, init_factor: float,
@@ -155,7 +154,7 @@ def input_grad_hashed(output_grad, hashed_weight, init_factor, M, K, N, H, R, BK
         raise TypeError("output_grad is %s but hashed_weight is %s" % (output_grad.dtype, hashed_weight.dtype))
     if M == 0:
         return torch.empty((0, K), device=output_grad.device, dtype=output_grad.dtype)
-    dy, lddy, N = _lib.whole_pieces(output_grad, N)   # (N: the extent the call is made with)
+    dy, lddy = _lib.rows(output_grad)
     hw = hashed_weight.contiguous()
     input_grad = torch.empty((M, K), device=output_grad.device, dtype=output_grad.dtype)
     lib = _lib.load()

@@ -53,7 +53,7 @@ def forward_hashed(input, hashed_weight, bias, init_factor, M, K, N, H, R, BK, B
         bias = bias.contiguous()
     if M == 0:   # an empty batch: nothing to launch, as the reference returns its empty zeros((0, N))
         return torch.empty((0, N), device=input.device, dtype=input.dtype)
-    x, ldx, K = _lib.whole_pieces(input, K)   # (K: the extent the call is made with)
+    x, ldx = _lib.rows(input)
     hw = hashed_weight.contiguous()
     output = torch.empty((M, N), device=input.device, dtype=input.dtype)
     lib = _lib.load()

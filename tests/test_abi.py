@@ -171,13 +171,15 @@ def _window_geometry(H):
 
 @pytest.mark.parametrize("cfg", [(1024, 1024, 65536, 64, 64), (300, 330, 70000, 32, 64), (4096, 8192, 40000, 64, 64),
                                  (640, 640, 2000001, 64, 64), (192, 128, 7000000, 64, 64), (96, 72, 100000, 32, 64),
-                                 (512, 512, 30000, 128, 128), (256, 256, 1000, 16, 16)])
+                                 (512, 512, 30000, 128, 128), (256, 256, 1000, 16, 16), (300, 520, 90000, 64, 32),
+                                 (512, 300, 200000, 256, 128), (256, 512, 70000, 32, 256)])
 @pytest.mark.parametrize("levels", [2, 3])
 def test_layer_plan_lists_every_strip_in_every_window_it_meets(lib, oracle, cfg, levels):
     """rz_layer_plan_build against a brute-force restatement: the tile offsets are the oracle's, and
-    the list of window b holds exactly the 32-row strips [off + 32*BN*s, + 32*BN) that meet
-    [b*w, (b+1)*w), in ascending (tile, strip) order, with their offsets.  Tiles the window kernel
-    does not serve (BN != 64, BK not 32 or 64) get a plan with the offsets alone."""
+    the list of window b holds exactly the units of work of the window kernel — 32 rows by min(BN, 64)
+    columns of a tile: unit s * parts + part starts at off + 32*BN*s + 64*part and spans 31*BN + min(BN, 64)
+    elements — that meet [b*w, (b+1)*w), in ascending (tile, unit) order, with their offsets.  Tiles the
+    window kernel does not serve (16 or 256 columns, 16 rows) get a plan with the offsets alone."""
     K, N, H, BK, BN = cfg
     R = R1024 if levels == 2 else oracle.legacy_constants(1024)
     nbytes = lib.rz_layer_plan_bytes(K, N, H, BK, BN)
@@ -189,7 +191,7 @@ def test_layer_plan_lists_every_strip_in_every_window_it_meets(lib, oracle, cfg,
     want = oracle.c_tile_offsets(K, N, H, BK, BN, R, levels).reshape(-1)
     assert plan[0] == 0x525A4C50 and list(plan[2:9]) == [K, N, H, BK, BN, levels, tiles]
     assert np.array_equal(plan[16:16 + tiles].astype(np.int64), want)
-    served = BN == 64 and BK in (32, 64)
+    served = BN in (32, 64, 128) and BK in (32, 64, 128, 256)
     windows, w = int(plan[9]), int(plan[10])
     if not served:
         assert windows == 0 and plan[11] == 0
@@ -197,14 +199,17 @@ def test_layer_plan_lists_every_strip_in_every_window_it_meets(lib, oracle, cfg,
     assert (w, windows) == _window_geometry(H)
     r16 = lambda v: (v + 15) & ~15
     start_at = r16(16 + tiles)
-    strips, selems = BK // 32, 32 * BN
+    uc = min(BN, 64)
+    parts = BN // uc
+    strips, selems = (BK // 32) * parts, 31 * BN + uc
     cap = tiles * strips * (-(-selems // w) + 1)
     list_at = r16(start_at + windows + 1)
     offs_at = r16(list_at + cap)
     assert nbytes == 4 * r16(offs_at + cap)
     start = plan[start_at:start_at + windows + 1]
     assert start[0] == 0 and start[-1] == plan[11] and np.all(np.diff(start) >= 0) and start[-1] <= cap
-    so = (want[:, None] + np.arange(strips)[None, :] * selems).reshape(-1)       # index = tile * strips + strip
+    u = np.arange(strips)
+    so = (want[:, None] + ((u // parts) * 32 * BN + (u % parts) * uc)[None, :]).reshape(-1)   # index = tile * units + unit
     for b in range(windows):
         meets = np.nonzero((so < (b + 1) * w) & (so + selems > b * w))[0]
         got = plan[list_at + start[b]:list_at + start[b + 1]]

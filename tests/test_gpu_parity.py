@@ -521,32 +521,53 @@ def test_random_shapes_16bit(oracle, shape):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=lambda d: str(d).split(".")[-1])
-@pytest.mark.parametrize("shape", [(1100, 1023, 1001, 40000, 32, 64), (1030, 1025, 2047, 300000, 64, 64)],
+@pytest.mark.parametrize("shape", [(1100, 1023, 1001, 40000, 32, 64), (1030, 1025, 2047, 300000, 64, 64),
+                                   (512, 1031, 1017, 9000, 64, 64), (300, 9, 15, 3000, 16, 16), (257, 2049, 263, 9000, 64, 64)],
                          ids=lambda s: "x".join(map(str, s)))
-def test_large_16_bit_operands_with_odd_rows_are_padded_to_whole_pieces(oracle, shape, dtype):
-    """K and N that are not multiples of 8 would keep the 16-bit kernels off their direct-to-LDS
-    path; the launchers copy a large operand into zero-padded rows once and make the call with
-    the padded extent.  All three products and the bias gradient against the oracle; untouched
-    slots of dHW stay zero (the padding adds zeros to slots that the tiles cover anyway)."""
+def test_16_bit_rows_that_are_not_whole_16_byte_pieces(oracle, shape, dtype):
+    """K and N that are not multiples of 8, the operands contiguous (so that every row starts at another
+    alignment and the last row ends with the allocation's last element): the kernels keep their
+    direct-to-LDS path, fetch the piece that straddles a row end as it lies, and put the last row's
+    right in LDS; nothing is copied or padded on the way (the reference masks element by element,
+    python/rz_linear/impl/RzLinearForward.py:338-341).  Straight through the C ABI, all three
+    products and the bias gradient against the oracle, element by element; a hashed_weight with an
+    inf in a slot that no tile of the layer touches must not show in any result."""
+    import ctypes
     from rzlinear_amd import _lib
-    from rzlinear_amd.impl.RzLinearBackward import (rz_linear_backward_input_grad_tl,
-                                                    rz_linear_backward_weight_bias_grad_tl)
-    from rzlinear_amd.impl.RzLinearForward import rz_linear_forward_bias_tl
+    lib = _lib.load()
     M, K, N, H, BK, BN = shape
-    _say("odd rows, padded", shape, dtype)
+    _say("odd rows, in the kernels", shape, dtype)
     (x, hw, dy), (x64, hw64, dy64) = make_inputs(M, K, N, H, dtype, seed=31)
-    assert _lib.whole_pieces(x, K)[2] == (K + 7) // 8 * 8 and _lib.whole_pieces(dy, N)[2] == (N + 7) // 8 * 8
-    bias = torch.randn((N,), generator=torch.Generator().manual_seed(5)).to(dtype)
-    kw = dict(BLOCK_SIZE_K=BK, BLOCK_SIZE_N=BN)
-    y = rz_linear_forward_bias_tl(x, hw, bias.cuda(), 1.0, M, K, N, H, *rargs(R1024), **kw)
-    dx = rz_linear_backward_input_grad_tl(dy, hw, 1.0, M, K, N, H, *rargs(R1024), **kw)
-    dhw, dbias = rz_linear_backward_weight_bias_grad_tl(x, dy, 1.0, M, K, N, H, *rargs(R1024), **kw)
+    # exact-size allocations: the row ends are where the tensors end
+    x, dy = x.clone(), dy.clone()
+    code = _lib.dtype_code(x)
+    R = (ctypes.c_int32 * 8)(*R1024)
+    stream = torch.cuda.current_stream().cuda_stream
+    bias = torch.randn((N,), generator=torch.Generator().manual_seed(5)).to(dtype).cuda()
+    # an inf where no tile reaches (if there is such a slot): the padded-copy scheme this replaces turned it into NaN
+    idx = oracle.index_map(K, N, H, BK, BN, R1024)
+    free = np.setdiff1d(np.arange(H), idx.reshape(-1))
+    if free.size:
+        hw[int(free[0])] = float("inf")
+    y = torch.full((M, N), float("nan"), dtype=dtype, device="cuda")
+    dx = torch.full((M, K), float("nan"), dtype=dtype, device="cuda")
+    dhw = torch.full((H,), float("nan"), dtype=dtype, device="cuda")
+    dbias = torch.full((N,), float("nan"), dtype=dtype, device="cuda")
+    fq = _lib.plan_query(0, M, K, N, H, BK, BN, code)
+    _lib.check(lib.rz_forward_bias(x.data_ptr(), hw.data_ptr(), bias.data_ptr(), y.data_ptr(), M, K, N, H, BK, BN, R, 1.0,
+                                   K, N, code, stream))
+    _lib.check(lib.rz_input_grad(dy.data_ptr(), hw.data_ptr(), dx.data_ptr(), M, K, N, H, BK, BN, R, 1.0, N, K, code, stream))
+    need = lib.rz_weight_grad_ex_workspace_bytes(M, K, N, H, BK, BN, code, 0, 1)
+    ws = torch.empty((max(need, 16),), dtype=torch.uint8, device="cuda")
+    _lib.check(lib.rz_weight_grad_ex(x.data_ptr(), dy.data_ptr(), dhw.data_ptr(), dbias.data_ptr(), ws.data_ptr(), need,
+                                     M, K, N, H, BK, BN, R, 1.0, K, N, code, 0, stream))
     torch.cuda.synchronize()
-    assert y.shape == (M, N) and dx.shape == (M, K) and dhw.shape == (H,) and dbias.shape == (N,)
     f = lambda t: t.float().cpu().numpy()
-    assert_close(f(y), oracle.forward(x64, hw64, N, BK, BN, R1024) + bias.double().numpy()[None, :], dtype, "Y")
+    assert_close(f(y), oracle.forward(x64, hw64, N, BK, BN, R1024) + bias.double().cpu().numpy()[None, :], dtype, "Y")
     assert_close(f(dx), oracle.input_grad(dy64, hw64, K, BK, BN, R1024), dtype, "dX")
     ref = oracle.weight_grad(x64, dy64, H, BK, BN, R1024)
     assert_close(f(dhw), ref, dtype, "dHW")
     assert (f(dhw)[ref == 0] == 0).all()
     assert rel_err(f(dbias), dy64.sum(axis=0)) <= TOL[dtype]
+    # (where the plan takes a 128 or 256 tile these shapes run the direct-to-LDS kernels: say which)
+    _say("   forward plan", fq, "weight-grad plan", _lib.plan_query(2, M, K, N, H, BK, BN, code))

@@ -24,6 +24,16 @@ CASES = [
     (40, 520, 264, 500000, 64, 64),       # 16-byte pieces whole, last tile row has one strip beyond K
     (17, 96, 72, 100000, 32, 64),         # one partial group of rows of M
     (8, 4096, 8192, 40000, 64, 64),       # more strips meet a window than its list holds (16-bit)
+    # the other hashed tiles of the reference's own tests (python/tests/test_rz_linear.py:38-39, :95-96) and of
+    # its autotuner: 128 columns are two 64-column units side by side, 32 columns a narrower unit, up to 256 rows
+    (48, 512, 1024, 300000, 32, 128),
+    (100, 520, 200, 90000, 64, 32),       # ragged: the last tiles reach beyond K and N
+    (33, 640, 768, 500000, 128, 128),
+    (70, 300, 330, 70000, 128, 64),
+    (20, 1024, 264, 200000, 256, 32),
+    (24, 200, 520, 150000, 32, 128),      # N ends inside the first unit of the last tile: its second lies beyond N
+    (16, 2048, 4096, 40000, 64, 32),      # more units meet a window than its list holds
+    (45, 257, 259, 80000, 64, 128),       # rows that are not whole 16-byte pieces: fragments element by element
 ]
 _dt_id = lambda d: str(d).split(".")[-1]
 _shape_id = lambda s: "x".join(map(str, s))
