@@ -70,25 +70,42 @@ PEAK = {"bf16": 2500.0, "fp16": 2500.0, "fp32": 157.3}
 # summary and are dropped (null) for a workload that has none.
 TRAFFIC = {
     # HBM bytes per launch of the contraction kernel of each leg: FETCH_SIZE * 2.0 + WRITE_SIZE * 1.0 KiB
-    # (factors from the copy calibration in the same profile)
+    # (factors from the copy calibration at the end of every profile: a 256 MiB device copy reads back
+    #  FETCH_SIZE = 131085, WRITE_SIZE = 262144)
     ("square4096", "bf16"): {
         "profile": "profiles/rz_gemm_bf16_square4096.txt",
-        "bytes": {"forward": int((16684.7 * 2.0 + 32768.0) * 1024),       # algorithmic: 64.03 MiB
-                  "input_grad": int((16687.2 * 2.0 + 32768.0) * 1024),
-                  "weight_grad": int((98460.5 * 2.0 + 16784.3) * 1024)},  # X, dY re-read by the XCDs' tile groups; + partial images
+        "bytes": {"forward": int((16680.8 * 2.0 + 32768.0) * 1024),       # algorithmic: 64.03 MiB
+                  "input_grad": int((16666.7 * 2.0 + 32768.0) * 1024),
+                  "weight_grad": int((98456.4 * 2.0 + 16784.8) * 1024)},  # X, dY re-read by the XCDs' tile groups; + partial images
+    },
+    ("square2048", "bf16"): {
+        "profile": "profiles/rz_gemm_bf16_square2048.txt",
+        "bytes": {"forward": int((4344.7 * 2.0 + 8192.0) * 1024), "input_grad": int((4344.5 * 2.0 + 8192.0) * 1024),
+                  "weight_grad": int((24694.3 * 2.0 + 16384.0) * 1024)},
     },
     ("square4096", "fp32"): {
         "profile": "profiles/rz_gemm_fp32_square4096.txt",
-        "bytes": {"forward": int((34806.3 * 2.0 + 70144.0) * 1024),       # algorithmic: 128.06 MiB
-                  "input_grad": int((33265.9 * 2.0 + 67072.0) * 1024),
-                  "weight_grad": int((196838.4 * 2.0 + 17808.0) * 1024)},
+        "bytes": {"forward": int((34823.8 * 2.0 + 70144.0) * 1024),       # algorithmic: 128.06 MiB
+                  "input_grad": int((33283.2 * 2.0 + 67072.0) * 1024),
+                  "weight_grad": int((196840.9 * 2.0 + 17808.0) * 1024)},
+    },
+    ("cpu_ref_1024", "fp32"): {
+        "profile": "profiles/rz_gemm_fp32_cpu_ref_1024.txt",
+        "bytes": {"forward": int((3165.9 * 2.0 + 4096.0) * 1024), "input_grad": int((3161.0 * 2.0 + 4096.0) * 1024),
+                  "weight_grad": int((12358.1 * 2.0 + 4096.0) * 1024)},   # X^T.dY written tile by tile: 4 MiB
     },
     ("ffn", "bf16"): {
         "profile": "profiles/rz_gemm_fold_bf16_ffn.txt",
-        "bytes": {"forward": int((70906.4 * 2.0 + 262144.0) * 1024),      # algorithmic: 320.1 MiB
-                  "input_grad": int((132355.8 * 2.0 + 65536.0) * 1024),
+        "bytes": {"forward": int((70832.2 * 2.0 + 262144.0) * 1024),      # algorithmic: 320.1 MiB
+                  "input_grad": int((132317.2 * 2.0 + 65536.0) * 1024),
                   # contraction (X, dY re-read by the XCDs' tile groups; X^T.dY written tile by tile: 256 MiB)
-                  "weight_grad": int((786918.0 * 2.0 + 262144.0) * 1024)},
+                  "weight_grad": int((786762.1 * 2.0 + 262144.0) * 1024)},
+    },
+    ("grid_1024_10240", "bf16"): {
+        "profile": "profiles/rz_gemm_fold_bf16_grid_1024_10240.txt",
+        "bytes": {"forward": int((353978.1 * 2.0 + 122880.0) * 1024),     # (three slices: fp32 partial planes written)
+                  "input_grad": int((345242.2 * 2.0 + 122880.0) * 1024),
+                  "weight_grad": int((173032.9 * 2.0 + 409600.0) * 1024)},
     },
 }
 

@@ -157,7 +157,12 @@ struct GemmKernel {
   // per step, halving the barriers per flop (8 % faster at 2048^3).
   static constexpr bool kLongStep = Tr::kBytes == 2 && (FULL || CLAMP) && NSTAGE == 2 && TI == 128 && TJ == 128 &&
                                     WI * WJ == 8;
-  static constexpr int TR = (kLongStep ? 256 : 128) / Tr::kBytes;
+  // ... and the fp32 tiles of at most 64 rows in forward / input-grad, whose 128-byte step is over in
+  // 0.4 us — less than a load from L2 takes, so that loads issued two steps ahead arrive late, and
+  // half as many barriers per flop (1024^3: forward 30.2 -> 28.3 us, input-grad 27.1 -> 25.9 us;
+  // the four-wavefront weight-grad form lost 3 % with it and keeps the short step)
+  static constexpr bool kLongStepF32 = Tr::kBytes == 4 && NSTAGE == 2 && TI <= 64 && OP != kWeightGrad;
+  static constexpr int TR = ((kLongStep || kLongStepF32) ? 256 : 128) / Tr::kBytes;
   static constexpr int kPpr = TR / (16 / Tr::kBytes);   // 16-byte pieces per R-contiguous row (8 or 16)
   // swizzle of an R-contiguous direct stage: piece p of row x sits at slot p ^ row_swizzle(x)
   static __device__ __forceinline__ int row_swizzle(int row) { return kPpr == 16 ? (row & 15) : ((row >> 1) & 7); }

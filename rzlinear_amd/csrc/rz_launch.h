@@ -42,7 +42,8 @@ static constexpr int kTargetWorkgroups = 1024;
 // Contracted elements per kernel step that every slice of a cut contraction must be a multiple
 // of: 128 bytes, and 256 for the 16-bit 128 tile, whose eight-wavefront form takes 256-byte steps
 // (a slice that began in the middle of such a step would start between two hashed tiles).
-static inline int slice_unit(int tile, int elem_bytes) {
+static inline int slice_unit(int tile, int elem_bytes, bool weight_grad = false) {
+  if (elem_bytes == 4 && tile <= 64 && !weight_grad) return 64;   // (fp32 forward / input-grad, 64 and 32 x 64 tiles: 256-byte steps as well)
   return ((tile == 128 && elem_bytes == 2) ? 256 : 128) / elem_bytes;
 }
 
@@ -252,7 +253,7 @@ static inline WeightGradPlan plan_weight_grad(int M, int K, int N, int H, int BK
     // a short M cut over many slices leaves a 256 workgroup a step or two between its prologue
     // and its scatter: the 128 tile then has less to set up and to scatter per workgroup
     const long long tiles256 = tile_count(K, N, 256);
-    const int step256 = slice_unit(256, elem_bytes);
+    const int step256 = slice_unit(256, elem_bytes, true);
     const bool cover128 = tile_cover(K, N, 128) * 10 <= tile_cover(K, N, 256) * 13;
     if (pl.tile == 256 && elem_bytes == 4 && tiles256 < kComputeUnits &&
         (long long)((M + step256 - 1) / step256) * tiles256 < 4LL * kComputeUnits && cover128)
@@ -303,7 +304,7 @@ static inline WeightGradPlan plan_weight_grad(int M, int K, int N, int H, int BK
     }
   }
   const long long tiles = (long long)((K + pl.tile - 1) / pl.tile) * ((N + pl.tile - 1) / pl.tile);
-  const int TR = slice_unit(pl.tile, elem_bytes);
+  const int TR = slice_unit(pl.tile, elem_bytes, true);
   const int r_steps = (M + TR - 1) / TR;
   // split the reduction over M when there are too few W tiles to fill the chip
   // (one workgroup per compute unit for the 128 tile too: a second one per compute unit would come
@@ -597,7 +598,7 @@ static inline KernelForm kernel_form(int op, int I, int J, int R, int chunk, int
             : tile == 64 ? ((elem_bytes == 4 && op != kWeightGrad) ? 8 : 4)
                          : (f.stages == 1 ? 4 : (workgroups <= kComputeUnits * 3 / 2 ? 8 : 4));
   const bool direct_capable = elem_bytes == 2 && f.stages == 2 && tile >= 128;
-  const int step_plain = 128 / elem_bytes;
+  const int step_plain = elem_bytes == 4 ? slice_unit(tile, elem_bytes, op == kWeightGrad) : 128 / elem_bytes;
   const int step_direct = (direct_capable && tile == 128 && f.waves == 8) ? 256 / elem_bytes : step_plain;
   f.full = (I % tile == 0) && (J % tile_cols(tile) == 0) && (R % step_direct == 0) && (chunk % step_direct == 0);
   // a plain operand's rows must hold at least one 16-byte piece (a piece that straddles the end of a
