@@ -302,7 +302,7 @@ static hipError_t launch_fold_small(const FoldParams& fp, hipStream_t s) {
   if (fp.partial != nullptr || fp.out == nullptr || fp.shares != 1 || tiles > kFoldSmallTiles ||
       fp.window != kFoldSmallThreads || (long long)fp.windows * fp.window < fp.H)
     return hipErrorInvalidValue;
-  hipLaunchKernelGGL(fold_small_kernel<1>, dim3((unsigned)fp.windows), dim3(kFoldSmallThreads), 0, s, fp);
+  hipLaunchKernelGGL(fold_small_kernel, dim3((unsigned)fp.windows), dim3(kFoldSmallThreads), 0, s, fp);
   return hipGetLastError();
 }
 

@@ -312,17 +312,17 @@ __global__ __launch_bounds__(kFoldThreads) void fold_tiles_kernel(const FoldPara
 // With a few thousand tiles at most, every workgroup can afford to look at every tile offset, and
 // the machinery above (windows in LDS, shares, run lists walked by wavefronts) costs more than it
 // saves: a 1024 x 1024 layer has 256 tiles and a hashed_weight of 65536 elements, and its whole
-// gradient is a few microseconds of reading.  Here a workgroup of 256 threads owns 256 * PER
-// consecutive elements of dHW, thread t the elements t, t + 256, ...; it lists the tiles whose
-// slice meets its elements (ascending tile index: one ballot and two barriers per 1024 tiles) and
-// every thread then walks down the list and adds what each tile holds for its elements — loads of
-// 256 consecutive floats per wavefront-row, fixed order of additions (tile by tile, slice by slice),
+// gradient is a few microseconds of reading.  Here a workgroup of 256 threads owns 256
+// consecutive elements of dHW, one per thread; it lists the tiles whose
+// slice meets its elements (ascending tile index: two barriers per 1024 tiles) and every thread
+// then walks down the list and adds what each tile holds for its element — loads of 64 consecutive
+// floats per wavefront, fixed order of additions (tile by tile, slice by slice),
 // no atomics, every element of dHW written once.
 static constexpr int kFoldSmallThreads = 256;
 static constexpr int kFoldSmallTiles = 4096;   // tiles at most: the list in LDS can hold every one of them
 
-template <int PER>
 __global__ __launch_bounds__(kFoldSmallThreads) void fold_small_kernel(const FoldParams p) {
+  constexpr int PER = 1;   // elements of dHW per thread
   __shared__ int list_id[kFoldSmallTiles];     // tiles that meet this workgroup's elements, ascending
   __shared__ int list_rel[kFoldSmallTiles];    // ... and where each starts, relative to the first element
   __shared__ int wave_count[kFoldSmallThreads / 64];

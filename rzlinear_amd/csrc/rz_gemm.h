@@ -1,7 +1,7 @@
 // One MFMA-tiled kernel template for the three RzLinear contractions on gfx950.
 //
 // A workgroup of WI*WJ wavefronts owns a TI x TJ tile of C and walks the contracted
-// dimension R in steps of TR (128 bytes of R per step).  Per step the A and B tiles are staged
+// dimension R in steps of TR (128 bytes of R per step, 256 for some forms: see TR below).  Per step the A and B tiles are staged
 // in LDS and read from there as MFMA fragments.  The hashed operand (W) is fetched as 16-byte
 // pieces of hashed_weight at off(tk,tn) + kk*BN + nn; the pieces may start at any element, so
 // the loads are unaligned and rely on the hardware's unaligned global access.  Tile offsets
