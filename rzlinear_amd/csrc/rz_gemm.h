@@ -38,6 +38,10 @@
 
 #include "rz_common.h"
 
+#ifndef RZ_F32_DIRECT
+#define RZ_F32_DIRECT 1
+#endif
+
 namespace rz {
 
 enum Layout { kRContig = 0, kRStrided = 1 };
@@ -115,7 +119,14 @@ __device__ __forceinline__ u32x4_t mask_tail(u32x4_t v, int col, int col_lim) {
   return v;
 }
 
-// The 16-bit elements sh .. 7 of a 16-byte piece moved down to positions 0 .. 7 - sh, zeros above (1 <= sh <= 7).
+// The elements sh .. VEC - 1 of a 16-byte piece moved down to positions 0 .. VEC - 1 - sh, zeros above
+// (1 <= sh < VEC; 16-bit: VEC = 8, 32-bit: VEC = 4).
+__device__ __forceinline__ u32x4_t shift_down_32(u32x4_t v, int sh) {
+  u32x4_t r;
+#pragma unroll
+  for (int e = 0; e < 4; e++) r[e] = (e + sh == 1) ? v[1] : (e + sh == 2) ? v[2] : (e + sh == 3) ? v[3] : 0u;
+  return r;
+}
 __device__ __forceinline__ u32x4_t shift_down_16(u32x4_t v, int sh) {
   const uint64_t lo = (uint64_t)v[0] | (uint64_t)v[1] << 32, hi = (uint64_t)v[2] | (uint64_t)v[3] << 32;
   const int bits = sh * 16;
@@ -148,7 +159,6 @@ struct GemmKernel {
   static_assert(!(FULL && CLAMP), "complete tiles need no clamping");
   static_assert(!COLSUM || OP == kWeightGrad, "column sums belong to the weight-grad contraction");
   typedef ElemTraits<T> Tr;
-  typedef typename Mfma<T>::Frag Frag;
   static constexpr int kThreads = 64 * WI * WJ * WK;
   static constexpr int VEC = Tr::kVec;
   static constexpr bool k16 = (Tr::kBytes == 2);
@@ -166,7 +176,15 @@ struct GemmKernel {
   static constexpr int kPpr = TR / (16 / Tr::kBytes);   // 16-byte pieces per R-contiguous row (8 or 16)
   // swizzle of an R-contiguous direct stage: piece p of row x sits at slot p ^ row_swizzle(x)
   static __device__ __forceinline__ int row_swizzle(int row) { return kPpr == 16 ? (row & 15) : ((row >> 1) & 7); }
-  static constexpr int KS = Tr::kMfmaK;
+  // swizzle of an X-contiguous direct stage: the unit of 32 elements u of row r sits at u ^ unit_swizzle(r)
+  // (32-bit: rows r and r + 4, which the two halves of a wavefront read together, land in different banks)
+  static __device__ __forceinline__ int unit_swizzle(int row) { return Tr::kBytes == 2 ? (row & 3) : ((row >> 2) & 1); }
+  static __device__ __forceinline__ int strided_at(int row, int col, int pitch) {
+    return row * pitch + ((((col >> 5) ^ unit_swizzle(row)) << 5) | (col & 31));
+  }
+  static __device__ __forceinline__ u32x4_t shift_down(u32x4_t v, int sh) {
+    return Tr::kBytes == 2 ? shift_down_16(v, sh) : shift_down_32(v, sh);
+  }
   static constexpr int A_LAYOUT = (OP == kWeightGrad) ? kRStrided : kRContig;
   static constexpr int B_LAYOUT = (OP == kInputGrad) ? kRContig : kRStrided;
   static constexpr int WTI = TI / WI, WTJ = TJ / WJ;   // wavefront tile
@@ -174,14 +192,30 @@ struct GemmKernel {
   static_assert(WTI % 32 == 0 && WTJ % 32 == 0, "wavefront tile must be a multiple of 32");
 
   // direct-to-LDS staging (see the head of this file)
-  static constexpr bool kDirect = k16 && (FULL || CLAMP) && NSTAGE == 2 && TI >= 128 && TJ >= 128;
+  static constexpr bool kDirect16 = k16 && (FULL || CLAMP) && NSTAGE == 2 && TI >= 128 && TJ >= 128;
+  // fp32, complete tiles: the same staging; a "sub-step" is then eight elements of R (four MFMAs per
+  // pair of blocks), and a fragment holds a lane's four values of it
+  static constexpr bool kDirect32 = !k16 && RZ_F32_DIRECT && (FULL || CLAMP) && NSTAGE == 2 && TJ >= 64;
+  static constexpr bool kDirect = kDirect16 || kDirect32;
+  static constexpr int KS = kDirect32 ? 8 : Tr::kMfmaK;
+  typedef typename std::conditional<kDirect32, f32x4_t, typename Mfma<T>::Frag>::type Frag;
+  static __device__ __forceinline__ f32x16_t mma(Frag a, Frag b, f32x16_t c) {
+    if constexpr (kDirect32) {
+#pragma unroll
+      for (int j = 0; j < 4; j++) c = __builtin_amdgcn_mfma_f32_32x32x2f32(a[j], b[j], c, 0, 0, 0);
+      return c;
+    } else {
+      return Mfma<T>::run(a, b, c);
+    }
+  }
 
   template <int LAYOUT, int TX> struct Lds {
     static constexpr int kPitch = kDirect ? (LAYOUT == kRContig ? TR : TX)
                                   : k16   ? (LAYOUT == kRContig ? TR + 8 : TX + 32)
                                           : (LAYOUT == kRContig ? TX + 1 : TX + 4);
-    static constexpr int kRows = (k16 && LAYOUT == kRContig) ? TX : TR;
+    static constexpr int kRows = ((k16 || kDirect) && LAYOUT == kRContig) ? TX : TR;
     static constexpr int kElems = ((kPitch * kRows + 7) / 8) * 8;
+    static_assert(!kDirect32 || LAYOUT == kRContig || (TX >= 64 && TX <= 256), "a direct load instruction fills whole rows of two or more 128-byte units");
     // source tile as seen by the global loads
     static constexpr int kSrcRows = (LAYOUT == kRContig) ? TX : TR;
     static constexpr int kSrcCols = (LAYOUT == kRContig) ? TR : TX;
@@ -230,7 +264,24 @@ struct GemmKernel {
   // ---- MFMA fragment of the 32-wide block starting at x_base, R sub-step ks ------------------
   template <int LAYOUT, typename L>
   static __device__ __forceinline__ Frag lds_frag(const T* lds, int x_base, int ks, int lane) {
-    if constexpr (!k16) {
+    if constexpr (kDirect32) {
+      // sub-step ks = elements 8 ks .. 8 ks + 7 of the R step; MFMA j of the sub-step contracts
+      // elements 8 ks + j and 8 ks + 4 + j (the lower and the upper half of the wavefront): any
+      // pairing does, as long as both operands use the same one, and this one makes a lane's four
+      // values one 16-byte piece where R is contiguous
+      const float* f = reinterpret_cast<const float*>(lds);
+      if constexpr (LAYOUT == kRContig) {
+        const int row = x_base + (lane & 31), piece = ks * 2 + (lane >> 5);
+        return *reinterpret_cast<const f32x4_t*>(f + row * L::kPitch + ((piece ^ row_swizzle(row)) << 2));
+      } else {
+        // rows 8 ks + 4 h .. + 3 (h = lane / 32), 32 consecutive columns: the 128-byte unit u of row r
+        // sits at u ^ ((r >> 2) & 1), so that the two halves of the wavefront read different banks
+        const int col = x_base + (lane & 31), row = ks * 8 + (lane >> 5) * 4;
+        const float* at = f + strided_at(row, col, L::kPitch);
+        f32x4_t v = {at[0], at[L::kPitch], at[2 * L::kPitch], at[3 * L::kPitch]};
+        return v;
+      }
+    } else if constexpr (!k16) {
       return reinterpret_cast<const float*>(lds)[(ks * 2 + (lane >> 5)) * L::kPitch + x_base +
                                                  (lane & 31)];
     } else if constexpr (LAYOUT == kRContig) {
@@ -242,8 +293,7 @@ struct GemmKernel {
       const int g = lane >> 4, jl = lane & 15;
       const int row = ks * 16 + 8 * (g >> 1) + (jl >> 2), col = x_base + 16 * (g & 1) + 4 * (jl & 3);
       // (row + 4 has the same swizzle as row, so the second read is one pitch-multiple further)
-      const T* p = kDirect ? lds + row * L::kPitch + ((((col >> 5) ^ (row & 3)) << 5) | (col & 31))
-                           : lds + row * L::kPitch + col;
+      const T* p = kDirect ? lds + strided_at(row, col, L::kPitch) : lds + row * L::kPitch + col;
       typedef s16x4_t __attribute__((address_space(3))) * lds_s16x4_ptr;
       const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(p));
       const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(p + 4 * L::kPitch));
@@ -493,18 +543,18 @@ struct GemmKernel {
       }
     };
     // Direct staging: the same sums out of the dY tile in LDS stage `st`.  Thread (g, c) =
-    // (tid / kCpr, tid % kCpr) adds rows g, g + groups, ... of the 16-byte column position c;
-    // the rows are a multiple of four apart, so they share one swizzle.
+    // (tid / kCpr, tid % kCpr) adds rows g, g + groups, ... of the 16-byte column position c
+    // (16-bit: the rows are a multiple of four apart, so they share one swizzle).
     auto colsum_from_stage = [&](int st) {
       constexpr int kGroups = kThreads / LB::kCpr;
-      static_assert(!(COLSUM && kDirect) || (kGroups % 4 == 0 && TR % kGroups == 0), "rows must share a swizzle");
+      static_assert(!(COLSUM && kDirect) || (TR % kGroups == 0 && (!k16 || kGroups % 4 == 0)), "rows must share a swizzle");
       if (colsum_turn == ti) {
         const int g = tid / LB::kCpr, c = tid % LB::kCpr;
-        const int slot = (((c >> 2) ^ (g & 3)) << 2) | (c & 3);
 #pragma unroll
         for (int i = 0; i < TR / kGroups; i++) {
+          const int row = g + i * kGroups;
           T elems[VEC];
-          __builtin_memcpy(elems, sm.b[st] + (g + i * kGroups) * LB::kPitch + slot * VEC, 16);
+          __builtin_memcpy(elems, sm.b[st] + strided_at(row, c * VEC, LB::kPitch), 16);
 #pragma unroll
           for (int e = 0; e < VEC; e++) colsum[e] += Tr::to_float(elems[e]);
         }
@@ -520,12 +570,13 @@ struct GemmKernel {
       const int n = wave * LL::kPieces + q;
       if (layout == kRContig) {
         row = n * (64 / kPpr) + lane / kPpr;
-        col = ((lane % kPpr) ^ row_swizzle(row)) * 8;
+        col = ((lane % kPpr) ^ row_swizzle(row)) * VEC;
       } else {
-        constexpr int kSlots = LL::kPitch / 8;          // 16-byte slots per row
+        constexpr int kSlots = LL::kPitch / VEC;        // 16-byte slots per row
         row = n * (64 / kSlots) + lane / kSlots;
         const int slot = lane % kSlots;
-        col = (((slot >> 2) ^ (row & 3)) << 5) | ((slot & 3) << 3);
+        constexpr int kPpu = 32 / VEC;                  // 16-byte slots per unit of 32 elements
+        col = (((slot / kPpu) ^ unit_swizzle(row)) << 5) | ((slot % kPpu) * VEC);
       }
     };
     auto direct_load = [&](const T* src, const T* stage, int q, int pieces) {
@@ -699,23 +750,22 @@ struct GemmKernel {
                 const int row = first - 1;
                 u32x4_t v;
                 __builtin_memcpy(&v, g + (int64_t)(p.R - 1) * ld + (ext - VEC), 16);
-                *reinterpret_cast<u32x4_t*>(stage + row * LL::kPitch + ((((c >> 5) ^ (row & 3)) << 5) | (c & 31))) =
-                    shift_down_16(v, VEC - rag_x);
+                *reinterpret_cast<u32x4_t*>(stage + strided_at(row, c, LL::kPitch)) = shift_down(v, VEC - rag_x);
               }
             } else {
               const int pieces = tail / VEC, first = TR / VEC - pieces;
               for (int i = tid; i < LL::kRows * pieces; i += kThreads) {
                 const int row = i / pieces, pz = first + i % pieces;
-                *reinterpret_cast<u32x4_t*>(stage + row * LL::kPitch + ((pz ^ row_swizzle(row)) << 3)) = z;
+                *reinterpret_cast<u32x4_t*>(stage + row * LL::kPitch + (pz ^ row_swizzle(row)) * VEC) = z;
               }
               if (rag_r) {
                 const int pz = first - 1;   // the piece that straddles R
                 for (int row = tid; row < LL::kRows; row += kThreads) {
-                  u32x4_t* at = reinterpret_cast<u32x4_t*>(stage + row * LL::kPitch + ((pz ^ row_swizzle(row)) << 3));
+                  u32x4_t* at = reinterpret_cast<u32x4_t*>(stage + row * LL::kPitch + (pz ^ row_swizzle(row)) * VEC);
                   u32x4_t v;
                   if (plain && x0 + row >= ext - 1) {   // the operand's last row, and the rows beyond that repeat it
                     __builtin_memcpy(&v, g + (int64_t)(ext - 1) * ld + (p.R - VEC), 16);
-                    v = shift_down_16(v, VEC - rag_r);
+                    v = shift_down(v, VEC - rag_r);
                   } else {
                     v = mask_tail<T>(*at, 0, rag_r);
                   }
@@ -750,7 +800,7 @@ struct GemmKernel {
         for (int a = 0; a < MI; a++)
 #pragma unroll
           for (int b = 0; b < MJ; b++)
-            acc[a][b] = Mfma<T>::run(fa[ks & 1][a], fb[ks & 1][b], acc[a][b]);
+            acc[a][b] = mma(fa[ks & 1][a], fb[ks & 1][b], acc[a][b]);
         // scheduling hint: spread the LDS reads of the next sub-step between this sub-step's
         // MFMAs (one read after each MFMA), so that their latency hides behind matrix work
         constexpr int kReads = (k16 && A_LAYOUT == kRStrided ? 2 : 1) * MI +
@@ -827,7 +877,7 @@ struct GemmKernel {
 #pragma unroll
         for (int a = 0; a < MI; a++)
 #pragma unroll
-          for (int b = 0; b < MJ; b++) acc[a][b] = Mfma<T>::run(fa[buf][a], fb[buf][b], acc[a][b]);
+          for (int b = 0; b < MJ; b++) acc[a][b] = mma(fa[buf][a], fb[buf][b], acc[a][b]);
       };
       // one R step; the flags say which of the side jobs still exist near the end of the loop
       // `late` staggers the side jobs of the two wavefronts that share a SIMD: one does them

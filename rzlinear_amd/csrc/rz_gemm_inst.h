@@ -66,8 +66,9 @@ static hipError_t launch_one(GemmParams p, const WeightGradPlan* plan, const Spl
 }
 
 // FULL kernels carry no bounds checks: every tile and every R step must be complete.  Ragged
-// shapes: 16-bit tiles can still be staged directly, with edge pieces fetched from inside the
-// operands (CLAMP); everything else takes the bounds-checked kernel.
+// shapes: the directly staged forms (16-bit tiles of 128 and more, all two-stage fp32 forms) still
+// stage directly, with edge pieces fetched from inside the operands (CLAMP); everything else takes
+// the bounds-checked kernel.
 template <typename T, int OP, int TILE, int WI, int WJ, int NSTAGE, bool COLSUM = false, int WK = 1, int TILE_J = TILE>
 static hipError_t launch_tile(GemmParams p, const WeightGradPlan* plan, const SplitPlan* split,
                               const KernelForm& form, hipStream_t stream) {
@@ -77,10 +78,10 @@ static hipError_t launch_tile(GemmParams p, const WeightGradPlan* plan, const Sp
     if (form.step != GemmKernel<T, OP, TILE, TILE_J, WI, WJ, NSTAGE, true>::TR) return hipErrorInvalidValue;
     return launch_one<T, OP, TILE, TILE_J, WI, WJ, NSTAGE, true, COLSUM, false, WK>(p, plan, split, stream);
   }
-  if constexpr (sizeof(T) == 2 && NSTAGE == 2 && TILE >= 128) {
+  if constexpr (NSTAGE == 2 && (sizeof(T) == 4 || TILE >= 128)) {
     if (form.clamp) {
-      if (form.step != GemmKernel<T, OP, TILE, TILE_J, WI, WJ, NSTAGE, false, false, true>::TR) return hipErrorInvalidValue;
-      return launch_one<T, OP, TILE, TILE_J, WI, WJ, NSTAGE, false, COLSUM, true>(p, plan, split, stream);
+      if (form.step != GemmKernel<T, OP, TILE, TILE_J, WI, WJ, NSTAGE, false, false, true, WK>::TR) return hipErrorInvalidValue;
+      return launch_one<T, OP, TILE, TILE_J, WI, WJ, NSTAGE, false, COLSUM, true, WK>(p, plan, split, stream);
     }
   }
   if (form.clamp || form.step != GemmKernel<T, OP, TILE, TILE_J, WI, WJ, NSTAGE, false>::TR) return hipErrorInvalidValue;

@@ -98,8 +98,14 @@ static inline double tile_score(int I, int J, int t, int elem_bytes) {
 
 // Relative throughput of `wgs` workgroups of tile t (see tile_score_full, which this restates for
 // a workgroup count that includes the slices of a cut contraction).
-static inline double tile_rate(double wgs, int t, int elem_bytes, double lo64_f32 = 0.60) {
+static inline double tile_rate(double wgs, int t, int elem_bytes, double lo64_f32 = 0.60, bool store_f32 = false) {
   const bool f32 = elem_bytes == 4;
+  if (f32 && store_f32) {
+    // fp32 forward / input-grad, staged directly: every tile runs the MFMA pipe at the 256 tile's rate
+    // once its loop is under way, at one workgroup per compute unit already (eight wavefronts); what a
+    // smaller tile costs is the longer fill and drain per workgroup, which plan_split prices per slice.
+    return occupancy_rate(wgs, t == 256 ? 1 : (t == 32 ? 4 : 2), 1.0, 1.0);
+  }
   // (32 x 64, four wavefronts: half a 64 workgroup's work in about its time, up to eight resident)
   if (t == 32) return occupancy_rate(wgs, 8, 0.40, 0.80);
   const int slots = (t == 256) ? 1 : (t == 128 ? 2 : 4);
@@ -250,13 +256,15 @@ static inline WeightGradPlan plan_weight_grad(int M, int K, int N, int H, int BK
     pl.tile = 64;
     if (tile_cover(K, N, 128) * 10 <= tile_cover(K, N, 64) * 13) pl.tile = 128;
     if (tile_cover(K, N, 256) * 10 <= tile_cover(K, N, pl.tile) * 13) pl.tile = 256;
-    // a short M cut over many slices leaves a 256 workgroup a step or two between its prologue
+    // a short M cut over many slices leaves a 256 workgroup a few steps between its prologue
     // and its scatter: the 128 tile then has less to set up and to scatter per workgroup
+    // (fp32, M = 2048, K = N = 1024: 53.0 -> 47.5 us; M = 512, K = N = 2048: 51.8 -> 48.4 us; 2048^3 and
+    //  M = 16384, K = 512, N = 1024 stay with the 256 tile: 135.8 against 138.8 us, 137 either way)
     const long long tiles256 = tile_count(K, N, 256);
     const int step256 = slice_unit(256, elem_bytes, true);
     const bool cover128 = tile_cover(K, N, 128) * 10 <= tile_cover(K, N, 256) * 13;
     if (pl.tile == 256 && elem_bytes == 4 && tiles256 < kComputeUnits &&
-        (long long)((M + step256 - 1) / step256) * tiles256 < 4LL * kComputeUnits && cover128)
+        (long long)((M + step256 - 1) / step256) * tiles256 < 16LL * kComputeUnits && cover128)
       pl.tile = 128;
     // (two 128 workgroups fit a compute unit only while two images fit its LDS: K = N = 10240, M = 2048,
     //  H = 36000: 3849 us against 3583 us with the 256 tile)
@@ -531,7 +539,7 @@ struct SplitPlan {
 static inline SplitPlan plan_split(int I, int J, int R, int elem_bytes, const rz_tuning& t) {
   SplitPlan best = {};
   double best_us = 0.0;
-  const double peak = elem_bytes == 4 ? 137e6 : 1150e6;   // flop per microsecond of the 256 tile on a full chip
+  const double peak = elem_bytes == 4 ? 149e6 : 1150e6;   // flop per microsecond of the 256 tile on a full chip
   const int tiles_of[4] = {256, 128, 64, 32};
   // (an override that asks for the 32 x 64 tile where it does not exist gets the 64 tile)
   const int forced = (t.tile == 32 && elem_bytes != 4) ? 64 : t.tile;
@@ -544,21 +552,31 @@ static inline SplitPlan plan_split(int I, int J, int R, int elem_bytes, const rz
     const long long tiles = tile_count(I, J, tile);
     const int r_steps = (R + TR - 1) / TR;
     const double useful = (double)I * (double)J / ((double)tiles * tile * tile_cols(tile));
-    // (the fp32 64 tile of forward / input-grad, eight wavefronts: 0.67 of the 256 tile's rate with one
-    //  workgroup per compute unit when no tile or step is partial — K = 2048, N = 8192, M = 128: 45 us
-    //  whole against 52 us with the 128 tile cut in four; the bounds-checked form stays at 0.60)
+    // fp32 staged directly (complete tiles, or ragged ones with rows of 16 bytes and more): see tile_rate;
+    // a workgroup's fill and drain cost about 2, 8 and 12 steps of 128 bytes for the tiles of 256, 128
+    // and 64 / 32 x 64 (4096^3: 941, 986, 1016 us; M = 4096, K = N = 1024: 128 tile 76 us, 64 tile 82 us;
+    // 1024^3: 64 tile 23.8 us, 128 tile cut in four 35 us).  The bounds-checked form, which only shapes
+    // with shorter rows or an override still take, keeps the older pricing.
     const bool whole = I % tile == 0 && J % tile_cols(tile) == 0 && R % TR == 0;
+    const bool direct = elem_bytes == 4 && (whole || (t.clamp != -1 && R * elem_bytes >= 16));
     const double lo64 = whole ? 0.67 : 0.60;
+    const double fill = !direct ? 2.0 : tile == 256 ? 2.0 : tile == 128 ? 8.0 : 12.0;
+    double whole_us = 0.0;
     for (int want = 1; want <= 16; want++) {
       if (want > 1 && t.split == -1) break;
+      // (a kernel of a dozen microseconds is not worth cutting: the second launch and the short loops
+      //  cost what the idle compute units would have gained — fp32, M = 32 and 96, K = N = 1024: 13 us
+      //  whole, 15 us cut in eight or four)
+      if (want > 1 && direct && whole_us <= 16.0) break;
       const int steps_per = (r_steps + want - 1) / want;
       const int slices = (r_steps + steps_per - 1) / steps_per;
       if (slices != want) continue;                           // (the same cut as a smaller `want`)
       if (slices > 1 && steps_per * (TR * elem_bytes / 128) < 4) break;   // slices of a few steps are all fill and drain
       const double steps = (double)steps_per * (TR * elem_bytes / 128);
-      const double rate = peak * tile_rate((double)tiles * slices, tile, elem_bytes, lo64) * useful * steps / (steps + 2.0);
+      const double rate = peak * tile_rate((double)tiles * slices, tile, elem_bytes, lo64, direct) * useful * steps / (steps + fill);
       double us = 2.0 * (double)I * (double)J * (double)R / rate + 4.0;
-      if (slices > 1) us += (2.0 * slices * (double)I * J * 4.0 + (double)I * J * elem_bytes) / 4.0e6 + 4.0;
+      if (slices > 1) us += (2.0 * slices * (double)I * J * 4.0 + (double)I * J * elem_bytes) / 4.0e6 + (direct ? 3.0 : 4.0);
+      else whole_us = us;
       // (near ties go to the larger tile and the fewer slices, which come first)
       if (best.tile == 0 || us < best_us * 0.97) {
         best.tile = tile;
@@ -597,9 +615,10 @@ static inline KernelForm kernel_form(int op, int I, int J, int R, int chunk, int
             : tile == 32 ? 4
             : tile == 64 ? ((elem_bytes == 4 && op != kWeightGrad) ? 8 : 4)
                          : (f.stages == 1 ? 4 : (workgroups <= kComputeUnits * 3 / 2 ? 8 : 4));
-  const bool direct_capable = elem_bytes == 2 && f.stages == 2 && tile >= 128;
+  // (32-bit: every two-stage form stages directly; 16-bit: the tiles of 128 and more)
+  const bool direct_capable = f.stages == 2 && (elem_bytes == 4 || tile >= 128);
   const int step_plain = elem_bytes == 4 ? slice_unit(tile, elem_bytes, op == kWeightGrad) : 128 / elem_bytes;
-  const int step_direct = (direct_capable && tile == 128 && f.waves == 8) ? 256 / elem_bytes : step_plain;
+  const int step_direct = (direct_capable && elem_bytes == 2 && tile == 128 && f.waves == 8) ? 256 / elem_bytes : step_plain;
   f.full = (I % tile == 0) && (J % tile_cols(tile) == 0) && (R % step_direct == 0) && (chunk % step_direct == 0);
   // a plain operand's rows must hold at least one 16-byte piece (a piece that straddles the end of a
   // row is handled in the kernel; a row shorter than a piece is not)

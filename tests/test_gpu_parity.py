@@ -520,12 +520,13 @@ def test_random_shapes_16bit(oracle, shape):
     assert_close(f(dbias), dy64.sum(axis=0), dtype, "dbias")
 
 
-@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=lambda d: str(d).split(".")[-1])
+@pytest.mark.parametrize("dtype", DTYPES, ids=lambda d: str(d).split(".")[-1])
 @pytest.mark.parametrize("shape", [(1100, 1023, 1001, 40000, 32, 64), (1030, 1025, 2047, 300000, 64, 64),
-                                   (512, 1031, 1017, 9000, 64, 64), (300, 9, 15, 3000, 16, 16), (257, 2049, 263, 9000, 64, 64)],
+                                   (512, 1031, 1017, 9000, 64, 64), (300, 9, 15, 3000, 16, 16), (257, 2049, 263, 9000, 64, 64),
+                                   (200, 5, 6, 3000, 16, 16), (4200, 1022, 1026, 16384, 64, 64)],
                          ids=lambda s: "x".join(map(str, s)))
-def test_16_bit_rows_that_are_not_whole_16_byte_pieces(oracle, shape, dtype):
-    """K and N that are not multiples of 8, the operands contiguous (so that every row starts at another
+def test_rows_that_are_not_whole_16_byte_pieces(oracle, shape, dtype):
+    """K and N that are not multiples of 8 (of 4 for fp32), the operands contiguous (so that every row starts at another
     alignment and the last row ends with the allocation's last element): the kernels keep their
     direct-to-LDS path, fetch the piece that straddles a row end as it lies, and put the last row's
     right in LDS; nothing is copied or padded on the way (the reference masks element by element,
