@@ -333,8 +333,12 @@ __global__ __launch_bounds__(kFoldSmallThreads) void fold_small_kernel(const Fol
   const int E = p.h.BK * p.h.BN, eshift = p.h.bk_shift + p.h.bn_shift;
   const int ntiles = p.tiles_k * p.tiles_n;
   const bool plan_ok = p.plan_header == nullptr || layer_plan_matches(p.plan_header, p.K, p.N, p.H, p.h);   // (uniform)
+  // (the offsets are fetched whether or not the header turns out to match — the caller vouches for the plan's
+  //  size, so the reads stay inside it — so that the two fetches travel together; a plan that does not
+  //  match lists nothing)
+  const bool even = p.K % p.h.BK == 0 && p.N % p.h.BN == 0;   // (uniform) every tile lies inside K x N
   int listed = 0;
-  for (int first = 0; first < ntiles && plan_ok; first += 4 * kFoldSmallThreads) {
+  for (int first = 0; first < ntiles; first += 4 * kFoldSmallThreads) {
     // thread t looks at the tiles first + 4 t .. first + 4 t + 3 (ascending over the threads)
     int rel[4];
     unsigned hit = 0u;
@@ -344,7 +348,7 @@ __global__ __launch_bounds__(kFoldSmallThreads) void fold_small_kernel(const Fol
       const int idc = id < ntiles ? id : ntiles - 1;
       // (without a table, the few offsets a thread needs are hashed on the spot)
       rel[u] = (p.offsets != nullptr ? p.offsets[idc] : (int)tile_offset(p.h, (uint32_t)(idc / p.tiles_n), (uint32_t)(idc % p.tiles_n))) - h0;
-      hit |= (unsigned)((id < ntiles) & (rel[u] > -E) & (rel[u] < span)) << u;
+      hit |= (unsigned)((id < ntiles) & (rel[u] > -E) & (rel[u] < span) & plan_ok) << u;
     }
     const int mine = __popc(hit);
     int incl = mine;
@@ -386,10 +390,13 @@ __global__ __launch_bounds__(kFoldSmallThreads) void fold_small_kernel(const Fol
     for (int u = 0; u < kBatch; u++) {
       const int e = e0 + u < listed ? e0 + u : listed - 1;
       const int id = list_id[e], rel = list_rel[e];
-      const int tk = id / p.tiles_n, tn = id - tk * p.tiles_n;
       // rows and columns of the tile inside K x N (what lies beyond was never written)
-      const int rows = (p.K - tk * p.h.BK) < p.h.BK ? (p.K - tk * p.h.BK) : p.h.BK;
-      const int cols = (p.N - tn * p.h.BN) < p.h.BN ? (p.N - tn * p.h.BN) : p.h.BN;
+      int rows = p.h.BK, cols = p.h.BN;
+      if (!even) {
+        const int tk = id / p.tiles_n, tn = id - tk * p.tiles_n;
+        rows = (p.K - tk * p.h.BK) < p.h.BK ? (p.K - tk * p.h.BK) : p.h.BK;
+        cols = (p.N - tn * p.h.BN) < p.h.BN ? (p.N - tn * p.h.BN) : p.h.BN;
+      }
       const bool whole = rows == p.h.BK && cols == p.h.BN;
 #pragma unroll
       for (int j = 0; j < PER; j++) {
