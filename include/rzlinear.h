@@ -79,11 +79,15 @@ typedef struct rz_tuning {
   int lds_image;  /* weight-grad: 0 = automatic, -1 = never sum tiles in an LDS image of dHW */
   int window;     /* weight-grad: 0 = automatic, 1 = dHW by windows whenever possible, -1 = never */
   int split;      /* forward / input-grad: 0 = automatic, -1 = never split the contraction */
-  int clamp;      /* ragged 16-bit shapes: 0 = automatic, -1 = always the bounds-checked kernels */
+  int clamp;      /* ragged shapes: 0 = automatic, -1 = always the bounds-checked kernels */
   int fold;       /* weight-grad with a hashed_weight too large for LDS: 0 = automatic, 1 = X^T.dY stored
                      tile by tile and folded into dHW by a second kernel whenever possible, 2 = the same
                      with the windowed fold kernel even for the few tiles that have a kernel of their own,
                      -1 = never */
+  int fold_tiles; /* weight-grad by the fold, 16-bit layer with a 16-bit dHW: 0 = automatic (X^T.dY is stored tile by
+                     tile in the layer's dtype: half the bytes written and read back; every stored value is
+                     rounded once more than in fp32, the sum over M and the sum of the tiles stay fp32),
+                     -1 = always fp32 tiles */
   int poll_limit; /* weight-grad by windows: 0 = default; > 0 = how often a wavefront looks at the flags of the
                      earlier strips it waits for before it gives up and the window is stored as NaN (a bounded
                      wait; tests set a tiny value to see every wavefront leave the kernel all the same) */
@@ -178,7 +182,10 @@ size_t rz_weight_grad_workspace_bytes(int M, int K, int N, int H, int BK, int BN
  * off(tk,tn); dHW is zeroed and fully overwritten by the call (element type `dtype`).
  * Replaces rz_linear_backward_weight_grad_tl                          impl/RzLinearBackward.py:23-97
  * (kernel rz_linear_backward_weight_grad_core                         impl/RzLinearBackward.py:291-371).
- * Accumulation and the scatter are done in fp32 for every dtype.  The LDS-image, fold and
+ * Accumulation and the scatter are done in fp32 for every dtype (one exception: a 16-bit layer with a
+ * 16-bit dHW on the fold path keeps the complete fp32 sums over M in its own dtype between the two
+ * kernels — one more rounding per stored value, still added up in fp32; see rz_tuning.fold_tiles — where
+ * the reference rounds the running sum at every atomic add).  The LDS-image, fold and
  * window paths add in a fixed order (plain read-add-write in LDS, ordered by barriers, by list
  * order or by flags; partial images are added in index order): the same inputs give the same
  * bits on every call.  Only the global-atomic path (few W tiles and a hashed_weight too large

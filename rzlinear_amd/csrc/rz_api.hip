@@ -297,16 +297,21 @@ static void launch_reduce_partials(int out_dtype, const float* part, void* out, 
     hipLaunchKernelGGL((reduce_partials_kernel<f16_t, ACC, GROUPS>), grid, block, 0, s, part, (f16_t*)out, H, pitch, nparts);
 }
 
-static hipError_t launch_fold_small(const FoldParams& fp, hipStream_t s) {
+// (tile_dtype: what the contraction kernel stored the tiles as — floats, or the layer's 16-bit dtype)
+static hipError_t launch_fold_small(const FoldParams& fp, int tile_dtype, hipStream_t s) {
   const long long tiles = (long long)fp.tiles_k * fp.tiles_n;
   if (fp.partial != nullptr || fp.out == nullptr || fp.shares != 1 || tiles > kFoldSmallTiles ||
       fp.window != kFoldSmallThreads || (long long)fp.windows * fp.window < fp.H)
     return hipErrorInvalidValue;
-  hipLaunchKernelGGL(fold_small_kernel, dim3((unsigned)fp.windows), dim3(kFoldSmallThreads), 0, s, fp);
+  const dim3 grid((unsigned)fp.windows), block(kFoldSmallThreads);
+  if (tile_dtype == RZ_BF16) hipLaunchKernelGGL(fold_small_kernel<bf16_t>, grid, block, 0, s, fp);
+  else if (tile_dtype == RZ_F16) hipLaunchKernelGGL(fold_small_kernel<f16_t>, grid, block, 0, s, fp);
+  else hipLaunchKernelGGL(fold_small_kernel<float>, grid, block, 0, s, fp);
   return hipGetLastError();
 }
 
-static hipError_t launch_fold(const FoldParams& fp, hipStream_t s) {
+template <typename TT>
+static hipError_t launch_fold_as(const FoldParams& fp, hipStream_t s) {
   static std::atomic<uint64_t> raised{0};
   const size_t lds = fold_lds_bytes(fp.window);
   const int E = fp.h.BK * fp.h.BN, runs = E > kFoldRun ? E / kFoldRun : 1;
@@ -314,11 +319,17 @@ static hipError_t launch_fold(const FoldParams& fp, hipStream_t s) {
       fp.slices * runs * 4 > kFoldList || runs > 8 || fp.h.BK > 16384 || fp.h.BN > 16384 || (long long)fp.windows * fp.window < fp.H)
     return hipErrorInvalidValue;
   if (lds > 64 * 1024) {
-    hipError_t e = raise_lds_limit(reinterpret_cast<const void*>(fold_tiles_kernel), raised);
+    hipError_t e = raise_lds_limit(reinterpret_cast<const void*>(fold_tiles_kernel<TT>), raised);
     if (e != hipSuccess) return e;
   }
-  hipLaunchKernelGGL(fold_tiles_kernel, dim3((unsigned)(fp.windows * fp.shares)), dim3(kFoldThreads), lds, s, fp);
+  hipLaunchKernelGGL(fold_tiles_kernel<TT>, dim3((unsigned)(fp.windows * fp.shares)), dim3(kFoldThreads), lds, s, fp);
   return hipGetLastError();
+}
+
+static hipError_t launch_fold(const FoldParams& fp, int tile_dtype, hipStream_t s) {
+  return tile_dtype == RZ_BF16 ? launch_fold_as<bf16_t>(fp, s)
+         : tile_dtype == RZ_F16 ? launch_fold_as<f16_t>(fp, s)
+                                : launch_fold_as<float>(fp, s);
 }
 
 template <bool ACC>
@@ -382,7 +393,8 @@ static int weight_grad_impl(const void* X, const void* dY, void* dHW, void* dbia
   const bool accumulate = (flags & RZ_WG_ACCUMULATE) != 0;
   const int dhw_dtype = (flags & RZ_WG_DHW_F32) ? RZ_F32 : dtype;
   const int dbias_dtype = (flags & RZ_WG_DBIAS_F32) ? RZ_F32 : dtype;
-  const WeightGradPlan plan = plan_weight_grad(M, K, N, H, BK, BN, dtype_bytes(dtype), tuning);
+  const WeightGradPlan plan = plan_weight_grad(M, K, N, H, BK, BN, dtype_bytes(dtype), tuning,
+                                               fold_tile_bytes(dtype_bytes(dtype), dhw_dtype == RZ_F32, tuning));
   // a layer plan (device memory, built for exactly this K, N, H, tile and hash) replaces the
   // per-call hashing of the tile offsets and the window kernel's search for its strips
   const bool planned = layer_plan != nullptr;
@@ -453,6 +465,9 @@ static int weight_grad_impl(const void* X, const void* dY, void* dHW, void* dbia
     const FoldPlan& f = plan.fold;
     p.scatter = nullptr;
     p.tiles_out = (float*)((char*)workspace + kFoldMarginBytes);   // (the fold kernel's loads reach a few floats beyond the tiles)
+    p.tiles_out_16 = f.tile_bytes == 2 ? 1 : 0;
+    if (p.tiles_out_16 && dtype_bytes(dtype) != 2) return RZ_ERR_BAD_ARGUMENT;   // (cannot happen: see fold_tile_bytes)
+    const int tile_dtype = p.tiles_out_16 ? dtype : RZ_F32;
     p.out_tiles_k = (K + BK - 1) / BK;
     p.out_tiles_n = (N + BN - 1) / BN;
     if (launch_gemm(dtype, kWeightGrad, p, &plan, nullptr, tuning, s) != hipSuccess) return RZ_ERR_LAUNCH;
@@ -486,7 +501,7 @@ static int weight_grad_impl(const void* X, const void* dY, void* dHW, void* dbia
     fp.window = f.window;
     fp.windows = f.windows;
     fp.shares = f.shares;
-    if ((f.small ? launch_fold_small(fp, s) : launch_fold(fp, s)) != hipSuccess) return RZ_ERR_LAUNCH;
+    if ((f.small ? launch_fold_small(fp, tile_dtype, s) : launch_fold(fp, tile_dtype, s)) != hipSuccess) return RZ_ERR_LAUNCH;
     if (f.shares > 1) {
       if (accumulate) launch_reduce_partials<true>(dhw_dtype, fp.partial, dHW, H, fp.pitch, f.shares, s);
       else launch_reduce_partials<false>(dhw_dtype, fp.partial, dHW, H, fp.pitch, f.shares, s);
@@ -767,8 +782,8 @@ RZ_API size_t rz_weight_grad_hashed_workspace_bytes(int M, int K, int N, int H, 
   const rz_tuning t = tuning_or_default(tuning);
   if (eb == 0 || M < 1 || K < 1 || N < 1 || H < 1 || !tuning_valid(t)) return 0;
   if (check_tile(BK, BN) != RZ_OK) return 0;
-  const WeightGradPlan plan = plan_weight_grad(M, K, N, H, BK, BN, eb, t);
   const bool dhw_f32 = (flags & RZ_WG_DHW_F32) != 0 || dtype == RZ_F32;
+  const WeightGradPlan plan = plan_weight_grad(M, K, N, H, BK, BN, eb, t, fold_tile_bytes(eb, dhw_f32, t));
   WindowPlan wp = {};
   if (!plan.lds_image()) wp = plan_window(M, K, N, H, BK, BN, eb, t, plan);
   return weight_grad_workspace(plan, wp, H, dhw_f32, with_dbias != 0).total_bytes;
@@ -891,7 +906,8 @@ RZ_API int rz_plan_query(int op, int M, int K, int N, int H, int BK, int BN, int
   if (st != RZ_OK) return st;
   for (int i = 0; i < 8; i++) out[i] = 0;
   if (op == kWeightGrad) {
-    const WeightGradPlan plan = plan_weight_grad(M, K, N, H, BK, BN, eb, t);
+    const bool dhw_f32 = (flags & RZ_WG_DHW_F32) != 0 || dtype == RZ_F32;
+    const WeightGradPlan plan = plan_weight_grad(M, K, N, H, BK, BN, eb, t, fold_tile_bytes(eb, dhw_f32, t));
     WindowPlan wp = {};
     if (!plan.lds_image())
       wp = plan_window(M, K, N, H, BK, BN, eb, t, plan, planned && layer_plan_layout(K, N, H, BK, BN).windows > 0);

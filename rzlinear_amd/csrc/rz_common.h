@@ -109,6 +109,7 @@ struct GemmParams {
                       // hashed tile by hashed tile, tile (tk, tn) of slice s as BK*BN contiguous floats
                       // at ((s * tiles_k + tk) * tiles_n + tn) * BK*BN (only the part inside K x N is defined), and a
                       // second kernel folds the tiles into dHW
+  int tiles_out_16;   // ... as elements of the layer's 16-bit dtype instead of floats (same element indices)
   int out_tiles_k, out_tiles_n;   // ... its tile grid: ceil(K / BK) x ceil(N / BN)
   float* colsum;      // weight-grad that also yields the bias gradient: partial column sums of B
                       // (dY), one row per (slice, tile row): [slices * tiles_i][colsum_pitch]

@@ -38,7 +38,7 @@
 namespace rz {
 
 struct FoldParams {
-  const float* tiles;   // [slices][tiles_k * tiles_n][BK * BN]
+  const void* tiles;    // [slices][tiles_k * tiles_n][BK * BN], floats or elements of a 16-bit dtype (the kernels' TT)
   const int32_t* offsets;   // [tiles_k * tiles_n] where every tile starts in hashed_weight (hashed once, by another kernel;
                             // null for the few-tiles kernel: it hashes them itself)
   const int32_t* plan_header;   // `offsets` belongs to a layer plan (else null): its header, checked against this call's
@@ -68,7 +68,30 @@ static inline size_t fold_lds_bytes(int window) {
 
 typedef float fold_f4 __attribute__((ext_vector_type(4)));
 typedef float fold_f4u __attribute__((ext_vector_type(4), aligned(4)));
+typedef uint16_t fold_h4 __attribute__((ext_vector_type(4)));
+typedef uint16_t fold_h4u __attribute__((ext_vector_type(4), aligned(2)));
 
+// Four consecutive tile elements as they lie in memory (TT = float, bf16_t or f16_t), and as floats.
+template <typename TT> struct FoldRaw { typedef fold_h4 type; typedef fold_h4u unaligned; };
+template <> struct FoldRaw<float> { typedef fold_f4 type; typedef fold_f4u unaligned; };
+template <typename TT>
+__device__ __forceinline__ fold_f4 fold_widen(typename FoldRaw<TT>::type raw) {
+  if constexpr (sizeof(TT) == 4) {
+    return raw;
+  } else {
+    fold_f4 v;
+#pragma unroll
+    for (int f = 0; f < 4; f++) {
+      TT e;
+      const uint16_t bits = raw[f];
+      __builtin_memcpy(&e, &bits, 2);
+      v[f] = ElemTraits<TT>::to_float(e);
+    }
+    return v;
+  }
+}
+
+template <typename TT>
 __global__ __launch_bounds__(kFoldThreads) void fold_tiles_kernel(const FoldParams p) {
   extern __shared__ __align__(16) float fold_lds[];
   float* img = fold_lds;
@@ -200,7 +223,7 @@ __global__ __launch_bounds__(kFoldThreads) void fold_tiles_kernel(const FoldPara
       // the next round's loads are in flight while this round's values are added.  What describes
       // an entry to the wavefront is uniform (scalar registers).
       struct Round {
-        fold_f4 v[kFoldRound];
+        typename FoldRaw<TT>::type v[kFoldRound];   // (as loaded: widened when added, so that the loads stay in flight)
         int pos[kFoldRound];   // window position of the block
         int e0[kFoldRound];    // float of the run that falls on the block's first position (-255 .. run - 1)
         int lim[kFoldRound];   // the entry's, -1: no entry
@@ -237,7 +260,7 @@ __global__ __launch_bounds__(kFoldThreads) void fold_tiles_kernel(const FoldPara
           //  loads their number is fixed, and the wait for this round's values can leave the next
           //  round's in flight)
           const long long first = any ? (long long)off : 0ll;
-          unsigned mine = lane16;   // byte offset of the lane's four floats from the block's first
+          unsigned mine = lane16;   // offset of the lane's four elements from the block's first, in bytes of floats
           if (any && (r.e0[u] < 0 || r.e0[u] + kFoldBlock > run)) {   // (uniform) an end of the run:
             // lanes that lie wholly outside the run fetch floats of the run that other lanes fetch
             // anyway (their values count as zero below) instead of a neighbouring tile's
@@ -247,8 +270,8 @@ __global__ __launch_bounds__(kFoldThreads) void fold_tiles_kernel(const FoldPara
           }
           // (read once and never again: a load that leaves the caches to the offsets and to the
           //  contraction's stores still on their way to memory — K = N = 10240: 129 -> 111 us)
-          r.v[u] = __builtin_nontemporal_load(
-              reinterpret_cast<const fold_f4u*>(reinterpret_cast<const char*>(p.tiles) + first * 4 + mine));
+          r.v[u] = __builtin_nontemporal_load(reinterpret_cast<const typename FoldRaw<TT>::unaligned*>(
+              reinterpret_cast<const char*>(p.tiles) + (first * 4 + mine) / (4 / (int)sizeof(TT))));
         }
       };
       // (plain read-add-write: LDS float atomics are several times slower, and nobody else touches
@@ -257,7 +280,7 @@ __global__ __launch_bounds__(kFoldThreads) void fold_tiles_kernel(const FoldPara
   #pragma unroll
         for (int u = 0; u < kFoldRound; u++) {
           if (r.lim[u] == -1) continue;   // (uniform)
-          fold_f4 v = r.v[u];
+          fold_f4 v = fold_widen<TT>(r.v[u]);
           const int lim = r.lim[u];
           if (r.e0[u] < 0 || r.e0[u] + kFoldBlock > run || (lim & 0x0fffffff) != full_lim) {
             // an end of the run, or a tile that sticks out of K x N: what is not the run's counts as zero
@@ -321,6 +344,7 @@ __global__ __launch_bounds__(kFoldThreads) void fold_tiles_kernel(const FoldPara
 static constexpr int kFoldSmallThreads = 256;
 static constexpr int kFoldSmallTiles = 4096;   // tiles at most: the list in LDS can hold every one of them
 
+template <typename TT>
 __global__ __launch_bounds__(kFoldSmallThreads) void fold_small_kernel(const FoldParams p) {
   constexpr int PER = 1;   // elements of dHW per thread
   __shared__ int list_id[kFoldSmallTiles];     // tiles that meet this workgroup's elements, ascending
@@ -407,8 +431,8 @@ __global__ __launch_bounds__(kFoldSmallThreads) void fold_small_kernel(const Fol
       }
     }
     for (int sl = 0; sl < p.slices; sl++) {
-      const float* base = p.tiles + (((size_t)sl * ntiles) << eshift);
-      float v[kBatch][PER];
+      const TT* base = reinterpret_cast<const TT*>(p.tiles) + (((size_t)sl * ntiles) << eshift);
+      TT v[kBatch][PER];
 #pragma unroll
       for (int u = 0; u < kBatch; u++)
 #pragma unroll
@@ -416,7 +440,7 @@ __global__ __launch_bounds__(kFoldSmallThreads) void fold_small_kernel(const Fol
 #pragma unroll
       for (int u = 0; u < kBatch; u++)
 #pragma unroll
-        for (int j = 0; j < PER; j++) acc[j] += ok[u][j] ? v[u][j] : 0.f;
+        for (int j = 0; j < PER; j++) acc[j] += ok[u][j] ? ElemTraits<TT>::to_float(v[u][j]) : 0.f;
     }
   }
 #pragma unroll

@@ -997,7 +997,10 @@ struct GemmKernel {
       __syncthreads();
       // No scatter: the accumulators are stored plainly, hashed tile by hashed tile (whole tiles:
       // zeros where a tile reaches beyond K x N); the fold kernel adds the tiles into dHW.
-      auto store_tiles = [&]() {
+      auto store_tiles = [&](auto narrow) {
+        // (narrow: the tiles are kept in the layer's 16-bit dtype — each value rounded once here, added up in fp32 by the fold)
+        constexpr bool kNarrow = decltype(narrow)::value;
+        T* const out16 = reinterpret_cast<T*>(p.tiles_out);
 #pragma unroll
         for (int a = 0; a < MI; a++)
 #pragma unroll
@@ -1014,8 +1017,12 @@ struct GemmKernel {
             for (int e = 0; e < 16; e++) {
               const int k = i0 + blk_i(a) + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
               const bool inside = FULL || (k < p.I && n < p.J);
-              if (FULL || base[e >> 2] >= 0)
-                p.tiles_out[(uint32_t)(base[e >> 2] + (e & 3) * p.h.BN)] = inside ? acc[a][b][e] * p.scale : 0.f;
+              if (FULL || base[e >> 2] >= 0) {
+                const float v = inside ? acc[a][b][e] * p.scale : 0.f;
+                const uint32_t at = (uint32_t)(base[e >> 2] + (e & 3) * p.h.BN);
+                if constexpr (kNarrow) out16[at] = Tr::from_float(v);
+                else p.tiles_out[at] = v;
+              }
             }
           }
       };
@@ -1048,7 +1055,8 @@ struct GemmKernel {
           }
       };
       if (tiled) {
-        store_tiles();
+        if (sizeof(T) == 2 && p.tiles_out_16) store_tiles(std::true_type{});   // (uniform)
+        else store_tiles(std::false_type{});
       } else if (image_mode) {
         // Tiles of one workgroup overlap in hashed_weight: sum them in an LDS image of dHW
         // first, then store the image as this workgroup's partial result.

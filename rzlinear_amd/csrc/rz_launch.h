@@ -19,7 +19,7 @@ static inline bool tuning_valid(const rz_tuning& t) {
   return (t.tile == 0 || t.tile == 32 || t.tile == 64 || t.tile == 128 || t.tile == 256) && (t.stages == 0 || t.stages == 1) &&
          (t.lds_image == 0 || t.lds_image == -1) && (t.window >= -1 && t.window <= 1) &&
          (t.split == 0 || t.split == -1) && (t.clamp == 0 || t.clamp == -1) &&
-         (t.fold >= -1 && t.fold <= 2) && t.poll_limit >= 0;
+         (t.fold >= -1 && t.fold <= 2) && (t.fold_tiles == 0 || t.fold_tiles == -1) && t.poll_limit >= 0;
 }
 
 // Kernels that use more than the default 64 KB of LDS need their limit raised once per kernel
@@ -142,13 +142,24 @@ struct FoldPlan {
   int small;             // few tiles: the kernel whose workgroups each look at every tile (no windows in LDS, no shares)
   int window, windows;   // floats per window (a multiple of 1024, at most 32768) and their number
   int shares;            // workgroups per window, each with an equal part of the window's tiles and an image of its own
-  size_t tiles_bytes;    // the tile-by-tile X^T.dY: slices * tiles * BK*BN floats, with a margin before and after
+  int tile_bytes;        // bytes of a stored element of X^T.dY: 4, or 2 (the layer's 16-bit dtype, see fold_tile_bytes)
+  size_t tiles_bytes;    // the tile-by-tile X^T.dY: slices * tiles * BK*BN elements, with a margin before and after
   size_t partial_bytes;  // shares images of dHW (none with a single share: the fold kernel writes dHW)
   size_t offsets_bytes;  // where every tile starts in hashed_weight, one int32 per tile
 };
 
-static inline FoldPlan plan_fold(int K, int N, int H, int BK, int BN, int slices, bool windowed = false) {
+// What the contraction kernel stores the tiles of X^T.dY as for the fold: floats — or, when the layer
+// and its dHW are both 16-bit, the layer's dtype: the sum over M is complete (fp32) by then and the
+// fold adds the stored values up in fp32 again, so this costs one more rounding per stored value (the
+// reference rounds the running sum at every atomic add, RzLinearBackward.py:364-371) and halves the
+// bytes written and read back, which is what the fold costs.
+static inline int fold_tile_bytes(int elem_bytes, bool dhw_f32, const rz_tuning& t) {
+  return (elem_bytes == 2 && !dhw_f32 && t.fold_tiles != -1) ? 2 : 4;
+}
+
+static inline FoldPlan plan_fold(int K, int N, int H, int BK, int BN, int slices, bool windowed = false, int tile_bytes = 4) {
   FoldPlan f = {};
+  f.tile_bytes = tile_bytes;
   const long long E = (long long)BK * BN;
   const long long tiles = (long long)((K + BK - 1) / BK) * ((N + BN - 1) / BN);
   // (element indices of the buffer are 32-bit in the kernels; the fold lists slices entries per tile)
@@ -163,7 +174,7 @@ static inline FoldPlan plan_fold(int K, int N, int H, int BK, int BN, int slices
     f.window = 256;
     f.windows = (H + f.window - 1) / f.window;
     f.shares = 1;
-    f.tiles_bytes = (((size_t)slices * tiles * E * sizeof(float) + 255) & ~(size_t)255) + 2 * kFoldMarginBytes;
+    f.tiles_bytes = (((size_t)slices * tiles * E * (size_t)tile_bytes + 255) & ~(size_t)255) + 2 * kFoldMarginBytes;
     f.partial_bytes = 0;
     f.offsets_bytes = ((size_t)tiles * sizeof(int32_t) + 255) & ~(size_t)255;
     f.use = 1;
@@ -180,7 +191,7 @@ static inline FoldPlan plan_fold(int K, int N, int H, int BK, int BN, int slices
   if (shares > slices * tiles / 8) shares = slices * tiles / 8;   // a share is worth a workgroup from some tiles on
   if (shares < 1) shares = 1;
   f.shares = (int)shares;
-  f.tiles_bytes = (((size_t)slices * tiles * E * sizeof(float) + 255) & ~(size_t)255) + 2 * kFoldMarginBytes;
+  f.tiles_bytes = (((size_t)slices * tiles * E * (size_t)tile_bytes + 255) & ~(size_t)255) + 2 * kFoldMarginBytes;
   const size_t pitch = (size_t)((H + 3) & ~3);
   f.partial_bytes = f.shares > 1 ? ((size_t)f.shares * pitch * sizeof(float) + 255) & ~(size_t)255 : 0;
   f.offsets_bytes = ((size_t)tiles * sizeof(int32_t) + 255) & ~(size_t)255;
@@ -244,7 +255,7 @@ static inline double filled_128(long long tiles) {
 static constexpr double kPairRate128F32 = 0.955;
 
 static inline WeightGradPlan plan_weight_grad(int M, int K, int N, int H, int BK, int BN, int elem_bytes,
-                                              const rz_tuning& t) {
+                                              const rz_tuning& t, int tile_bytes = 4) {
   WeightGradPlan pl;
   const int pitch = (H + 3) & ~3;
   const bool image = t.lds_image != -1 && (size_t)pitch * sizeof(float) <= kMaxImageBytes;
@@ -350,7 +361,7 @@ static inline WeightGradPlan plan_weight_grad(int M, int K, int N, int H, int BK
   pl.fold = FoldPlan{};
   pl.fold_us = 0.0;
   if (!image && t.fold != -1) {
-    const FoldPlan f = plan_fold(K, N, H, BK, BN, pl.splits, t.fold == 2);
+    const FoldPlan f = plan_fold(K, N, H, BK, BN, pl.splits, t.fold == 2, tile_bytes);
     if (f.use) {
       // what the two ways cost beyond the contraction itself, in microseconds: the part of the
       // K*N global atomics per slice that the contraction does not hide (2.8 to 5.2 ps each,
@@ -358,19 +369,19 @@ static inline WeightGradPlan plan_weight_grad(int M, int K, int N, int H, int BK
       // it is shorter than they are), writing and reading the images, and two more launches
       const double elems = (double)pl.splits * (double)K * (double)N;
       const double product_us = 2.0 * (double)M * K * N / (elem_bytes == 4 ? 110e6 : 900e6);
-      const double store_us = elems * 4.0 / 4.0e6;
+      const double store_us = elems * tile_bytes / 4.0e6;
       // (K*N atomics take about 5.2 ps each; a long contraction hides up to 2.4 ps of that — K = 2048,
       //  N = 8192, bf16: M = 128 87 us in all against 57 us folded, M = 1024 108 against 79 us)
       const double hidden = 0.45 * product_us < elems * 2.4e-6 ? 0.45 * product_us : elems * 2.4e-6;
       const double atomics_us = elems * 5.2e-6 - hidden;
       // (a workgroup of the fold kernel reads some 15 GB/s: few workgroups cannot use the memory system)
-      const double read_bytes = elems * 4.0 * (1.0 + (double)BK * BN / f.window);
+      const double read_bytes = elems * tile_bytes * (1.0 + (double)BK * BN / f.window);
       const double all_us = (read_bytes + 2.0 * (double)f.partial_bytes) / 4.5e6;
       const double one_us = read_bytes / ((double)f.windows * f.shares) / 15e3;
       // (few tiles: every element is read once, by a kernel of a few microseconds; it is taken even where
       //  the atomics would be a little faster — K = N = 1024: 5 us against 3 us on top of the contraction —
       //  because it adds in a fixed order: the same bits on every call)
-      const double fold_us = f.small ? (store_us > product_us ? store_us - product_us : 0.0) + elems * 4.0 / 4.5e6 + 5.0
+      const double fold_us = f.small ? (store_us > product_us ? store_us - product_us : 0.0) + elems * tile_bytes / 4.5e6 + 5.0
                                      : (store_us > product_us ? store_us - product_us : 0.0) + (all_us > one_us ? all_us : one_us) + 10.0;
       if (t.fold >= 1 || f.small || fold_us < atomics_us) {
         pl.fold = f;

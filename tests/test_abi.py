@@ -112,8 +112,13 @@ def test_status_codes(lib):
     # of 2 KB) and the table of tile offsets; with the fold switched off, the atomic scatter: nothing for an
     # fp32 gradient, its fp32 image for a 16-bit one
     from rzlinear_amd import _lib
-    for code in (0, 1):
-        assert lib.rz_weight_grad_workspace_bytes(8, 128, 128, 65536, 64, 64, code) == 4 * 16384 + 2 * 2048 + 256
+    # (a 16-bit layer with a 16-bit dHW keeps the tiles in its own dtype: half the bytes; with an fp32 dHW, or told
+    #  to, floats)
+    assert lib.rz_weight_grad_workspace_bytes(8, 128, 128, 65536, 64, 64, 0) == 4 * 16384 + 2 * 2048 + 256
+    assert lib.rz_weight_grad_workspace_bytes(8, 128, 128, 65536, 64, 64, 1) == 4 * 8192 + 2 * 2048 + 256
+    assert lib.rz_weight_grad_ex_workspace_bytes(8, 128, 128, 65536, 64, 64, 1, 2, 0) == 4 * 16384 + 2 * 2048 + 256   # RZ_WG_DHW_F32
+    wide = _lib.Tuning(fold_tiles=-1)
+    assert lib.rz_weight_grad_hashed_workspace_bytes(8, 128, 128, 65536, 64, 64, 1, 0, 0, ctypes.byref(wide)) == 4 * 16384 + 2 * 2048 + 256
     no_fold = _lib.Tuning(fold=-1)
     assert lib.rz_weight_grad_hashed_workspace_bytes(8, 128, 128, 65536, 64, 64, 0, 0, 0, ctypes.byref(no_fold)) == 0
     assert lib.rz_weight_grad_hashed_workspace_bytes(8, 128, 128, 65536, 64, 64, 1, 0, 0, ctypes.byref(no_fold)) == 65536 * 4

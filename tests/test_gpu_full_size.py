@@ -11,7 +11,7 @@ import numpy as np
 import pytest
 import torch
 
-from helpers import SEED_CONSTANTS, TOL, ULP, rargs
+from helpers import SEED_CONSTANTS, TOL, ULP, rargs, ROUNDING
 
 pytestmark = pytest.mark.gpu
 
@@ -50,15 +50,15 @@ def _rel(out, ref):
     return float((out.double() - ref).abs().max() / ref.abs().max())
 
 
-def _check(out, ref, dtype, what):
-    """The stated normalised tolerance and the element-wise rounding bound of helpers.assert_close,
-    evaluated on the GPU (the tensors are large)."""
+def _check(out, ref, dtype, what, slack=None):
+    """The stated normalised tolerance and the element-wise rounding bound of helpers.assert_close
+    (with its allowance `slack` per element, if any), evaluated on the GPU (the tensors are large)."""
     ref = ref.double()
     err = (out.double() - ref).abs()
     scale = float(ref.abs().max())
     assert torch.isfinite(out).all(), what
     assert float(err.max()) / scale <= TOL[dtype], "%s: normalised max error %.3g" % (what, float(err.max()) / scale)
-    excess = err / (ULP[dtype] * ref.abs() + 1e-5 * scale)
+    excess = err / (ULP[dtype] * ref.abs() + 1e-5 * scale + (0.0 if slack is None else slack))
     worst = float(excess.max())
     assert worst <= 1.0, "%s: %.2f x the element-wise bound at flat index %d (%d elements beyond it)" % (
         what, worst, int(excess.argmax()), int((excess > 1.0).sum()))
@@ -97,7 +97,23 @@ def test_baseline_configuration_at_full_size(oracle, name):
     _check(dx, dy.double() @ W.t(), dtype, "dX")
     dW = x.double().t() @ dy.double()
     ref = torch.zeros((H,), dtype=torch.float64, device="cuda").index_add_(0, idx.reshape(-1), dW.reshape(-1))
-    _check(dhw, ref, dtype, "dHW")
+    # (a 16-bit layer whose weight gradient goes through the fold keeps the tiles of X^T.dY in its own dtype:
+    #  every stored value, one per element of X^T.dY and slice of M, is rounded once before the slots are
+    #  added up in fp32 — see helpers.stored_tiles_slack)
+    slack = None
+    if dtype != torch.float32:
+        from rzlinear_amd import _lib
+        code = _lib.RZ_BF16 if dtype == torch.bfloat16 else _lib.RZ_F16
+        folds = [q for q in (_lib.plan_query(2, M, K, N, H, BK, BN, code, planned=p) for p in (False, True)) if q["mode"] == "fold"]
+        for q in folds:
+            step = q["slice_len"] if q["slices"] > 1 else M
+            stored = sum((x[m:m + step].double().t() @ dy[m:m + step].double()).abs() for m in range(0, M, step))
+            s = torch.zeros((H,), dtype=torch.float64, device="cuda").index_add_(0, idx.reshape(-1), stored.reshape(-1))
+            slack = s if slack is None else torch.maximum(slack, s)
+            del stored
+        if slack is not None:
+            slack = ROUNDING[dtype] * slack
+    _check(dhw, ref, dtype, "dHW", slack)
     # mass conservation, a check that does not go through the index map: every element of
     # X^T.dY lands in exactly one slot
     assert abs(float(dhw.double().sum() - dW.sum())) <= TOL[dtype] * float(dW.abs().sum()) / 10

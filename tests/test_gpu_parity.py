@@ -6,7 +6,7 @@ import numpy as np
 import pytest
 import torch
 
-from helpers import SEED_CONSTANTS, TOL, assert_close, make_inputs, rargs, rel_err
+from helpers import SEED_CONSTANTS, TOL, assert_close, make_inputs, rargs, rel_err, stored_tiles_slack
 
 pytestmark = pytest.mark.gpu
 
@@ -516,7 +516,8 @@ def test_random_shapes_16bit(oracle, shape):
     f = lambda t: t.float().cpu().numpy()
     assert_close(f(y), oracle.forward(x64, hw64, N, BK, BN, R, 0.75) + bias.double().cpu().numpy(), dtype, "Y")
     assert_close(f(dx), oracle.input_grad(dy64, hw64, K, BK, BN, R, 0.75), dtype, "dX")
-    assert_close(f(dhw), oracle.weight_grad(x64, dy64, H, BK, BN, R, 0.75), dtype, "dHW")
+    assert_close(f(dhw), oracle.weight_grad(x64, dy64, H, BK, BN, R, 0.75), dtype, "dHW",
+                 slack=stored_tiles_slack(oracle, x64, dy64, shape, R, 0.75, dtype))
     assert_close(f(dbias), dy64.sum(axis=0), dtype, "dbias")
 
 
@@ -567,7 +568,7 @@ def test_rows_that_are_not_whole_16_byte_pieces(oracle, shape, dtype):
     assert_close(f(y), oracle.forward(x64, hw64, N, BK, BN, R1024) + bias.double().cpu().numpy()[None, :], dtype, "Y")
     assert_close(f(dx), oracle.input_grad(dy64, hw64, K, BK, BN, R1024), dtype, "dX")
     ref = oracle.weight_grad(x64, dy64, H, BK, BN, R1024)
-    assert_close(f(dhw), ref, dtype, "dHW")
+    assert_close(f(dhw), ref, dtype, "dHW", slack=stored_tiles_slack(oracle, x64, dy64, shape, R1024, 1.0, dtype))
     assert (f(dhw)[ref == 0] == 0).all()
     assert rel_err(f(dbias), dy64.sum(axis=0)) <= TOL[dtype]
     # (where the plan takes a 128 or 256 tile these shapes run the direct-to-LDS kernels: say which)

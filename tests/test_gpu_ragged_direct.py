@@ -7,7 +7,7 @@ import sys
 import pytest
 import torch
 
-from helpers import SEED_CONSTANTS, TOL, assert_close, make_inputs, rargs, rel_err
+from helpers import SEED_CONSTANTS, TOL, assert_close, make_inputs, rargs, rel_err, stored_tiles_slack
 
 pytestmark = pytest.mark.gpu
 
@@ -50,6 +50,7 @@ def test_ragged_edges_with_direct_staging(oracle, tuned, shape, form):
                                                     rz_linear_backward_weight_bias_grad_tl,
                                                     rz_linear_backward_weight_grad_tl)
     from rzlinear_amd.impl.RzLinearForward import rz_linear_forward_bias_tl
+    from rzlinear_amd import _lib
     tuned(tile=tile)
     M, K, N, H, BK, BN = shape
     _say("ragged direct", shape, tile, dtype)
@@ -67,8 +68,10 @@ def test_ragged_edges_with_direct_staging(oracle, tuned, shape, form):
     assert_close(f(y), oracle.forward(x64, hw64, N, BK, BN, R1024) + bias.double().cpu().numpy(), dtype, "Y")
     assert_close(f(dx), oracle.input_grad(dy64, hw64, K, BK, BN, R1024), dtype, "dX")
     ref = oracle.weight_grad(x64, dy64, H, BK, BN, R1024)
-    assert_close(f(dhw), ref, dtype, "dHW")
-    assert_close(f(dhw2), ref, dtype, "dHW (with bias gradient)")
+    with _lib.tuning(tile=tile):
+        slack = stored_tiles_slack(oracle, x64, dy64, shape, R1024, 1.0, dtype)
+    assert_close(f(dhw), ref, dtype, "dHW", slack=slack)
+    assert_close(f(dhw2), ref, dtype, "dHW (with bias gradient)", slack=slack)
     assert_close(f(dbias), dy64.sum(axis=0), dtype, "dbias")
     # the bounds-checked kernels give the same results
     tuned(tile=tile, clamp=-1)
@@ -83,5 +86,5 @@ def test_ragged_edges_with_direct_staging(oracle, tuned, shape, form):
         assert_close(f(dx2), oracle.input_grad(dy64, hw64, K, BK, BN, R1024), dtype, "dX (bounds-checked)")
     else:
         assert torch.equal(y, y2) and torch.equal(dx, dx2)
-    assert_close(f(dhw3), ref, dtype, "dHW (bounds-checked)")
+    assert_close(f(dhw3), ref, dtype, "dHW (bounds-checked)", slack=slack)
     assert_close(f(dbias3), dy64.sum(axis=0), dtype, "dbias (bounds-checked)")

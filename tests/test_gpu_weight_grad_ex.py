@@ -1,6 +1,7 @@
 """GPU parity of rz_weight_grad_ex: bias gradient from the same pass, accumulation into an
 existing buffer, fp32 gradient buffers for 16-bit operands.  Checked against the CPU oracle's
 weight-grad and against the column sums of dY in float64."""
+import ctypes
 import sys
 
 import numpy as np
@@ -183,6 +184,51 @@ def test_tiles_stored_plainly_and_folded_into_the_gradient(oracle, tuned, shape,
     c = rz_linear_backward_weight_grad_tl(x, dy, 0.5, M, K, N, H, *rargs(R1024), **kw)
     torch.cuda.synchronize()
     assert rel_err(f(c), ref) <= TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=_dt_id)
+@pytest.mark.parametrize("shape", [(1024, 512, 768, 70000, 64, 64), (4100, 320, 200, 300000, 32, 64),
+                                   (300, 1000, 1100, 1 << 20, 16, 16)], ids=_shape_id)
+def test_tiles_stored_in_the_layers_dtype_cost_one_rounding_each(oracle, tuned, shape, dtype):
+    """A 16-bit layer with a 16-bit dHW keeps the tiles of X^T.dY for the fold in its own dtype (half the
+    bytes).  Every stored value is a complete fp32 sum over M (or a slice of it), rounded once; the fold adds
+    the values of a slot up in fp32: so the error of an element is bounded by one rounding of each of its
+    addends plus the output's own — checked element by element against the oracle with exactly that
+    allowance.  rz_tuning.fold_tiles = -1, and an fp32 dHW (RZ_WG_DHW_F32), keep fp32 tiles: one rounding
+    in all, the element-wise bound without any allowance.  Same bits on every call either way."""
+    from helpers import assert_close, stored_tiles_slack
+    from rzlinear_amd import _lib
+    from rzlinear_amd.impl.RzLinearBackward import rz_linear_backward_weight_grad_tl
+    M, K, N, H, BK, BN = shape
+    code = _lib.dtype_code(torch.empty(0, dtype=dtype))
+    (x, _, dy), (x64, _, dy64) = make_inputs(M, K, N, H, dtype, seed=83)
+    kw = dict(BLOCK_SIZE_K=BK, BLOCK_SIZE_N=BN)
+    ref = oracle.weight_grad(x64, dy64, H, BK, BN, R1024, 0.5)
+    f = lambda t: t.float().cpu().numpy()
+    lib = _lib.load()
+    for kernel in (1, 2):   # the kernel for few tiles where it applies, and the windowed one
+        tuned(fold=kernel, window=-1, lds_image=-1)
+        plan = _lib.plan_query(2, M, K, N, H, BK, BN, code)
+        _say("tiles in the layer's dtype", shape, dtype, plan)
+        assert plan["mode"] == "fold", plan
+        narrow_ws = lib.rz_weight_grad_hashed_workspace_bytes(M, K, N, H, BK, BN, code, 0, 0, ctypes.byref(_lib.Tuning(fold=kernel, window=-1, lds_image=-1)))
+        a = rz_linear_backward_weight_grad_tl(x, dy, 0.5, M, K, N, H, *rargs(R1024), **kw)
+        a2 = rz_linear_backward_weight_grad_tl(x, dy, 0.5, M, K, N, H, *rargs(R1024), **kw)
+        slack = stored_tiles_slack(oracle, x64, dy64, shape, R1024, 0.5, dtype)
+        assert slack is not None
+        assert_close(f(a), ref, dtype, "dHW (tiles in the layer's dtype)", slack=slack)
+        assert torch.equal(a, a2)
+        tuned(fold=kernel, window=-1, lds_image=-1, fold_tiles=-1)
+        wide_ws = lib.rz_weight_grad_hashed_workspace_bytes(M, K, N, H, BK, BN, code, 0, 0, ctypes.byref(_lib.Tuning(fold=kernel, window=-1, lds_image=-1, fold_tiles=-1)))
+        assert wide_ws > narrow_ws
+        b = rz_linear_backward_weight_grad_tl(x, dy, 0.5, M, K, N, H, *rargs(R1024), **kw)
+        assert_close(f(b), ref, dtype, "dHW (fp32 tiles)")
+        # an fp32 gradient buffer never goes through 16-bit tiles
+        tuned(fold=kernel, window=-1, lds_image=-1)
+        c = torch.zeros((H,), dtype=torch.float32, device="cuda")
+        rz_linear_backward_weight_grad_tl(x, dy, 0.5, M, K, N, H, *rargs(R1024), out=c, **kw)
+        torch.cuda.synchronize()
+        assert_close(f(c), ref, torch.float32, "dHW (fp32 buffer)")
 
 
 def test_fold_shares_take_a_partition_of_a_window_even_when_their_lists_overflow(oracle):

@@ -9,7 +9,7 @@ import numpy as np
 import pytest
 import torch
 
-from helpers import SEED_CONSTANTS, TOL, assert_close, make_inputs, rel_err
+from helpers import SEED_CONSTANTS, TOL, assert_close, make_inputs, rel_err, stored_tiles_slack
 
 pytestmark = pytest.mark.gpu
 
@@ -42,7 +42,8 @@ def _both(lib, shape, dtype, seed, oracle):
     _lib.check(lib.rz_weight_grad(x.data_ptr(), dy.data_ptr(), b.data_ptr(), ws.data_ptr(), need, M, K, N, H,
                                   BK, BN, R, 0.5, K, N, code, stream))
     torch.cuda.synchronize()
-    return a, b, oracle.weight_grad(x64, dy64, H, BK, BN, R1024, 0.5), need <= SCRATCH_BYTES
+    slack = stored_tiles_slack(oracle, x64, dy64, shape, R1024, 0.5, dtype)
+    return a, b, oracle.weight_grad(x64, dy64, H, BK, BN, R1024, 0.5), need <= SCRATCH_BYTES, slack
 
 
 # (first problem, smaller second problem, how the plan carries the first one out in bf16)
@@ -66,7 +67,7 @@ def test_static_scratch_matches_the_workspace_entry_point(oracle, pair, dtype):
         _say("static scratch", mode, "call", i, shape, dtype, plan)
         if dtype == torch.bfloat16 and i == 0:
             assert plan["mode"] == mode, plan      # the scratch layouts are all exercised
-        a, b, ref, fits = _both(lib, shape, dtype, seed=50 + i, oracle=oracle)
+        a, b, ref, fits, slack = _both(lib, shape, dtype, seed=50 + i, oracle=oracle)
         assert fits or dtype != torch.bfloat16   # (the bf16 pairs exercise the scratch layouts named above)
         f = lambda t: t.float().cpu().numpy()
         if plan["mode"] == "atomics" or not fits:
@@ -74,8 +75,8 @@ def test_static_scratch_matches_the_workspace_entry_point(oracle, pair, dtype):
             assert rel_err(f(a), f(b).astype(np.float64)) <= TOL[dtype]
         else:
             assert torch.equal(a, b)            # fixed summation order: the same bits
-        assert_close(f(a), ref, dtype, "dHW (static scratch)")
-        assert_close(f(b), ref, dtype, "dHW (workspace)")
+        assert_close(f(a), ref, dtype, "dHW (static scratch)", slack=slack)
+        assert_close(f(b), ref, dtype, "dHW (workspace)", slack=slack)
 
 
 def test_static_scratch_gives_up_the_fold_when_its_buffer_does_not_fit(oracle):
