@@ -11,9 +11,9 @@
 // thread (a 32-bit byte offset per piece); the step only moves a uniform base in scalar
 // registers, and a hashed piece adds its tile's table entry.
 //
-// Register staging (fp32, the 64 tile, ragged contracted dimension): global -> registers (issued
-// one or two steps ahead) -> LDS (one or two stages).  LDS layouts (X = I or J extent of the
-// operand)
+// Register staging (the 16-bit 64 tile, rows shorter than 16 bytes, the single-stage form):
+// global -> registers (issued one or two steps ahead) -> LDS (one or two stages).  LDS layouts
+// (X = I or J extent of the operand)
 //   16-bit, R contiguous in the source : [X][TR + 8]   fragment = one ds_read_b128 per lane
 //   16-bit, X contiguous in the source : [TR][X + 32]  fragment = two ds_read_b64_tr_b16
 //       (the LDS transpose read returns, to lane c of a 16-lane group, column c of a 4 x 16
@@ -22,16 +22,21 @@
 //   fp32                                : [TR][X + pad], one ds_read_b32 per lane; a source
 //       with R contiguous is transposed while it is written (pad 1), else copied (pad 4)
 //
-// Direct staging (16-bit types, 128 and 256 tiles, two stages; complete tiles, or ragged ones
-// with CLAMP below): the tiles go global -> LDS with
+// Direct staging (16-bit types: the 128 and 256 tiles; fp32: every tile; two stages; complete
+// tiles, or ragged ones with CLAMP below): the tiles go global -> LDS with
 // direct-to-LDS loads, no registers and no LDS write instructions in between.  Such a load
 // puts the 64 lanes' 16-byte pieces at consecutive LDS addresses, so rows cannot be padded;
 // the stages are unpadded and swizzled instead, and the swizzle is applied on the global side
 // (each lane fetches the piece that belongs at its LDS slot):
 //   R contiguous : [X][TR], row = 8 pieces; piece p of row x sits at slot p ^ ((x >> 1) & 7)
 //                  (16 pieces with the 256-byte R step: slot p ^ (x & 15))
-//   X contiguous : [TR][X], row = X/32 chunks of 64 bytes; chunk c of row r sits at c ^ (r & 3)
-// Both keep the fragment reads above free of bank conflicts.
+//   X contiguous : [TR][X], row = X/32 units of 32 elements; unit u of row r sits at u ^ (r & 3)
+//                  (fp32: u ^ ((r >> 2) & 1))
+// Both keep the fragment reads free of bank conflicts.  fp32 fragments of a directly staged tile
+// cover eight elements of R at a time, four MFMAs per pair of blocks: MFMA j of the four contracts
+// elements j (lanes 0-31) and 4 + j (lanes 32-63) — any pairing of the two halves is a valid sum as
+// long as A and B use the same one — so a lane's four values are one 16-byte piece where R is
+// contiguous (one ds_read_b128) and four ds_read_b32 of one column where X is.
 #pragma once
 
 #include <type_traits>
