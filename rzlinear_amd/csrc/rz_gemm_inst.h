@@ -74,6 +74,15 @@ static hipError_t launch_tile(GemmParams p, const WeightGradPlan* plan, const Sp
                               const KernelForm& form, hipStream_t stream) {
   // (the form was derived on the host from the same rules that select the instantiation here:
   //  refuse to launch if the two ever disagree about the step length)
+  // A directly staged load addresses the hashed operand by a 32-bit byte offset from its first
+  // element: an fp32 hashed_weight of 4 GB and more takes the bounds-checked kernel, whose loads
+  // carry full pointers (the step is the same for both fp32 forms).
+  const bool far = sizeof(T) == 4 && OP != kWeightGrad &&
+                   ((unsigned long long)p.h.range + (unsigned long long)p.h.BK * (unsigned long long)p.h.BN) * sizeof(T) > 0xffffffffull;
+  if (far) {
+    if (form.step != GemmKernel<T, OP, TILE, TILE_J, WI, WJ, NSTAGE, false>::TR) return hipErrorInvalidValue;
+    return launch_one<T, OP, TILE, TILE_J, WI, WJ, NSTAGE, false, COLSUM, false, WK>(p, plan, split, stream);
+  }
   if (form.full) {
     if (form.step != GemmKernel<T, OP, TILE, TILE_J, WI, WJ, NSTAGE, true>::TR) return hipErrorInvalidValue;
     return launch_one<T, OP, TILE, TILE_J, WI, WJ, NSTAGE, true, COLSUM, false, WK>(p, plan, split, stream);
