@@ -88,6 +88,9 @@ typedef struct rz_tuning {
                      tile in the layer's dtype: half the bytes written and read back; every stored value is
                      rounded once more than in fp32, the sum over M and the sum of the tiles stay fp32),
                      -1 = always fp32 tiles */
+  int finish;     /* forward / input-grad with a cut contraction: 0 = automatic (the slice that arrives last at a
+                     tile of the output adds the slices' partial results up and stores it: no second kernel),
+                     -1 = always a second kernel; the results are the same bits either way */
   int poll_limit; /* weight-grad by windows: 0 = default; > 0 = how often a wavefront looks at the flags of the
                      earlier strips it waits for before it gives up and the window is stored as NaN (a bounded
                      wait; tests set a tiny value to see every wavefront leave the kernel all the same) */

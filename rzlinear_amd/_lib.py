@@ -33,7 +33,7 @@ class Tuning(ctypes.Structure):
     automatic).  Only tests and benchmarks set any of it."""
     _fields_ = [("tile", ctypes.c_int), ("stages", ctypes.c_int), ("lds_image", ctypes.c_int),
                 ("window", ctypes.c_int), ("split", ctypes.c_int), ("clamp", ctypes.c_int),
-                ("fold", ctypes.c_int), ("fold_tiles", ctypes.c_int), ("poll_limit", ctypes.c_int)]
+                ("fold", ctypes.c_int), ("fold_tiles", ctypes.c_int), ("finish", ctypes.c_int), ("poll_limit", ctypes.c_int)]
 
 
 # What the launchers of this package pass as `tuning` (None = automatic).  The C library keeps no

@@ -246,6 +246,43 @@ static hipError_t reduce_slices_dtype(int dtype, const float* part, void* C, con
   }
 }
 
+// ---- counters of the cut contractions that finish in one kernel ---------------------------------
+// One 32-bit counter per tile of the output and launch (GemmParams::finish), in a file-scope device
+// array: zero when the library is loaded, and set back to zero by the workgroup that finishes a tile.
+// Launches take consecutive ranges of the array in turn, so two launches share counters only if
+// kFinishCounters tiles' worth of launches are in flight at once.  In host code the array's name is a
+// handle for hipGetSymbolAddress, looked up once per device with that device current.
+static constexpr unsigned kFinishCounters = 1u << 16;
+static constexpr int kFinishMaxDevices = 64;
+static __device__ __align__(256) unsigned finish_counters[kFinishCounters];
+static std::atomic<unsigned*> finish_counters_ptr[kFinishMaxDevices];
+static std::atomic<unsigned> finish_turn{0};
+
+// Counters for a launch with `tiles` output tiles, or null (the caller then launches the second kernel).
+static unsigned* finish_counters_for(long long tiles) {
+  if (tiles < 1 || tiles > (long long)(kFinishCounters / 4)) return nullptr;
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kFinishMaxDevices) return nullptr;
+  unsigned* base = finish_counters_ptr[dev].load(std::memory_order_acquire);
+  if (base == nullptr) {
+    void* q = nullptr;
+    if (hipGetSymbolAddress(&q, HIP_SYMBOL(finish_counters)) != hipSuccess || q == nullptr) {
+      (void)hipGetLastError();
+      return nullptr;
+    }
+    base = static_cast<unsigned*>(q);
+    finish_counters_ptr[dev].store(base, std::memory_order_release);   // (a racing thread stores the same value)
+  }
+  // the next `tiles` counters, from the start of the array if they would run off its end
+  unsigned seen = finish_turn.load(std::memory_order_relaxed);
+  for (;;) {
+    const unsigned at = seen % kFinishCounters;
+    const unsigned start = at + (unsigned)tiles <= kFinishCounters ? at : 0u;
+    const unsigned next = seen - at + start + (unsigned)tiles + (start == 0u && at != 0u ? kFinishCounters : 0u);
+    if (finish_turn.compare_exchange_weak(seen, next, std::memory_order_relaxed)) return base + start;
+  }
+}
+
 // Forward (op kForward) or input-grad through one code path: p holds the operands; with a
 // workspace the contraction may be split over R (skinny problems).
 static int run_plain_op(int op, int dtype, GemmParams p, const void* bias, void* workspace,
@@ -259,8 +296,15 @@ static int run_plain_op(int op, int dtype, GemmParams p, const void* bias, void*
     if (sp.splits > 1) {
       if (workspace == nullptr || workspace_bytes < sp.workspace_bytes) return RZ_ERR_WORKSPACE;
       p.partial = (float*)workspace;
-      p.bias = nullptr;
+      // the slice that arrives last at a tile finishes it (adds the slices in slice order, then the
+      // bias: the bits of the second kernel's sum) — unless told otherwise, or out of counters
+      // (the 32 x 64 tile has two wavefronts to read the other slices with: three slices at most — fp32,
+      //  M = 16, K = 4096, N = 11008 input-grad in four slices: 36 -> 39 us)
+      const int most = sp.tile == 32 ? kFinishSlices - 1 : kFinishSlices;
+      p.finish = (tuning.finish != -1 && sp.splits <= most) ? finish_counters_for(tile_count(p.I, p.J, sp.tile)) : nullptr;
+      p.bias = p.finish != nullptr ? bias : nullptr;
       if (launch_gemm(dtype, op, p, nullptr, &sp, tuning, s) != hipSuccess) return RZ_ERR_LAUNCH;
+      if (p.finish != nullptr) return RZ_OK;
       return reduce_slices_dtype(dtype, p.partial, p.C, bias, p.I, p.J, p.ldc, sp.splits, s) == hipSuccess
                  ? RZ_OK : RZ_ERR_LAUNCH;
     }

@@ -93,6 +93,12 @@ __host__ __device__ __forceinline__ uint32_t tile_offset(const HashParams& h, ui
 //   weight-grad  I=K J=N R=M   A = X  (rows r=m, contiguous i) B = dY      (rows r=m, contiguous j)
 enum Op { kForward = 0, kInputGrad = 1, kWeightGrad = 2 };
 
+// A cut contraction of at most this many slices is finished by its own kernel (GemmParams::finish):
+// the slice that comes last reads the others' planes by itself, which pays up to here; beyond, a
+// second kernel whose every workgroup shares that reading is faster (bf16, K = N = 10240: three
+// slices at M = 1024 229 -> 212 us; six slices at M = 32 40 -> 52 us).
+static constexpr int kFinishSlices = 4;
+
 struct GemmParams {
   const void* A;
   const void* B;      // plain B operand (weight-grad) — else unused
@@ -102,6 +108,9 @@ struct GemmParams {
   const void* bias;   // optional [J] vector added to every row of C (forward), or null
   float* partial;     // forward/input-grad with R split over blockIdx.y: fp32 partial results
                       // [slices][I][J] (scaled, no bias) instead of C; null = no split
+  unsigned* finish;   // ... with one counter per C tile (zero between launches): the slice that arrives
+                      // last at a tile adds the slices up itself and stores C (+ bias); null = a second
+                      // kernel does
   float* scatter;     // weight-grad target: fp32 image of dHW (direct atomics), or the
                       // per-workgroup partial images [workgroups][image_pitch] (LDS mode)
   int image_pitch;    // > 0 selects the LDS mode: floats per partial image (H rounded up to 4)
@@ -121,5 +130,15 @@ struct GemmParams {
   float scale;
   HashParams h;
 };
+
+// Loads and stores at agent scope: for data that another workgroup of the SAME kernel wrote or will
+// read (such accesses go to the point where the GPU's L2 caches agree; a wavefront that has waited
+// for its own stores may then tell the others, through an atomic, that they are there).
+__device__ __forceinline__ void store_agent_f32(float* at, float v) {
+  __hip_atomic_store(at, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float load_agent_f32(const float* at) {
+  return __hip_atomic_load(at, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
 
 }  // namespace rz

@@ -1166,36 +1166,21 @@ struct GemmKernel {
                 park[(wave_k - 1) * TI * TJ + slot + ((a * MJ + b) * 16 + e) * 64] = acc[a][b][e];
         }
         __syncthreads();
-        if (wave_k > 0) return;
+        if (wave_k == 0) {
 #pragma unroll
-        for (int g = 1; g < WK; g++)
+          for (int g = 1; g < WK; g++)
 #pragma unroll
-          for (int a = 0; a < MI; a++)
+            for (int a = 0; a < MI; a++)
 #pragma unroll
-            for (int b = 0; b < MJ; b++)
+              for (int b = 0; b < MJ; b++)
 #pragma unroll
-              for (int e = 0; e < 16; e++)
-                acc[a][b][e] += park[(g - 1) * TI * TJ + slot + ((a * MJ + b) * 16 + e) * 64];
-      }
-      if (p.partial != nullptr) {
-        // R is split over the slices `by` (few C tiles, long R): this slice's scaled fp32 partial
-        // result goes to its own [I][J] plane; a second kernel adds the planes up
-        float* __restrict__ gP = p.partial + (size_t)by * (size_t)p.I * (size_t)p.J;
-#pragma unroll
-        for (int a = 0; a < MI; a++) {
-#pragma unroll
-          for (int e = 0; e < 16; e++) {
-            const int row = i0 + blk_i(a) + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
-#pragma unroll
-            for (int b = 0; b < MJ; b++) {
-              const int col = j0 + blk_j(b) + (lane & 31);
-              if (FULL || (row < p.I && col < p.J)) gP[(size_t)row * p.J + col] = acc[a][b][e] * p.scale;
-            }
-          }
+                for (int e = 0; e < 16; e++)
+                  acc[a][b][e] += park[(g - 1) * TI * TJ + slot + ((a * MJ + b) * 16 + e) * 64];
         }
-        return;
       }
-      T* __restrict__ gC = static_cast<T*>(p.C);
+      // (of several groups of wavefronts that shared the R steps, the first holds the sums and stores)
+      const bool writer = wave_k == 0;   // (uniform)
+      float out_scale = p.scale;
       const T* __restrict__ gBias = static_cast<const T*>(p.bias);
       // optional bias of this lane's columns, added in fp32 before the single rounding
       float bias[MJ];
@@ -1205,6 +1190,85 @@ struct GemmKernel {
         bias[b] = 0.f;
         if (gBias != nullptr && (FULL || col < p.J)) bias[b] = Tr::to_float(gBias[col]);
       }
+      if (p.partial != nullptr) {
+        // R is split over the slices `by` (few C tiles, long R): this slice's scaled fp32 partial
+        // result goes to its own [I][J] plane.  The planes are added up by a second kernel — or,
+        // with a counter per C tile (p.finish), by the slice that arrives at the tile last: it
+        // adds the planes in slice order, its own from its registers (the same bits it stored),
+        // so the sum does not depend on who came last; nobody waits for anybody.
+        float* __restrict__ gP = p.partial + (size_t)by * (size_t)p.I * (size_t)p.J;
+        const bool finishing = p.finish != nullptr;   // (uniform)
+        if (writer) {
+#pragma unroll
+          for (int a = 0; a < MI; a++) {
+#pragma unroll
+            for (int e = 0; e < 16; e++) {
+              const int row = i0 + blk_i(a) + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
+#pragma unroll
+              for (int b = 0; b < MJ; b++) {
+                const int col = j0 + blk_j(b) + (lane & 31);
+                if (FULL || (row < p.I && col < p.J)) {
+                  if (finishing) store_agent_f32(gP + (size_t)row * p.J + col, acc[a][b][e] * p.scale);
+                  else gP[(size_t)row * p.J + col] = acc[a][b][e] * p.scale;
+                }
+              }
+            }
+          }
+        }
+        if (!finishing) return;
+        const int slices = (int)gridDim.y;
+        unsigned* counter = p.finish + (size_t)ti * (size_t)p.tiles_j + tj;
+        int* arrived = reinterpret_cast<int*>(&sm);   // (the stages are dead)
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this wavefront's part of the plane is where the others will look
+        __syncthreads();
+        if (tid == 0) *arrived = (int)__hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();
+        if (*arrived != slices - 1) return;   // (uniform) another slice will finish this tile
+        if (tid == 0) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // (as the next launch expects it)
+        if (!writer) return;
+        const size_t plane = (size_t)p.I * (size_t)p.J;
+#pragma unroll
+        for (int a = 0; a < MI; a++) {
+#pragma unroll
+          for (int b = 0; b < MJ; b++) {
+            const int col = j0 + blk_j(b) + (lane & 31);
+            // (all the other slices' values of the block are fetched before the first is used)
+            float v[kFinishSlices][16];
+#pragma unroll
+            for (int sl = 0; sl < kFinishSlices; sl++) {
+              if (sl < slices && sl != by) {   // (uniform)
+#pragma unroll
+                for (int e = 0; e < 16; e++) {
+                  const int row = i0 + blk_i(a) + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
+                  v[sl][e] = (FULL || (row < p.I && col < p.J)) ? load_agent_f32(p.partial + (size_t)sl * plane + (size_t)row * p.J + col) : 0.f;
+                }
+              }
+            }
+            float sum[16];
+#pragma unroll
+            for (int e = 0; e < 16; e++) sum[e] = 0.f;
+#pragma unroll
+            for (int sl = 0; sl < kFinishSlices; sl++) {
+              if (sl == by) {
+#pragma unroll
+                for (int e = 0; e < 16; e++) sum[e] += __fmul_rn(acc[a][b][e], p.scale);   // (the product as it was stored: not fused into the add)
+              } else if (sl < slices) {
+#pragma unroll
+                for (int e = 0; e < 16; e++) sum[e] += v[sl][e];
+              }
+            }
+            // (the bias joins the fp32 sum as in the second kernel: an add of its own, rounded to fp32,
+            //  not part of a fused multiply-add that rounds straight to the output type)
+#pragma unroll
+            for (int e = 0; e < 16; e++) acc[a][b][e] = __fadd_rn(sum[e], bias[b]);
+          }
+        }
+        out_scale = 1.f;
+#pragma unroll
+        for (int b = 0; b < MJ; b++) bias[b] = 0.f;
+      }
+      if (!writer) return;
+      T* __restrict__ gC = static_cast<T*>(p.C);
       // the column blocks of a row go out back to back, so that the halves of a cache line
       // reach L2 together.  A large C is stored with streaming stores: nothing here reads it
       // again, and kept in L2 it would push out the operand panels that the workgroups of the
@@ -1219,7 +1283,7 @@ struct GemmKernel {
             for (int b = 0; b < MJ; b++) {
               const int col = j0 + blk_j(b) + (lane & 31);
               if (FULL || (row < p.I && col < p.J)) {
-                const T value = Tr::from_float(acc[a][b][e] * p.scale + bias[b]);
+                const T value = Tr::from_float(acc[a][b][e] * out_scale + bias[b]);
                 T* dst = gC + (int64_t)row * p.ldc + col;
                 if constexpr (!decltype(streaming)::value) *dst = value;
                 else if constexpr (sizeof(T) == 4) __builtin_nontemporal_store(value, dst);

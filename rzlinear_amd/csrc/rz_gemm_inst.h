@@ -44,9 +44,12 @@ static hipError_t launch_one(GemmParams p, const WeightGradPlan* plan, const Spl
     // a slice must begin on a step boundary: the offset table of a step assumes that the step
     // lies inside one hashed tile or covers whole ones
     if (p.r_chunk % K::TR != 0) return hipErrorInvalidValue;
+    // (the kernel that finishes its own tiles holds the other slices' values in registers)
+    if (p.finish != nullptr && splits > kFinishSlices) return hipErrorInvalidValue;
   } else {
     p.r_chunk = r_steps * K::TR;
     p.partial = nullptr;
+    p.finish = nullptr;
   }
   auto kernel = rz_gemm_kernel<T, OP, TI, TJ, WI, WJ, NSTAGE, FULL, COLSUM, CLAMP, WK>;
   size_t smem = sizeof(typename K::Smem);

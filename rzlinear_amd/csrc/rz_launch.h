@@ -19,7 +19,7 @@ static inline bool tuning_valid(const rz_tuning& t) {
   return (t.tile == 0 || t.tile == 32 || t.tile == 64 || t.tile == 128 || t.tile == 256) && (t.stages == 0 || t.stages == 1) &&
          (t.lds_image == 0 || t.lds_image == -1) && (t.window >= -1 && t.window <= 1) &&
          (t.split == 0 || t.split == -1) && (t.clamp == 0 || t.clamp == -1) &&
-         (t.fold >= -1 && t.fold <= 2) && (t.fold_tiles == 0 || t.fold_tiles == -1) && t.poll_limit >= 0;
+         (t.fold >= -1 && t.fold <= 2) && (t.fold_tiles == 0 || t.fold_tiles == -1) && (t.finish == 0 || t.finish == -1) && t.poll_limit >= 0;
 }
 
 // Kernels that use more than the default 64 KB of LDS need their limit raised once per kernel

@@ -178,6 +178,54 @@ def test_fp32_batches_of_at_most_32_rows_take_the_32_row_tile(oracle, shape, spl
     assert rel_err(dx.cpu().numpy(), oracle.input_grad(dy64, hw64, K, BK, BN, R1024, 0.5)) <= TOL[torch.float32]
 
 
+FINISH_CASES = [
+    # (M, K, N, H, BK, BN, tile override or 0)
+    (32, 10240, 1024, 1 << 20, 64, 64, 0),      # skinny forward: many slices of few tiles
+    (128, 2048, 8192, 16384, 64, 64, 0),        # input-grad contracts 8192
+    (1024, 10240, 10240, 6553600, 32, 64, 256), # the reference's large grid shape: 160 tiles of 256 in three slices
+    (100, 3000, 500, 9000, 32, 64, 0),          # ragged tiles and a ragged last slice
+    (300, 4100, 260, 70000, 64, 64, 128),
+    (17, 5000, 150, 5000, 16, 16, 64),
+]
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=lambda d: str(d).split(".")[-1])
+@pytest.mark.parametrize("case", FINISH_CASES, ids=lambda s: "x".join(map(str, s)))
+def test_the_last_slice_to_arrive_finishes_the_tile(oracle, case, dtype):
+    """A cut contraction (forward / input-grad of skinny problems) leaves no second kernel behind: the
+    slices store their fp32 partial results, count themselves in at their tile, and the one that comes
+    last adds the slices up in slice order — its own from its registers — adds the bias and stores.
+    The bits are those of the two-kernel form (rz_tuning.finish = -1) whoever comes last; checked over
+    several calls (the counters return to zero), with a bias, against the oracle."""
+    from rzlinear_amd import _lib
+    from rzlinear_amd.impl.RzLinearBackward import rz_linear_backward_input_grad_tl
+    from rzlinear_amd.impl.RzLinearForward import rz_linear_forward_bias_tl
+    M, K, N, H, BK, BN, tile = case
+    shape = (M, K, N, H, BK, BN)
+    _say("last slice finishes", case, dtype)
+    code = _lib.dtype_code(torch.empty(0, dtype=dtype))
+    (x, hw, dy), (x64, hw64, dy64) = make_inputs(M, K, N, H, dtype, seed=14)
+    bias = torch.randn((N,), generator=torch.Generator().manual_seed(4)).to(dtype).cuda()
+    kw = dict(BLOCK_SIZE_K=BK, BLOCK_SIZE_N=BN)
+    tn = dict(tile=tile) if tile else {}
+    with _lib.tuning(**tn):
+        plans = [_lib.plan_query(op, M, K, N, H, BK, BN, code) for op in (0, 1)]
+        assert any(q["slices"] > 1 for q in plans), plans
+        ys = [rz_linear_forward_bias_tl(x, hw, bias, 0.5, M, K, N, H, *rargs(R1024), **kw) for _ in range(3)]
+        dxs = [rz_linear_backward_input_grad_tl(dy, hw, 0.5, M, K, N, H, *rargs(R1024), **kw) for _ in range(3)]
+    with _lib.tuning(finish=-1, **tn):
+        y2 = rz_linear_forward_bias_tl(x, hw, bias, 0.5, M, K, N, H, *rargs(R1024), **kw)
+        dx2 = rz_linear_backward_input_grad_tl(dy, hw, 0.5, M, K, N, H, *rargs(R1024), **kw)
+    torch.cuda.synchronize()
+    for y in ys:
+        assert torch.equal(y, y2)
+    for dx in dxs:
+        assert torch.equal(dx, dx2)
+    f = lambda t: t.float().cpu().numpy()
+    assert_close(f(ys[0]), oracle.forward(x64, hw64, N, BK, BN, R1024, 0.5) + bias.double().cpu().numpy()[None, :], dtype, "Y")
+    assert_close(f(dxs[0]), oracle.input_grad(dy64, hw64, K, BK, BN, R1024, 0.5), dtype, "dX")
+
+
 @pytest.mark.parametrize("M", [32, 96, 160, 288])
 def test_the_32_row_tile_is_chosen_where_64_rows_would_be_half_padding(oracle, M):
     """K = N = 4096, fp32: the plan takes the 32 x 64 tile by itself for these batch sizes (and not for
