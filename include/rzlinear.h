@@ -78,7 +78,8 @@ typedef struct rz_tuning {
   int stages;     /* 0 = automatic, 1 = the single-stage form of the 128 tile */
   int lds_image;  /* weight-grad: 0 = automatic, -1 = never sum tiles in an LDS image of dHW */
   int window;     /* weight-grad: 0 = automatic, 1 = dHW by windows whenever possible, -1 = never */
-  int split;      /* forward / input-grad: 0 = automatic, -1 = never split the contraction */
+  int split;      /* forward / input-grad: 0 = automatic, -1 = never split the contraction, 2 .. 16 = into exactly
+                     that many slices where such a cut exists */
   int clamp;      /* ragged shapes: 0 = automatic, -1 = always the bounds-checked kernels */
   int fold;       /* weight-grad with a hashed_weight too large for LDS: 0 = automatic, 1 = X^T.dY stored
                      tile by tile and folded into dHW by a second kernel whenever possible, 2 = the same
@@ -310,7 +311,8 @@ int rz_weight_grad_planned(const void* X, const void* dY, void* dHW, void* dbias
  * RZ_PLAN_WITH_LAYER_PLAN in flags: answer for a call that carries a layer plan (rz_weight_grad_planned), which
  * changes what the window kernel costs and hence when it is taken.
  * Fills out[8] = { C-tile edge, slices, contracted elements per slice, contracted elements per
- * kernel step, mode, workgroups, workgroups per window of the fold kernel (mode 5, else 0), windows of dHW
+ * kernel step, mode, workgroups, workgroups per window of the fold kernel (mode 5; mode 1: 1 if the kernel
+ * finishes its own tiles, 0 if a second kernel adds the slices up; else 0), windows of dHW
  * (modes 4 and 5, else 0) } with mode 0 = plain store, 1 = split contraction with
  * fp32 partial planes, 2 = weight-grad through LDS images of dHW, 3 = weight-grad by global
  * atomics, 4 = weight-grad by windows of dHW, 5 = weight-grad stored tile by tile and folded

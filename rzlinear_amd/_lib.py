@@ -294,7 +294,8 @@ PLAN_WITH_LAYER_PLAN = 0x100
 def plan_query(op, M, K, N, H, BK, BN, dtype_code_, flags=0, with_dbias=False, planned=False):
     """How the library would carry out a call (rz_plan_query), under the current tuning:
     dict(tile, slices, slice_len, step, mode, workgroups, shares, windows).  op: 0 forward, 1 input-grad,
-    2 weight-grad; planned: the call will carry a layer plan (rz_weight_grad_planned)."""
+    2 weight-grad; planned: the call will carry a layer plan (rz_weight_grad_planned).  For mode "split",
+    shares = 1 says that the kernel finishes its own tiles (no second kernel)."""
     t = _tuning
     if planned:
         flags |= PLAN_WITH_LAYER_PLAN

@@ -298,10 +298,7 @@ static int run_plain_op(int op, int dtype, GemmParams p, const void* bias, void*
       p.partial = (float*)workspace;
       // the slice that arrives last at a tile finishes it (adds the slices in slice order, then the
       // bias: the bits of the second kernel's sum) — unless told otherwise, or out of counters
-      // (the 32 x 64 tile has two wavefronts to read the other slices with: three slices at most — fp32,
-      //  M = 16, K = 4096, N = 11008 input-grad in four slices: 36 -> 39 us)
-      const int most = sp.tile == 32 ? kFinishSlices - 1 : kFinishSlices;
-      p.finish = (tuning.finish != -1 && sp.splits <= most) ? finish_counters_for(tile_count(p.I, p.J, sp.tile)) : nullptr;
+      p.finish = (tuning.finish != -1 && sp.splits <= finish_slices(sp.tile, p.I, p.J)) ? finish_counters_for(tile_count(p.I, p.J, sp.tile)) : nullptr;
       p.bias = p.finish != nullptr ? bias : nullptr;
       if (launch_gemm(dtype, op, p, nullptr, &sp, tuning, s) != hipSuccess) return RZ_ERR_LAUNCH;
       if (p.finish != nullptr) return RZ_OK;
@@ -977,6 +974,7 @@ RZ_API int rz_plan_query(int op, int M, int K, int N, int H, int BK, int BN, int
   const KernelForm f = kernel_form(op, I, J, R, chunk, sp.tile, tile_count(I, J, sp.tile) * sp.splits, eb, t);
   out[0] = sp.tile; out[1] = sp.splits; out[2] = chunk; out[3] = f.step; out[4] = cut ? 1 : 0;
   out[5] = (int32_t)(tile_count(I, J, sp.tile) * sp.splits);
+  out[6] = (cut && t.finish != -1 && sp.splits <= finish_slices(sp.tile, I, J)) ? 1 : 0;
   return RZ_OK;
 }
 

@@ -93,10 +93,8 @@ __host__ __device__ __forceinline__ uint32_t tile_offset(const HashParams& h, ui
 //   weight-grad  I=K J=N R=M   A = X  (rows r=m, contiguous i) B = dY      (rows r=m, contiguous j)
 enum Op { kForward = 0, kInputGrad = 1, kWeightGrad = 2 };
 
-// A cut contraction of at most this many slices is finished by its own kernel (GemmParams::finish):
-// the slice that comes last reads the others' planes by itself, which pays up to here; beyond, a
-// second kernel whose every workgroup shares that reading is faster (bf16, K = N = 10240: three
-// slices at M = 1024 229 -> 212 us; six slices at M = 32 40 -> 52 us).
+// Slices of a cut contraction whose values the kernel that finishes its own tiles holds at a time
+// (GemmParams::finish; see finish_slices in rz_launch.h).
 static constexpr int kFinishSlices = 4;
 
 struct GemmParams {

@@ -1232,35 +1232,39 @@ struct GemmKernel {
 #pragma unroll
           for (int b = 0; b < MJ; b++) {
             const int col = j0 + blk_j(b) + (lane & 31);
-            // (all the other slices' values of the block are fetched before the first is used)
-            float v[kFinishSlices][16];
+            // (half a block at a time: the other slices' values of eight rows are fetched before the first is
+            //  used — a whole block's would cost registers that the two-workgroup forms do not have)
 #pragma unroll
-            for (int sl = 0; sl < kFinishSlices; sl++) {
-              if (sl < slices && sl != by) {   // (uniform)
+            for (int h = 0; h < 2; h++) {
+              float v[kFinishSlices][8];
 #pragma unroll
-                for (int e = 0; e < 16; e++) {
-                  const int row = i0 + blk_i(a) + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
-                  v[sl][e] = (FULL || (row < p.I && col < p.J)) ? load_agent_f32(p.partial + (size_t)sl * plane + (size_t)row * p.J + col) : 0.f;
+              for (int sl = 0; sl < kFinishSlices; sl++) {
+                if (sl < slices && sl != by) {   // (uniform)
+#pragma unroll
+                  for (int e = 0; e < 8; e++) {
+                    const int row = i0 + blk_i(a) + (h * 2 + (e >> 2)) * 8 + (lane >> 5) * 4 + (e & 3);
+                    v[sl][e] = (FULL || (row < p.I && col < p.J)) ? load_agent_f32(p.partial + (size_t)sl * plane + (size_t)row * p.J + col) : 0.f;
+                  }
                 }
               }
-            }
-            float sum[16];
+              float sum[8];
 #pragma unroll
-            for (int e = 0; e < 16; e++) sum[e] = 0.f;
+              for (int e = 0; e < 8; e++) sum[e] = 0.f;
 #pragma unroll
-            for (int sl = 0; sl < kFinishSlices; sl++) {
-              if (sl == by) {
+              for (int sl = 0; sl < kFinishSlices; sl++) {
+                if (sl == by) {
 #pragma unroll
-                for (int e = 0; e < 16; e++) sum[e] += __fmul_rn(acc[a][b][e], p.scale);   // (the product as it was stored: not fused into the add)
-              } else if (sl < slices) {
+                  for (int e = 0; e < 8; e++) sum[e] += __fmul_rn(acc[a][b][h * 8 + e], p.scale);   // (the product as it was stored: not fused into the add)
+                } else if (sl < slices) {
 #pragma unroll
-                for (int e = 0; e < 16; e++) sum[e] += v[sl][e];
+                  for (int e = 0; e < 8; e++) sum[e] += v[sl][e];
+                }
               }
-            }
-            // (the bias joins the fp32 sum as in the second kernel: an add of its own, rounded to fp32,
-            //  not part of a fused multiply-add that rounds straight to the output type)
+              // (the bias joins the fp32 sum as in the second kernel: an add of its own, rounded to fp32,
+              //  not part of a fused multiply-add that rounds straight to the output type)
 #pragma unroll
-            for (int e = 0; e < 16; e++) acc[a][b][e] = __fadd_rn(sum[e], bias[b]);
+              for (int e = 0; e < 8; e++) acc[a][b][h * 8 + e] = __fadd_rn(sum[e], bias[b]);
+            }
           }
         }
         out_scale = 1.f;

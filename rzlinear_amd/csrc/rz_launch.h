@@ -18,7 +18,7 @@ static inline rz_tuning tuning_or_default(const rz_tuning* t) {
 static inline bool tuning_valid(const rz_tuning& t) {
   return (t.tile == 0 || t.tile == 32 || t.tile == 64 || t.tile == 128 || t.tile == 256) && (t.stages == 0 || t.stages == 1) &&
          (t.lds_image == 0 || t.lds_image == -1) && (t.window >= -1 && t.window <= 1) &&
-         (t.split == 0 || t.split == -1) && (t.clamp == 0 || t.clamp == -1) &&
+         (t.split >= -1 && t.split <= 16) && (t.clamp == 0 || t.clamp == -1) &&
          (t.fold >= -1 && t.fold <= 2) && (t.fold_tiles == 0 || t.fold_tiles == -1) && (t.finish == 0 || t.finish == -1) && t.poll_limit >= 0;
 }
 
@@ -98,21 +98,32 @@ static inline double tile_score(int I, int J, int t, int elem_bytes) {
 
 // Relative throughput of `wgs` workgroups of tile t (see tile_score_full, which this restates for
 // a workgroup count that includes the slices of a cut contraction).
-static inline double tile_rate(double wgs, int t, int elem_bytes, double lo64_f32 = 0.60, bool store_f32 = false) {
+// (store_op: the figures of forward / input-grad as they are now — fp32 staged directly, 16-bit fitted
+//  again with them; weight-grad keeps its own)
+static inline double tile_rate(double wgs, int t, int elem_bytes, double lo64_f32 = 0.60, bool store_op = false) {
   const bool f32 = elem_bytes == 4;
-  if (f32 && store_f32) {
+  if (f32 && store_op) {
     // fp32 forward / input-grad, staged directly: every tile runs the MFMA pipe at the 256 tile's rate
     // once its loop is under way, at one workgroup per compute unit already (eight wavefronts); what a
     // smaller tile costs is the longer fill and drain per workgroup, which plan_split prices per slice.
-    return occupancy_rate(wgs, t == 256 ? 1 : (t == 32 ? 4 : 2), 1.0, 1.0);
+    // (the 32 x 64 tile, four wavefronts, needs a second workgroup on the compute unit for that: 0.7 alone —
+    //  M = 8, K = N = 8192: 256 workgroups 51 us, 512 45 us; M = 16, K = 4096, N = 11008: 172 workgroups 46 us,
+    //  688 34 us)
+    if (t == 32) return occupancy_rate(wgs, 4, 0.7, 1.0, 2);
+    // (the 64 tile alone on a compute unit: 0.85 — M = 96, K = N = 4096 in two slices, 256 workgroups: 48 us)
+    return occupancy_rate(wgs, t == 256 ? 1 : 2, t == 64 ? 0.85 : 1.0, 1.0);
   }
   // (32 x 64, four wavefronts: half a 64 workgroup's work in about its time, up to eight resident)
   if (t == 32) return occupancy_rate(wgs, 8, 0.40, 0.80);
+  // (the 16-bit 128 tile in its eight-wavefront form — up to one and a half workgroups per compute unit, see
+  //  kernel_form — has a compute unit to itself and runs at 0.80 there; beyond one per compute unit that
+  //  means a second round: K = N = 10240, M = 128: 80 tiles whole 92 us, in two slices 55, three 43, four 62)
+  if (!f32 && store_op && t == 128 && wgs <= kComputeUnits * 3 / 2) return occupancy_rate(wgs, 1, 0.80, 0.80);
   const int slots = (t == 256) ? 1 : (t == 128 ? 2 : 4);
-  // (the 16-bit 64 tile: 0.24 with one workgroup per compute unit, 0.33 from two on — K = 2048, N = 8192:
-  //  M = 128 14.9 us, M = 256 22.7 us; priced at 0.16 it lost to cut 128 tiles that take 21 and 30 us)
-  const double lo = (t == 256) ? 1.0 : (t == 128 ? (f32 ? 0.86 : 0.51) : (f32 ? lo64_f32 : 0.24));
-  const double hi = (t == 256) ? 1.0 : (t == 128 ? (f32 ? 0.90 : 0.75) : (f32 ? 0.80 : 0.33));
+  // (the 16-bit 64 tile: 0.29 with one workgroup per compute unit, 0.40 from two on — K = N = 10240, M = 128:
+  //  320 workgroups 93 us, 640 68 us; M = 512, K = 4096, N = 1024 in four slices 16 us)
+  const double lo = (t == 256) ? 1.0 : (t == 128 ? (f32 ? 0.86 : 0.51) : (f32 ? lo64_f32 : (store_op ? 0.29 : 0.24)));
+  const double hi = (t == 256) ? 1.0 : (t == 128 ? (f32 ? 0.90 : 0.75) : (f32 ? 0.80 : (store_op ? 0.40 : 0.33)));
   return occupancy_rate(wgs, slots, lo, hi, (t == 64 && !f32) ? 2 : 0);
 }
 
@@ -542,12 +553,28 @@ struct SplitPlan {
   int splits;        // 1 = no split, no workspace
   int r_chunk;
   size_t workspace_bytes;
+  double est_us;     // what the model expects the launch(es) to take
 };
+
+// Slices up to which a cut contraction is finished by its own kernel (GemmParams::finish; 0: never).  The
+// slice that comes last at a tile reads the others' planes by itself, four bytes per lane and load, after
+// an atomic's round trip: that pays up to four slices, where the rows of a tile are real (a batch of
+// fewer rows than the tile has is finished in 3 us by a second kernel too), and with the 256 tile only
+// where the planes are large.  Measured, forward, GPU-bound (finished in the kernel / second kernel):
+// bf16 K = N = 10240: M = 128, 128 tile, three slices 47 / 54 us; M = 32 49 / 46; M = 1024, 256 tile 252 / 260;
+// M = 128, 256 tile 104 / 93.  M = 128, K = 2048, N = 8192: 128 tile, three slices 14.7 / 20.8 us.
+// M = 64, K = N = 4096: 64 tile, four slices 12.7 / 13.6; 128 tile 21.3 / 18.4.  Six slices at M = 32: 52 / 40.
+// The 32 x 64 tile has two wavefronts to read with: two slices.
+static inline int finish_slices(int tile, int I, int J) {
+  if (I < (tile == 32 ? 32 : tile)) return 0;
+  if (tile == 256 && (double)I * J * 4.0 < 16.0e6) return 0;
+  return tile == 32 ? 2 : kFinishSlices;
+}
 
 // Tile and number of slices together: the pair with the least estimated time.  A slice pays the
 // fill and drain of its pipeline (about three steps), the cut pays the fp32 partial planes
 // (written, read back) and the launch of the kernel that adds them.
-static inline SplitPlan plan_split(int I, int J, int R, int elem_bytes, const rz_tuning& t) {
+static inline SplitPlan plan_split(int I, int J, int R, int elem_bytes, const rz_tuning& t, int depth = 0) {
   SplitPlan best = {};
   double best_us = 0.0;
   const double peak = elem_bytes == 4 ? 149e6 : 1150e6;   // flop per microsecond of the 256 tile on a full chip
@@ -578,15 +605,21 @@ static inline SplitPlan plan_split(int I, int J, int R, int elem_bytes, const rz
       // (a kernel of a dozen microseconds is not worth cutting: the second launch and the short loops
       //  cost what the idle compute units would have gained — fp32, M = 32 and 96, K = N = 1024: 13 us
       //  whole, 15 us cut in eight or four)
-      if (want > 1 && direct && whole_us <= 16.0) break;
+      if (want > 1 && direct && whole_us <= 16.0 && t.split <= 0) break;
       const int steps_per = (r_steps + want - 1) / want;
       const int slices = (r_steps + steps_per - 1) / steps_per;
       if (slices != want) continue;                           // (the same cut as a smaller `want`)
-      if (slices > 1 && steps_per * (TR * elem_bytes / 128) < 4) break;   // slices of a few steps are all fill and drain
+      if (t.split > 0 && slices != t.split) continue;         // (an override asks for exactly that many slices)
+      if (slices > 1 && steps_per * (TR * elem_bytes / 128) < 4 && t.split <= 0) break;   // slices of a few steps are all fill and drain
       const double steps = (double)steps_per * (TR * elem_bytes / 128);
-      const double rate = peak * tile_rate((double)tiles * slices, tile, elem_bytes, lo64, direct) * useful * steps / (steps + fill);
+      const double rate = peak * tile_rate((double)tiles * slices, tile, elem_bytes, lo64, direct || elem_bytes == 2) * useful * steps / (steps + fill);
       double us = 2.0 * (double)I * (double)J * (double)R / rate + 4.0;
-      if (slices > 1) us += (2.0 * slices * (double)I * J * 4.0 + (double)I * J * elem_bytes) / 4.0e6 + (direct ? 3.0 : 4.0);
+      // (up to finish_slices the kernel finishes its own tiles: every plane is written, all but one are read
+      //  back by the finishing workgroups, and no second kernel is launched — worth a couple of microseconds
+      //  and a plane; fp32, M = 16384, K = 512, N = 1024 input-grad, planes of 33 MB: the 256 tile in two
+      //  slices 155 us against the whole 128 tile's 136)
+      if (slices > 1 && slices <= finish_slices(tile, I, J) && t.finish != -1) us += (2.0 * slices - 1.0) * (double)I * J * 4.0 / 4.0e6 + 2.0;
+      else if (slices > 1) us += (2.0 * slices * (double)I * J * 4.0 + (double)I * J * elem_bytes) / 4.0e6 + (direct ? 3.0 : 4.0);
       else whole_us = us;
       // (near ties go to the larger tile and the fewer slices, which come first)
       if (best.tile == 0 || us < best_us * 0.97) {
@@ -597,7 +630,21 @@ static inline SplitPlan plan_split(int I, int J, int R, int elem_bytes, const rz
       }
     }
   }
+  // (16-bit: a problem that some tile does whole in a dozen microseconds is not cut — M = 128, K = N = 1024:
+  //  64 tile whole 10.2 us; every cut, finished in the kernel or not, 12 to 16 us)
+  if (elem_bytes == 2 && t.split == 0 && best.splits > 1 && depth == 0) {
+    rz_tuning whole_only = t;
+    whole_only.split = -1;
+    const SplitPlan w = plan_split(I, J, R, elem_bytes, whole_only, 1);
+    if (w.est_us <= 14.0) return w;
+  }
+  if (best.tile == 0 && t.split > 0) {   // (no cut comes out at exactly that many slices: the library's own choice)
+    rz_tuning free_cut = t;
+    free_cut.split = 0;
+    return plan_split(I, J, R, elem_bytes, free_cut);
+  }
   best.workspace_bytes = best.splits > 1 ? (size_t)best.splits * (size_t)I * (size_t)J * sizeof(float) : 0;
+  best.est_us = best_us;
   return best;
 }
 

@@ -23,14 +23,14 @@ PLANS = {
     "rec_mlp bf16": ((16384, 512, 1024, 5243, 64, 64, BF16), [(256, 1, "store"), (128, 1, "store"), (128, 8, "lds_image")]),
     "ffn bf16": ((8192, 4096, 16384, 67109, 64, 64, BF16), [(256, 1, "store"), (256, 1, "store"), (256, 1, "fold")]),
     "collision fp32": ((32768, 2048, 2048, 32768, 64, 64, F32), [(256, 1, "store"), (256, 1, "store"), (256, 4, "lds_image")]),
-    "grid_32_1024 fp32": ((32, 1024, 1024, 65536, 32, 64, F32), [(32, 1, "store"), (32, 1, "store"), (64, 1, "fold")]),
-    "grid_32_1024 bf16": ((32, 1024, 1024, 65536, 32, 64, BF16), [(64, 4, "split"), (64, 4, "split"), (64, 1, "fold")]),
+    "grid_32_1024 fp32": ((32, 1024, 1024, 65536, 32, 64, F32), [(32, 6, "split"), (32, 6, "split"), (64, 1, "fold")]),
+    "grid_32_1024 bf16": ((32, 1024, 1024, 65536, 32, 64, BF16), [(64, 1, "store"), (64, 1, "store"), (64, 1, "fold")]),
     "grid_32_10240 fp32": ((32, 10240, 10240, 6553600, 32, 64, F32), [(32, 3, "split"), (32, 3, "split"), (0, 1, "window")]),
-    "grid_32_10240 bf16": ((32, 10240, 10240, 6553600, 32, 64, BF16), [(128, 6, "split"), (128, 6, "split"), (0, 1, "window")]),
+    "grid_32_10240 bf16": ((32, 10240, 10240, 6553600, 32, 64, BF16), [(128, 3, "split"), (128, 3, "split"), (0, 1, "window")]),
     "grid_128_1024 fp32": ((128, 1024, 1024, 65536, 32, 64, F32), [(64, 6, "split"), (64, 6, "split"), (64, 1, "fold")]),
-    "grid_128_1024 bf16": ((128, 1024, 1024, 65536, 32, 64, BF16), [(64, 3, "split"), (64, 3, "split"), (64, 1, "fold")]),
+    "grid_128_1024 bf16": ((128, 1024, 1024, 65536, 32, 64, BF16), [(64, 1, "store"), (64, 1, "store"), (64, 1, "fold")]),
     "grid_128_10240 fp32": ((128, 10240, 10240, 6553600, 32, 64, F32), [(128, 3, "split"), (128, 3, "split"), (0, 1, "window")]),
-    "grid_128_10240 bf16": ((128, 10240, 10240, 6553600, 32, 64, BF16), [(128, 6, "split"), (128, 6, "split"), (0, 1, "window")]),
+    "grid_128_10240 bf16": ((128, 10240, 10240, 6553600, 32, 64, BF16), [(128, 3, "split"), (128, 3, "split"), (0, 1, "window")]),
     "grid_1024_1024 fp32": ((1024, 1024, 1024, 65536, 32, 64, F32), [(64, 1, "store"), (64, 1, "store"), (64, 1, "fold")]),
     "grid_1024_1024 bf16": ((1024, 1024, 1024, 65536, 32, 64, BF16), [(64, 1, "store"), (64, 1, "store"), (64, 1, "fold")]),
     "grid_1024_10240 fp32": ((1024, 10240, 10240, 6553600, 32, 64, F32), [(64, 1, "store"), (64, 1, "store"), (128, 1, "fold")]),
