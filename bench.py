@@ -74,14 +74,14 @@ TRAFFIC = {
     #  FETCH_SIZE = 131085, WRITE_SIZE = 262144)
     ("square4096", "bf16"): {
         "profile": "profiles/rz_gemm_bf16_square4096.txt",
-        "bytes": {"forward": int((16680.8 * 2.0 + 32768.0) * 1024),       # algorithmic: 64.03 MiB
-                  "input_grad": int((16666.7 * 2.0 + 32768.0) * 1024),
-                  "weight_grad": int((98456.4 * 2.0 + 16784.8) * 1024)},  # X, dY re-read by the XCDs' tile groups; + partial images
+        "bytes": {"forward": int((16679.6 * 2.0 + 32768.0) * 1024),       # algorithmic: 64.03 MiB
+                  "input_grad": int((16676.4 * 2.0 + 32768.0) * 1024),
+                  "weight_grad": int((98478.0 * 2.0 + 16784.6) * 1024)},  # X, dY re-read by the XCDs' tile groups; + partial images
     },
     ("square2048", "bf16"): {
         "profile": "profiles/rz_gemm_bf16_square2048.txt",
-        "bytes": {"forward": int((4344.7 * 2.0 + 8192.0) * 1024), "input_grad": int((4344.5 * 2.0 + 8192.0) * 1024),
-                  "weight_grad": int((24694.3 * 2.0 + 16384.0) * 1024)},
+        "bytes": {"forward": int((4349.3 * 2.0 + 8192.0) * 1024), "input_grad": int((4342.2 * 2.0 + 8192.0) * 1024),
+                  "weight_grad": int((24699.1 * 2.0 + 16384.0) * 1024)},
     },
     ("square4096", "fp32"): {
         "profile": "profiles/rz_gemm_fp32_square4096.txt",
