@@ -134,6 +134,31 @@ def test_status_codes(lib):
     assert lib.rz_status_string(-99) == b"unknown status"
 
 
+def test_tuning_overrides_of_the_cut_and_of_the_fold_tiles(lib):
+    """rz_tuning.split = n asks for exactly n slices (the library's own choice where no such cut exists),
+    rz_tuning.finish = -1 sends a cut to the second kernel, rz_tuning.fold_tiles = -1 keeps fp32 tiles;
+    values outside their ranges are refused."""
+    from rzlinear_amd import _lib
+    out = (ctypes.c_int32 * 8)()
+    shape = (128, 2048, 8192, 16384, 64, 64)
+    for n in (2, 3, 4, 6):
+        t = _lib.Tuning(tile=128, split=n)
+        assert lib.rz_plan_query(0, *shape, 1, 0, 0, ctypes.byref(t), out) == 0
+        assert (out[0], out[1], out[4]) == (128, n, 1)
+        assert out[1] * out[2] >= 2048 and out[2] % out[3] == 0
+        assert out[6] == (1 if n <= 4 else 0)          # up to four slices the kernel finishes its own tiles
+        t = _lib.Tuning(tile=128, split=n, finish=-1)
+        assert lib.rz_plan_query(0, *shape, 1, 0, 0, ctypes.byref(t), out) == 0 and out[6] == 0
+    # a batch smaller than the tile goes to the second kernel
+    t = _lib.Tuning(tile=128, split=3)
+    assert lib.rz_plan_query(0, 32, 2048, 8192, 16384, 64, 64, 1, 0, 0, ctypes.byref(t), out) == 0 and (out[1], out[6]) == (3, 0)
+    # 64 steps of K = 2048 cannot make 13 slices of whole steps that are all used: the library's own cut
+    t = _lib.Tuning(tile=64, split=13)
+    assert lib.rz_plan_query(0, 128, 2048, 8192, 16384, 64, 64, 0, 0, 0, ctypes.byref(t), out) == 0 and out[1] != 13
+    for bad in (_lib.Tuning(split=17), _lib.Tuning(split=-2), _lib.Tuning(finish=1), _lib.Tuning(fold_tiles=1), _lib.Tuning(fold_tiles=-2)):
+        assert lib.rz_plan_query(0, *shape, 1, 0, 0, ctypes.byref(bad), out) == -9
+
+
 def test_plan_slices_begin_on_step_boundaries(lib):
     """Every slice of a cut contraction must start on a boundary of the kernel's step: a step's
     table of tile offsets assumes that the step lies inside one hashed tile or covers whole
