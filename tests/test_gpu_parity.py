@@ -241,6 +241,39 @@ def test_the_last_slice_to_arrive_finishes_the_tile(oracle, case, dtype):
     assert_close(f(dxs[0]), oracle.input_grad(dy64, hw64, K, BK, BN, R1024, 0.5), dtype, "dX")
 
 
+def test_finishing_slices_read_what_this_launch_wrote():
+    """The slice that finishes a tile reads the other slices' planes out of a workspace that earlier calls
+    have filled with other values: alternating between two inputs over the same workspace, every call must
+    give its own input's result (the bits of the two-kernel form), never a mixture with the call before."""
+    import ctypes
+    from rzlinear_amd import _lib
+    lib = _lib.load()
+    M, K, N, H, BK, BN = 256, 4096, 2048, 70000, 64, 64
+    R = (ctypes.c_int32 * 8)(*R1024)
+    stream = torch.cuda.current_stream().cuda_stream
+    for dtype, code in ((torch.bfloat16, _lib.RZ_BF16), (torch.float32, _lib.RZ_F32)):
+        fin = _lib.Tuning(tile=128, split=4)
+        two = _lib.Tuning(tile=128, split=4, finish=-1)
+        out = (ctypes.c_int32 * 8)()
+        assert lib.rz_plan_query(0, M, K, N, H, BK, BN, code, 0, 0, ctypes.byref(fin), out) == 0 and (out[1], out[6]) == (4, 1)
+        need = lib.rz_forward_hashed_workspace_bytes(M, K, N, H, BK, BN, code, ctypes.byref(fin))
+        ws = torch.empty((need,), dtype=torch.uint8, device="cuda")
+        inputs = [make_inputs(M, K, N, H, dtype, seed=s)[0] for s in (21, 22)]
+        _say("finishing slices, alternating inputs", dtype)
+
+        def forward(x, hw, tuning):
+            y = torch.full((M, N), float("nan"), dtype=dtype, device="cuda")
+            _lib.check(lib.rz_forward_hashed(x.data_ptr(), hw.data_ptr(), None, y.data_ptr(), ws.data_ptr(), need, M, K, N, H,
+                                             BK, BN, R, 2, 1.0, K, N, code, ctypes.byref(tuning), stream))
+            return y
+        want = [forward(x, hw, two) for (x, hw, _) in inputs]
+        torch.cuda.synchronize()
+        assert not torch.equal(want[0], want[1])
+        for i in range(8):
+            x, hw, _ = inputs[i % 2]
+            assert torch.equal(forward(x, hw, fin), want[i % 2]), (dtype, i)
+
+
 @pytest.mark.parametrize("M", [32, 96, 160, 288])
 def test_the_32_row_tile_is_chosen_where_64_rows_would_be_half_padding(oracle, M):
     """K = N = 4096, fp32: the plan takes the 32 x 64 tile by itself for these batch sizes (and not for
