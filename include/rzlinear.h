@@ -279,10 +279,11 @@ int rz_weight_grad_hashed(const void* X, const void* dY, void* dHW, void* dbias,
 /*
  * Layer plan: the part of a weight-grad call that depends only on the layer — K, N, H, the tile
  * and the hash constants — and not on the batch: where every W tile starts in hashed_weight and,
- * for every window of dHW that the window kernel works on, the ordered list of tile strips that
- * land in it.  Without a plan every weight-grad call on a large hashed_weight hashes the tile
- * offsets again and every workgroup searches them for its strips (some 25 us of an 85 us call at
- * M = 32, K = N = 10240); with one it reads its list.  The result is the same bit for bit.
+ * for every window of dHW that the window kernel or the fold kernel works on, the ordered list of
+ * tile strips (of tiles) that land in it.  Without a plan every weight-grad call on a large
+ * hashed_weight hashes the tile offsets again and every workgroup searches them for its strips or
+ * tiles (some 25 us of an 85 us call at M = 32, K = N = 10240; 5 us of the fold kernel's 60 to 90);
+ * with one it reads its list.  The result is the same bit for bit.
  *   rz_layer_plan_bytes   size of the plan (0: bad arguments)
  *   rz_layer_plan_build   fills plan_host[plan_bytes] on the HOST (no device is touched); the
  *                         caller copies it to device memory once and keeps it with the layer

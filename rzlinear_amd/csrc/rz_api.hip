@@ -515,9 +515,15 @@ static int weight_grad_impl(const void* X, const void* dY, void* dHW, void* dbia
     FoldParams fp;
     fp.tiles = p.tiles_out;
     fp.plan_header = nullptr;
+    fp.plan_start = nullptr;
+    fp.plan_list = nullptr;
     if (planned) {
       fp.offsets = layer_plan + lay.offsets_at;
       fp.plan_header = layer_plan;
+      if (!f.small && lay.fold_windows == f.windows && lay.fold_window == f.window) {
+        fp.plan_start = layer_plan + lay.fold_start_at;
+        fp.plan_list = layer_plan + lay.fold_list_at;
+      }
     } else if (f.small) {
       fp.offsets = nullptr;   // (the kernel hashes the few offsets it needs)
     } else {
@@ -915,9 +921,34 @@ RZ_API int rz_layer_plan_build(void* plan_host, size_t plan_bytes, int K, int N,
     for (int b = l.windows; b > 0; b--) start[b] = start[b - 1];
     start[0] = 0;
   }
+  {
+    // The fold kernel's lists, by the same counting sort.  The tiles are visited in the order in which the
+    // kernel's own search numbers them (pass by pass of kFoldScan * kFoldThreads tile indices; inside a pass
+    // thread by thread, and tile t + 1024 j of the pass is bit j of thread t), so that a window's tiles are
+    // added in the same order, and come out in the same bits, with a plan and without.
+    int32_t* start = w + l.fold_start_at;
+    int32_t* list = w + l.fold_list_at;
+    const long long E = (long long)BK * BN;
+    auto for_each_pair = [&](auto&& f) {
+      for (int first = 0; first < l.tiles; first += kFoldScan * kFoldThreads)
+        for (int t = 0; t < kFoldThreads; t++)
+          for (int j = 0; j < kFoldScan; j++) {
+            const long long id = (long long)first + t + (long long)j * kFoldThreads;
+            if (id >= l.tiles) break;
+            const long long off = offsets[id];
+            for (long long b = off / l.fold_window; b <= (off + E - 1) / l.fold_window && b < l.fold_windows; b++) f((int)b, (int)id);
+          }
+    };
+    for_each_pair([&](int b, int) { start[b + 1]++; });
+    for (int b = 0; b < l.fold_windows; b++) start[b + 1] += start[b];
+    if (start[l.fold_windows] > l.fold_capacity) return RZ_ERR_BAD_ARGUMENT;   // (cannot happen: see layer_plan_layout)
+    for_each_pair([&](int b, int id) { list[start[b]++] = id; });
+    for (int b = l.fold_windows; b > 0; b--) start[b] = start[b - 1];
+    start[0] = 0;
+  }
   const int32_t header[kLayerPlanHeader] = {kLayerPlanMagic, kLayerPlanVersion, K, N, H, BK, BN, hash_levels, l.tiles,
                                             l.windows, l.window, (int32_t)entries, l.strips_per_tile,
-                                            layer_plan_hash_sum(h), 0, 0};
+                                            layer_plan_hash_sum(h), l.fold_windows, l.fold_window};
   for (int i = 0; i < kLayerPlanHeader; i++) w[i] = header[i];
   return RZ_OK;
 }

@@ -7,21 +7,22 @@
 //
 // A hashed tile is BK*BN contiguous elements of hashed_weight and BK*BN contiguous floats of the
 // tile-by-tile buffer, so its reads are whole cache lines whatever its offset.  The list holds
-// the tiles in runs of at most 2048 floats.  The window is cut into blocks of 256 positions;
+// the tiles in runs of at most 2048 elements.  The window is cut into blocks of 256 positions (of
+// 512 where the tiles are kept in a 16-bit type): sixteen bytes of tile elements per lane;
 // wavefront w owns the blocks w, w + 16, w + 32, ..., and inside a block lane l owns the four
-// positions 4 l .. 4 l + 3.  A run meets at most nine blocks in a row, so at most one of a
+// (eight) positions from 4 l (8 l) on.  A run meets at most nine blocks in a row, so at most one of a
 // wavefront's: the wavefront walks down the list, skips the runs that miss its blocks, and for
-// each of the others reads the 256 floats that fall on its block with ONE 16-byte load per lane
-// (from a scalar base: the run starts anywhere, on a 4-byte boundary) and adds them with one
-// 16-byte LDS read, four additions and one 16-byte LDS write per lane.  What a run needs per
+// each of the others reads the elements that fall on its block with ONE 16-byte load per lane
+// (from a scalar base: the run starts anywhere, on an element's boundary) and adds them with
+// 16-byte LDS reads, additions and 16-byte LDS writes.  What a run needs per
 // wavefront is scalar arithmetic; no two lanes ever touch the same LDS word, so the wavefronts
 // need no barrier between runs and each goes down the list at its own pace.  Only the blocks
 // at the two ends of a run, and runs of tiles that stick out of K x N (whose buffer holds floats
 // that the contraction never wrote), need their elements masked one by one: a branch of its
 // own; there, lanes wholly outside the run re-fetch floats of the run, so that a block costs no
-// memory traffic beyond the run's own cache lines.  The loads reach up to three floats before
-// and after a run (an empty slot of a round reads the buffer's first kilobyte): the buffer is
-// allocated with a margin on both sides.
+// memory traffic beyond the run's own cache lines.  The loads reach up to one element short of
+// sixteen bytes before and after a run (an empty slot of a round reads the buffer's first kilobyte):
+// the buffer is allocated with a margin on both sides.
 //
 // A window is at most 32768 floats (128 KB of LDS).  When hashed_weight has fewer windows than
 // the chip has compute units, `shares` workgroups share a window: each takes an equal part of the
@@ -42,6 +43,8 @@ struct FoldParams {
   const int32_t* offsets;   // [tiles_k * tiles_n] where every tile starts in hashed_weight (hashed once, by another kernel;
                             // null for the few-tiles kernel: it hashes them itself)
   const int32_t* plan_header;   // `offsets` belongs to a layer plan (else null): its header, checked against this call's
+  const int32_t* plan_start;    // the plan's list of every window's tiles (else null: the kernel looks for them): [windows + 1] ...
+  const int32_t* plan_list;     // ... and the tile indices, in the order in which the kernel's own search numbers them
   float* partial;       // [shares][pitch]: every workgroup writes its window of its share's image ...
   void* out;            // ... or, with a single share (partial == null), its window of dHW itself:
   int out_dtype;        //     an rz_dtype code,
@@ -60,7 +63,7 @@ static constexpr int kFoldScan = 64;         // tile indices per thread and list
 static constexpr int kFoldWindowMax = 32768;
 static constexpr int kFoldRun = 2048;        // floats of a run at most (tiles are powers of two: whole runs)
 static constexpr int kFoldRound = 8;         // runs whose loads a wavefront issues together
-static constexpr int kFoldBlock = 256;       // window positions of a wavefront's block: four per lane
+// (a wavefront's block of window positions: sixteen bytes of tile elements per lane — see FoldRaw)
 
 static inline size_t fold_lds_bytes(int window) {
   return (size_t)window * sizeof(float) + 3 * kFoldList * sizeof(int) + 32 * sizeof(int);
@@ -68,26 +71,33 @@ static inline size_t fold_lds_bytes(int window) {
 
 typedef float fold_f4 __attribute__((ext_vector_type(4)));
 typedef float fold_f4u __attribute__((ext_vector_type(4), aligned(4)));
-typedef uint16_t fold_h4 __attribute__((ext_vector_type(4)));
-typedef uint16_t fold_h4u __attribute__((ext_vector_type(4), aligned(2)));
+typedef uint16_t fold_h8 __attribute__((ext_vector_type(8)));
+typedef uint16_t fold_h8u __attribute__((ext_vector_type(8), aligned(2)));
 
-// Four consecutive tile elements as they lie in memory (TT = float, bf16_t or f16_t), and as floats.
-template <typename TT> struct FoldRaw { typedef fold_h4 type; typedef fold_h4u unaligned; };
-template <> struct FoldRaw<float> { typedef fold_f4 type; typedef fold_f4u unaligned; };
+// The sixteen bytes of consecutive tile elements that a lane loads at a time, as they lie in memory
+// (TT = float: four, bf16_t or f16_t: eight), and as floats.
+template <typename TT> struct FoldRaw {
+  typedef fold_h8 type;
+  typedef fold_h8u unaligned;
+  static constexpr int kPer = 8;
+};
+template <> struct FoldRaw<float> {
+  typedef fold_f4 type;
+  typedef fold_f4u unaligned;
+  static constexpr int kPer = 4;
+};
 template <typename TT>
-__device__ __forceinline__ fold_f4 fold_widen(typename FoldRaw<TT>::type raw) {
-  if constexpr (sizeof(TT) == 4) {
-    return raw;
-  } else {
-    fold_f4 v;
+__device__ __forceinline__ void fold_widen(typename FoldRaw<TT>::type raw, float* v) {
 #pragma unroll
-    for (int f = 0; f < 4; f++) {
+  for (int f = 0; f < FoldRaw<TT>::kPer; f++) {
+    if constexpr (sizeof(TT) == 4) {
+      v[f] = raw[f];
+    } else {
       TT e;
       const uint16_t bits = raw[f];
       __builtin_memcpy(&e, &bits, 2);
       v[f] = ElemTraits<TT>::to_float(e);
     }
-    return v;
   }
 }
 
@@ -100,7 +110,10 @@ __global__ __launch_bounds__(kFoldThreads) void fold_tiles_kernel(const FoldPara
   int* list_lim = list_rel + kFoldList;                          // (rows - 1) | (columns - 1) << 14 of the tile inside K x N | run << 28
   int* wave_sum = list_lim + kFoldList;                          // [16] per-wavefront counts, [16] = total
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int lane4 = lane * 4;
+  constexpr int kPer = FoldRaw<TT>::kPer;          // window positions of a lane inside a block
+  constexpr int kFoldBlock = 64 * kPer;            // ... and of the block: 256 or 512
+  constexpr int kBlockShift = kPer == 4 ? 8 : 9;
+  const int lane_e = lane * kPer;
   const unsigned lane16 = lane * 16;
   const int win = blockIdx.x % p.windows, share = blockIdx.x / p.windows;
   const int w0 = win * p.window;
@@ -112,7 +125,9 @@ __global__ __launch_bounds__(kFoldThreads) void fold_tiles_kernel(const FoldPara
   const int full_lim = (p.h.BK - 1) | (p.h.BN - 1) << 14;
   // Offsets from a plan that was built for another layer, tile or hash would be in range and
   // wrong: then the image is NaN and nothing is added (what the output paths below store).
-  const bool plan_ok = p.plan_header == nullptr || layer_plan_matches(p.plan_header, p.K, p.N, p.H, p.h);   // (uniform)
+  const bool plan_ok = p.plan_header == nullptr ||
+                       (layer_plan_matches(p.plan_header, p.K, p.N, p.H, p.h) &&
+                        (p.plan_list == nullptr || (p.plan_header[14] == p.windows && p.plan_header[15] == p.window)));   // (uniform)
   for (int q = tid; q < p.window; q += kFoldThreads) img[q] = plan_ok ? 0.f : __builtin_nanf("");   // (own positions only)
 
   // bit j: tile first + i + 1024 j (below `stop`) lands in the window.  The offsets are fetched
@@ -167,16 +182,149 @@ __global__ __launch_bounds__(kFoldThreads) void fold_tiles_kernel(const FoldPara
   // wavefront, thread by thread, bit by bit of the thread's mask.  A share takes an equal part of
   // the numbers, so the workgroups of a window have the same work to within a tile whatever the
   // hash does, and — every share numbering alike — their parts are a partition of the window's tiles.
+  const int cap = kFoldList / per_tile;    // tiles whose runs the list holds at a time (at least four)
+  // the runs of tile `id`, the at-th tile of the list
+  auto put = [&](int at, int id) {
+    const int rel = p.offsets[id] - w0;
+    const int tk = id / p.tiles_n, tn = id - tk * p.tiles_n;
+    const int rows = (p.K - tk * p.h.BK) < p.h.BK ? (p.K - tk * p.h.BK) : p.h.BK;
+    const int cols = (p.N - tn * p.h.BN) < p.h.BN ? (p.N - tn * p.h.BN) : p.h.BN;
+    for (int s = 0; s < p.slices; s++)
+      for (int c = 0; c < runs; c++) {
+        const int slot = (at * p.slices + s) * runs + c;
+        list_at[slot] = ((s * ntiles + id) << eshift) + c * run;
+        list_rel[slot] = rel + c * run;
+        list_lim[slot] = (rows - 1) | (cols - 1) << 14 | c << 28;
+      }
+  };
+  auto walk = [&](int total) {
+    // --- add the listed runs into the window ---------------------------------------------------
+    // Every wavefront on its own: lane u holds entry u of a chunk of 64 list entries; the entries
+    // that meet one of the wavefront's blocks are taken in list order, in rounds of kFoldRound;
+    // the next round's loads are in flight while this round's values are added.  What describes
+    // an entry to the wavefront is uniform (scalar registers).
+    struct Round {
+      typename FoldRaw<TT>::type v[kFoldRound];   // (as loaded: widened when added, so that the loads stay in flight)
+      int pos[kFoldRound];   // window position of the block
+      int e0[kFoldRound];    // float of the run that falls on the block's first position (-255 .. run - 1)
+      int lim[kFoldRound];   // the entry's, -1: no entry
+    };
+    unsigned long long todo = 0ull;   // entries of the chunk that this wavefront still has to add
+    int next = 0;                     // first list entry behind the chunk
+    int c_pos = 0, c_e0 = 0, c_off = 0, c_lim = 0;
+    auto refill = [&]() {
+      while (todo == 0ull && next < total) {   // (uniform)
+        const int t = next + lane;
+        const bool have = t < total;
+        const int rel = have ? list_rel[t] : 0, at = have ? list_at[t] : 0;
+        c_lim = have ? list_lim[t] : 0;
+        const int first = rel >> kBlockShift;          // (arithmetic shift: the block of the run's first float)
+        const int b = first + ((wave - first) & 15);   // the wavefront's only block among the sixteen from there on
+        c_pos = b * kFoldBlock;
+        c_e0 = c_pos - rel;
+        c_off = at + c_e0;
+        todo = __ballot(have && b >= 0 && c_pos < wlen && c_e0 < run);
+        next += 64;
+      }
+    };
+    auto issue = [&](Round& r) {
+#pragma unroll
+      for (int u = 0; u < kFoldRound; u++) {
+        const bool any = todo != 0ull;
+        const int src = any ? (int)__builtin_ctzll(todo) : 0;
+        todo &= todo - 1ull;
+        const int off = __builtin_amdgcn_readlane(c_off, src), lim = __builtin_amdgcn_readlane(c_lim, src);
+        r.pos[u] = __builtin_amdgcn_readlane(c_pos, src);
+        r.e0[u] = __builtin_amdgcn_readlane(c_e0, src);
+        r.lim[u] = any ? lim : -1;
+        // (every slot loads, an empty one the buffer's first floats: with no branch around the
+        //  loads their number is fixed, and the wait for this round's values can leave the next
+        //  round's in flight)
+        const char* first = reinterpret_cast<const char*>(p.tiles) + (any ? (long long)off : 0ll) * (long long)sizeof(TT);   // (scalar)
+        unsigned mine = lane16;   // offset of the lane's elements from the block's first, in bytes
+        if (any && (r.e0[u] < 0 || r.e0[u] + kFoldBlock > run)) {   // (uniform) an end of the run:
+          // lanes that lie wholly outside the run fetch floats of the run that other lanes fetch
+          // anyway (their values count as zero below) instead of a neighbouring tile's
+          const int e = r.e0[u] + lane_e;
+          const int inside = e <= -kPer ? 0 : (e >= run ? max(run - kPer, r.e0[u]) : e);
+          mine = (unsigned)(inside - r.e0[u]) * (unsigned)sizeof(TT);
+        }
+        // (read once and never again: a load that leaves the caches to the offsets and to the
+        //  contraction's stores still on their way to memory — K = N = 10240: 129 -> 111 us)
+        r.v[u] = __builtin_nontemporal_load(reinterpret_cast<const typename FoldRaw<TT>::unaligned*>(
+            first + mine));
+      }
+    };
+    // (plain read-add-write: LDS float atomics are several times slower, and nobody else touches
+    //  this lane's words; runs that overlap are added one after the other, in list order)
+    auto add = [&](const Round& r) {
+#pragma unroll
+      for (int u = 0; u < kFoldRound; u++) {
+        if (r.lim[u] == -1) continue;   // (uniform)
+        float v[kPer];
+        fold_widen<TT>(r.v[u], v);
+        const int lim = r.lim[u];
+        if (r.e0[u] < 0 || r.e0[u] + kFoldBlock > run) {   // (uniform) an end of the run: what is not the run's counts as zero
+          const unsigned e = (unsigned)(r.e0[u] + lane_e);   // (a float before the run wraps round to a large number)
+#pragma unroll
+          for (int f = 0; f < kPer; f++) v[f] = e + (unsigned)f < (unsigned)run ? v[f] : 0.f;
+        }
+        if ((lim & 0x0fffffff) != full_lim) {   // (uniform) a tile that sticks out of K x N: what lies outside was never written
+          asm volatile("" ::: "memory");   // (keeps this arithmetic out of the common path)
+          const int rows = (lim & 0x3fff) + 1, cols = ((lim >> 14) & 0x3fff) + 1, base = (lim >> 28) * run;
+#pragma unroll
+          for (int f = 0; f < kPer; f++) {
+            const int in_tile = base + r.e0[u] + lane_e + f;
+            const bool ok = ((in_tile >> p.h.bn_shift) < rows) & ((in_tile & (p.h.BN - 1)) < cols);
+            v[f] = ok ? v[f] : 0.f;
+          }
+        }
+        fold_f4* at = reinterpret_cast<fold_f4*>(img + r.pos[u] + lane_e);
+#pragma unroll
+        for (int g = 0; g < kPer / 4; g++) {
+          fold_f4 w = at[g];
+#pragma unroll
+          for (int f = 0; f < 4; f++) w[f] += v[4 * g + f];
+          at[g] = w;
+        }
+      }
+    };
+    Round r0, r1;
+    refill();
+    issue(r0);
+    while (true) {   // (uniform per wavefront; no barrier inside)
+      refill();
+      issue(r1);
+      add(r0);
+      if (r1.lim[0] == -1) break;   // (entries fill a round from its first slot)
+      refill();
+      issue(r0);
+      add(r1);
+      if (r0.lim[0] == -1) break;
+    }
+  };
+
+  if (p.plan_list != nullptr) {
+    // The layer plan lists the window's tiles, numbered as below: nothing to look for.
+    const int begin = p.plan_start[win], all = plan_ok ? p.plan_start[win + 1] - begin : 0;
+    const int want_lo = (int)((long long)share * all / p.shares), want_hi = (int)((long long)(share + 1) * all / p.shares);
+    for (int chunk_lo = want_lo; chunk_lo < want_hi; chunk_lo += cap) {   // (uniform)
+      const int chunk_hi = (chunk_lo + cap) < want_hi ? (chunk_lo + cap) : want_hi;
+      if (chunk_lo != want_lo) __syncthreads();   // (the wavefronts are done reading the previous chunk's list)
+      for (int q = chunk_lo + tid; q < chunk_hi; q += kFoldThreads) put(q - chunk_lo, p.plan_list[begin + q]);
+      __syncthreads();
+      walk((chunk_hi - chunk_lo) * per_tile);
+    }
+  }
   int rank_lo = 0, rank_hi = 0x7fffffff;
-  if (p.shares > 1) {
+  if (p.shares > 1 && p.plan_list == nullptr) {
     int mine = 0, before;
     for (int first = 0; first < ntiles; first += kFoldScan * kFoldThreads) mine += __popcll(scan(first, ntiles));
     const int all = total_of(wave_scan(mine), &before);
     rank_lo = (int)((long long)share * all / p.shares);
     rank_hi = (int)((long long)(share + 1) * all / p.shares);
   }
-  const int cap = kFoldList / per_tile;    // tiles whose runs the list holds at a time (at least four)
-  int lo = plan_ok ? 0 : ntiles, seen = 0;   // tiles [0, lo) hold `seen` tiles of the window
+  int lo = plan_ok && p.plan_list == nullptr ? 0 : ntiles, seen = 0;   // tiles [0, lo) hold `seen` tiles of the window
   while (lo < ntiles && seen < rank_hi) {   // (uniform: every thread of the workgroup goes round together)
     const int span = (ntiles - lo) < kFoldScan * kFoldThreads ? (ntiles - lo) : kFoldScan * kFoldThreads;
     const unsigned long long pass_mask = scan(lo, lo + span);
@@ -200,116 +348,11 @@ __global__ __launch_bounds__(kFoldThreads) void fold_tiles_kernel(const FoldPara
       while (mask != 0ull) {
         const int j = __ffsll((long long)mask) - 1;
         mask &= mask - 1ull;
-        if (rank >= chunk_lo && rank < chunk_hi) {
-          const int id = lo - span + tid + j * kFoldThreads;
-          const int rel = p.offsets[id] - w0;
-          const int tk = id / p.tiles_n, tn = id - tk * p.tiles_n;
-          const int rows = (p.K - tk * p.h.BK) < p.h.BK ? (p.K - tk * p.h.BK) : p.h.BK;
-          const int cols = (p.N - tn * p.h.BN) < p.h.BN ? (p.N - tn * p.h.BN) : p.h.BN;
-          for (int s = 0; s < p.slices; s++)
-            for (int c = 0; c < runs; c++) {
-              const int slot = ((rank - chunk_lo) * p.slices + s) * runs + c;
-              list_at[slot] = ((s * ntiles + id) << eshift) + c * run;
-              list_rel[slot] = rel + c * run;
-              list_lim[slot] = (rows - 1) | (cols - 1) << 14 | c << 28;
-            }
-        }
+        if (rank >= chunk_lo && rank < chunk_hi) put(rank - chunk_lo, lo - span + tid + j * kFoldThreads);
         rank++;
       }
       __syncthreads();
-      // --- add the listed runs into the window ---------------------------------------------------
-      // Every wavefront on its own: lane u holds entry u of a chunk of 64 list entries; the entries
-      // that meet one of the wavefront's blocks are taken in list order, in rounds of kFoldRound;
-      // the next round's loads are in flight while this round's values are added.  What describes
-      // an entry to the wavefront is uniform (scalar registers).
-      struct Round {
-        typename FoldRaw<TT>::type v[kFoldRound];   // (as loaded: widened when added, so that the loads stay in flight)
-        int pos[kFoldRound];   // window position of the block
-        int e0[kFoldRound];    // float of the run that falls on the block's first position (-255 .. run - 1)
-        int lim[kFoldRound];   // the entry's, -1: no entry
-      };
-      unsigned long long todo = 0ull;   // entries of the chunk that this wavefront still has to add
-      int next = 0;                     // first list entry behind the chunk
-      int c_pos = 0, c_e0 = 0, c_off = 0, c_lim = 0;
-      auto refill = [&]() {
-        while (todo == 0ull && next < total) {   // (uniform)
-          const int t = next + lane;
-          const bool have = t < total;
-          const int rel = have ? list_rel[t] : 0, at = have ? list_at[t] : 0;
-          c_lim = have ? list_lim[t] : 0;
-          const int first = rel >> 8;                    // (arithmetic shift: the block of the run's first float)
-          const int b = first + ((wave - first) & 15);   // the wavefront's only block among the sixteen from there on
-          c_pos = b * kFoldBlock;
-          c_e0 = c_pos - rel;
-          c_off = at + c_e0;
-          todo = __ballot(have && b >= 0 && c_pos < wlen && c_e0 < run);
-          next += 64;
-        }
-      };
-      auto issue = [&](Round& r) {
-  #pragma unroll
-        for (int u = 0; u < kFoldRound; u++) {
-          const bool any = todo != 0ull;
-          const int src = any ? (int)__builtin_ctzll(todo) : 0;
-          todo &= todo - 1ull;
-          const int off = __builtin_amdgcn_readlane(c_off, src), lim = __builtin_amdgcn_readlane(c_lim, src);
-          r.pos[u] = __builtin_amdgcn_readlane(c_pos, src);
-          r.e0[u] = __builtin_amdgcn_readlane(c_e0, src);
-          r.lim[u] = any ? lim : -1;
-          // (every slot loads, an empty one the buffer's first floats: with no branch around the
-          //  loads their number is fixed, and the wait for this round's values can leave the next
-          //  round's in flight)
-          const long long first = any ? (long long)off : 0ll;
-          unsigned mine = lane16;   // offset of the lane's four elements from the block's first, in bytes of floats
-          if (any && (r.e0[u] < 0 || r.e0[u] + kFoldBlock > run)) {   // (uniform) an end of the run:
-            // lanes that lie wholly outside the run fetch floats of the run that other lanes fetch
-            // anyway (their values count as zero below) instead of a neighbouring tile's
-            const int e = r.e0[u] + lane4;
-            const int inside = e <= -4 ? 0 : (e >= run ? max(run - 4, r.e0[u]) : e);
-            mine = (unsigned)(inside - r.e0[u]) * 4u;
-          }
-          // (read once and never again: a load that leaves the caches to the offsets and to the
-          //  contraction's stores still on their way to memory — K = N = 10240: 129 -> 111 us)
-          r.v[u] = __builtin_nontemporal_load(reinterpret_cast<const typename FoldRaw<TT>::unaligned*>(
-              reinterpret_cast<const char*>(p.tiles) + (first * 4 + mine) / (4 / (int)sizeof(TT))));
-        }
-      };
-      // (plain read-add-write: LDS float atomics are several times slower, and nobody else touches
-      //  this lane's words; runs that overlap are added one after the other, in list order)
-      auto add = [&](const Round& r) {
-  #pragma unroll
-        for (int u = 0; u < kFoldRound; u++) {
-          if (r.lim[u] == -1) continue;   // (uniform)
-          fold_f4 v = fold_widen<TT>(r.v[u]);
-          const int lim = r.lim[u];
-          if (r.e0[u] < 0 || r.e0[u] + kFoldBlock > run || (lim & 0x0fffffff) != full_lim) {
-            // an end of the run, or a tile that sticks out of K x N: what is not the run's counts as zero
-            asm volatile("" ::: "memory");   // (keeps this arithmetic out of the common path)
-            const int rows = (lim & 0x3fff) + 1, cols = ((lim >> 14) & 0x3fff) + 1, base = (lim >> 28) * run;
-  #pragma unroll
-            for (int f = 0; f < 4; f++) {
-              const int e = r.e0[u] + lane4 + f, in_tile = base + e;
-              const bool ok = e >= 0 && e < run && (in_tile >> p.h.bn_shift) < rows && (in_tile & (p.h.BN - 1)) < cols;
-              v[f] = ok ? v[f] : 0.f;
-            }
-          }
-          fold_f4* at = reinterpret_cast<fold_f4*>(img + r.pos[u] + lane4);
-          *at = *at + v;
-        }
-      };
-      Round r0, r1;
-      refill();
-      issue(r0);
-      while (true) {   // (uniform per wavefront; no barrier inside)
-        refill();
-        issue(r1);
-        add(r0);
-        if (r1.lim[0] == -1) break;   // (entries fill a round from its first slot)
-        refill();
-        issue(r0);
-        add(r1);
-        if (r0.lim[0] == -1) break;
-      }
+      walk(total);
     }
   }
   // --- the window of this share's image ---------------------------------------------------------

@@ -168,6 +168,18 @@ static inline int fold_tile_bytes(int elem_bytes, bool dhw_f32, const rz_tuning&
   return (elem_bytes == 2 && !dhw_f32 && t.fold_tiles != -1) ? 2 : 4;
 }
 
+// The windows of hashed_weight that the fold kernel's workgroups own (a function of H alone: a layer
+// plan lists every window's tiles).
+static inline void fold_geometry(int H, int* window, int* windows) {
+  const int kWindowMax = 32768, kThreads = 1024;
+  int n = (int)(((long long)H + kWindowMax - 1) / kWindowMax);
+  // from half a window per compute unit on, the windows are cut so that whole rounds of workgroups
+  // come out, and every workgroup writes its window of dHW itself (no shares, no images)
+  if (n * 2 >= kComputeUnits) n = (n + kComputeUnits - 1) / kComputeUnits * kComputeUnits;
+  *window = (int)(((((long long)H + n - 1) / n) + kThreads - 1) / kThreads * kThreads);
+  *windows = (int)(((long long)H + *window - 1) / *window);
+}
+
 static inline FoldPlan plan_fold(int K, int N, int H, int BK, int BN, int slices, bool windowed = false, int tile_bytes = 4) {
   FoldPlan f = {};
   f.tile_bytes = tile_bytes;
@@ -175,7 +187,6 @@ static inline FoldPlan plan_fold(int K, int N, int H, int BK, int BN, int slices
   const long long tiles = (long long)((K + BK - 1) / BK) * ((N + BN - 1) / BN);
   // (element indices of the buffer are 32-bit in the kernels; the fold lists slices entries per tile)
   if (E > 16384 || slices > 64 || (long long)slices * tiles * E >= (1LL << 31)) return f;
-  const int kWindowMax = 32768, kThreads = 1024;
   // (few tiles over a hashed_weight of up to 2^18 elements: measured 5 to 8 us; with a larger one every
   //  workgroup would still look at every tile for the handful that reach it, and the windowed kernel or
   //  the window kernel do better — K = 2048, N = 4096, H = 2^20: 20 us against the window kernel's 25 in all)
@@ -191,12 +202,7 @@ static inline FoldPlan plan_fold(int K, int N, int H, int BK, int BN, int slices
     f.use = 1;
     return f;
   }
-  f.windows = (H + kWindowMax - 1) / kWindowMax;
-  // from half a window per compute unit on, the windows are cut so that whole rounds of workgroups
-  // come out, and every workgroup writes its window of dHW itself (no shares, no images)
-  if (f.windows * 2 >= kComputeUnits) f.windows = (f.windows + kComputeUnits - 1) / kComputeUnits * kComputeUnits;
-  f.window = (((H + f.windows - 1) / f.windows) + kThreads - 1) / kThreads * kThreads;
-  f.windows = (H + f.window - 1) / f.window;
+  fold_geometry(H, &f.window, &f.windows);
   // (a workgroup fills a compute unit: no more workgroups than compute units, or two would wait for a second round)
   long long shares = f.windows * 2 >= kComputeUnits ? 1 : kComputeUnits / f.windows;
   if (shares > slices * tiles / 8) shares = slices * tiles / 8;   // a share is worth a workgroup from some tiles on
@@ -496,14 +502,18 @@ static inline WindowPlan plan_window(int M, int K, int N, int H, int BK, int BN,
 // K, N, H, the tile and the hash constants, not on M, the element type or the data), computed once
 // on the host and kept by the caller in device memory.  int32 words:
 //   [0, 16)   header: magic, version, K, N, H, BK, BN, hash_levels, tiles, windows, window,
-//             entries, strips per tile, checksum of the hash constants (layer_plan_hash_sum), 0, 0
+//             entries, strips per tile, checksum of the hash constants (layer_plan_hash_sum),
+//             fold windows, fold window
 //   offsets   [tiles]           where every W tile starts in hashed_weight (index tk * tiles_n + tn)
 //   start     [windows + 1]     first entry of every window of the window kernel (window_geometry)
 //   list      [capacity]        the units of work (tile * units per tile + unit: 32 rows by up to 64 columns of
 //                               a tile, see window_units) that meet the window, ascending
 //   offs      [capacity]        ... and where each starts in hashed_weight
-// The lists exist for the tiles the window kernel supports (windows = 0 otherwise).
-static constexpr int32_t kLayerPlanMagic = 0x525a4c50, kLayerPlanVersion = 1;
+//   fold_start [fold windows + 1]  first entry of every window of the fold kernel (fold_geometry)
+//   fold_list  [fold capacity]     the tiles that meet the window, in the order in which the fold kernel's
+//                                  own search numbers them (fold_rank_order)
+// The first two lists exist for the tiles the window kernel supports (windows = 0 otherwise).
+static constexpr int32_t kLayerPlanMagic = 0x525a4c50, kLayerPlanVersion = 2;
 static constexpr int kLayerPlanHeader = 16;
 // What a plan's header says of the hash constants that its offsets were computed with (the kernels
 // that read a plan compare it with their own call's constants).
@@ -522,7 +532,9 @@ struct LayerPlanLayout {
   bool ok;
   int tiles, windows, window, strips_per_tile, strip_elems;   // (units per tile, elements a unit spans)
   long long capacity;                 // list entries reserved (an upper bound of those used)
-  size_t offsets_at, start_at, list_at, offs_at, words;
+  int fold_window, fold_windows;
+  long long fold_capacity;
+  size_t offsets_at, start_at, list_at, offs_at, fold_start_at, fold_list_at, words;
 };
 static inline LayerPlanLayout layer_plan_layout(int K, int N, int H, int BK, int BN) {
   LayerPlanLayout l = {};
@@ -541,7 +553,12 @@ static inline LayerPlanLayout layer_plan_layout(int K, int N, int H, int BK, int
   }
   l.list_at = round16(l.start_at + (size_t)l.windows + 1);
   l.offs_at = round16(l.list_at + (size_t)l.capacity);
-  l.words = round16(l.offs_at + (size_t)l.capacity);
+  // a tile of BK * BN consecutive elements meets at most ceil(BK * BN / window) + 1 fold windows
+  fold_geometry(H, &l.fold_window, &l.fold_windows);
+  l.fold_capacity = tiles * (((long long)BK * BN + l.fold_window - 1) / l.fold_window + 1);
+  l.fold_start_at = round16(l.offs_at + (size_t)l.capacity);
+  l.fold_list_at = round16(l.fold_start_at + (size_t)l.fold_windows + 1);
+  l.words = round16(l.fold_list_at + (size_t)l.fold_capacity);
   l.ok = l.words < (1u << 30);
   return l;
 }

@@ -199,17 +199,51 @@ def _window_geometry(H):
     return w, -(-H // w)
 
 
+def _fold_geometry(H):
+    """Restated from the comments of fold_geometry: windows of at most 32768 elements; from 128 windows on,
+    whole rounds of 256; a window is a multiple of 1024 elements."""
+    n = -(-H // 32768)
+    if 2 * n >= 256:
+        n = -(-n // 256) * 256
+    w = -(-(-(-H // n)) // 1024) * 1024
+    return w, -(-H // w)
+
+
+def _check_fold_lists(plan, at, tiles, offsets, H, E):
+    """The fold kernel's lists behind word `at` of a plan: window b's list holds exactly the tiles whose
+    E elements meet [b*w, (b+1)*w), in the order in which the kernel's own search numbers tiles: pass by pass
+    of 65536 tile indices, and inside a pass thread t (of 1024) holds the tiles t, t + 1024, ... of the pass.
+    Returns the word behind the lists."""
+    w, windows = _fold_geometry(H)
+    assert (int(plan[14]), int(plan[15])) == (windows, w)
+    r16 = lambda v: (v + 15) & ~15
+    cap = tiles * (-(-E // w) + 1)
+    list_at = r16(at + windows + 1)
+    start = plan[at:at + windows + 1]
+    assert start[0] == 0 and np.all(np.diff(start) >= 0) and start[-1] <= cap
+    ids = np.arange(tiles)
+    order = np.lexsort(((ids % 65536) // 1024, ids % 1024, ids // 65536))   # (last key first)
+    total = 0
+    for b in range(windows):
+        meets = order[(offsets[order] < (b + 1) * w) & (offsets[order] + E > b * w)]
+        assert np.array_equal(plan[list_at + start[b]:list_at + start[b + 1]], meets), b
+        total += len(meets)
+    assert total == start[-1] and total >= tiles
+    return r16(list_at + cap)
+
+
 @pytest.mark.parametrize("cfg", [(1024, 1024, 65536, 64, 64), (300, 330, 70000, 32, 64), (4096, 8192, 40000, 64, 64),
                                  (640, 640, 2000001, 64, 64), (192, 128, 7000000, 64, 64), (96, 72, 100000, 32, 64),
                                  (512, 512, 30000, 128, 128), (256, 256, 1000, 16, 16), (300, 520, 90000, 64, 32),
-                                 (512, 300, 200000, 256, 128), (256, 512, 70000, 32, 256)])
+                                 (512, 300, 200000, 256, 128), (256, 512, 70000, 32, 256), (4800, 4800, 500000, 16, 16)])
 @pytest.mark.parametrize("levels", [2, 3])
 def test_layer_plan_lists_every_strip_in_every_window_it_meets(lib, oracle, cfg, levels):
     """rz_layer_plan_build against a brute-force restatement: the tile offsets are the oracle's, and
     the list of window b holds exactly the units of work of the window kernel — 32 rows by min(BN, 64)
     columns of a tile: unit s * parts + part starts at off + 32*BN*s + 64*part and spans 31*BN + min(BN, 64)
     elements — that meet [b*w, (b+1)*w), in ascending (tile, unit) order, with their offsets.  Tiles the
-    window kernel does not serve (16 or 256 columns, 16 rows) get a plan with the offsets alone."""
+    window kernel does not serve (16 or 256 columns, 16 rows) get a plan with the offsets and, like every
+    plan, the fold kernel's lists (_check_fold_lists)."""
     K, N, H, BK, BN = cfg
     R = R1024 if levels == 2 else oracle.legacy_constants(1024)
     nbytes = lib.rz_layer_plan_bytes(K, N, H, BK, BN)
@@ -223,19 +257,20 @@ def test_layer_plan_lists_every_strip_in_every_window_it_meets(lib, oracle, cfg,
     assert np.array_equal(plan[16:16 + tiles].astype(np.int64), want)
     served = BN in (32, 64, 128) and BK in (32, 64, 128, 256)
     windows, w = int(plan[9]), int(plan[10])
-    if not served:
-        assert windows == 0 and plan[11] == 0
-        return
-    assert (w, windows) == _window_geometry(H)
     r16 = lambda v: (v + 15) & ~15
     start_at = r16(16 + tiles)
+    if not served:
+        assert windows == 0 and plan[11] == 0
+        assert nbytes == 4 * _check_fold_lists(plan, r16(r16(start_at + 1)), tiles, want, H, BK * BN)
+        return
+    assert (w, windows) == _window_geometry(H)
     uc = min(BN, 64)
     parts = BN // uc
     strips, selems = (BK // 32) * parts, 31 * BN + uc
     cap = tiles * strips * (-(-selems // w) + 1)
     list_at = r16(start_at + windows + 1)
     offs_at = r16(list_at + cap)
-    assert nbytes == 4 * r16(offs_at + cap)
+    assert nbytes == 4 * _check_fold_lists(plan, r16(offs_at + cap), tiles, want, H, BK * BN)
     start = plan[start_at:start_at + windows + 1]
     assert start[0] == 0 and start[-1] == plan[11] and np.all(np.diff(start) >= 0) and start[-1] <= cap
     u = np.arange(strips)

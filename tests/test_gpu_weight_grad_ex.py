@@ -266,6 +266,41 @@ def test_fold_shares_take_a_partition_of_a_window_even_when_their_lists_overflow
     assert torch.equal(a, b)
 
 
+PLANNED_FOLDS = [
+    # (M, K, N, H, BK, BN, dtype)
+    (64, 4096, 4096, 300000, 16, 16, torch.bfloat16),      # 65536 tiles; ten windows, 25 workgroups to a window
+    (48, 4800, 4800, 500000, 16, 16, torch.float32),       # 90000 tiles: more than one listing pass of the search
+    (1000, 700, 1100, 2000000, 128, 128, torch.float32),   # runs of a tile in several list entries; tiles beyond K x N
+    (2100, 1000, 900, 600000, 64, 64, torch.bfloat16),     # M in slices: several list entries per tile; 16-bit tiles
+    (128, 2048, 2048, 9000000, 32, 64, torch.float16),     # whole rounds of 256 windows, no shares
+]
+
+
+@pytest.mark.parametrize("shape", PLANNED_FOLDS, ids=lambda s: "x".join(str(v) for v in s[:6]))
+def test_fold_lists_of_a_layer_plan_give_the_bits_of_the_search(oracle, tuned, shape):
+    """With a layer plan the fold kernel's workgroups read their windows' tiles from the plan's lists; without
+    one they look for them among all tile offsets.  The lists hold the tiles in the order in which the search
+    numbers them, so the additions happen in the same order: the same bits, also where a window is shared by
+    several workgroups, where a workgroup's part overflows its list, and where a tile has several entries."""
+    from rzlinear_amd import _lib
+    from rzlinear_amd.impl.RzLinearBackward import weight_grad_hashed
+    M, K, N, H, BK, BN, dtype = shape
+    tuned(fold=1, window=-1)
+    code = _lib.dtype_code(torch.empty(0, dtype=dtype))
+    plan = _lib.plan_query(2, M, K, N, H, BK, BN, code, planned=True)
+    _say("fold lists", shape, plan)
+    assert plan["mode"] == "fold"
+    (x, _, dy), (x64, _, dy64) = make_inputs(M, K, N, H, dtype, seed=72)
+    R = _lib.hash_constants(*rargs(R1024))
+    outs = []
+    for planned in (False, True, True):
+        outs.append(weight_grad_hashed(x, dy, 0.5, M, K, N, H, R, BK, BN, use_layer_plan=planned)[0])
+    torch.cuda.synchronize()
+    assert torch.equal(outs[0], outs[1]) and torch.equal(outs[1], outs[2])
+    ref = oracle.weight_grad(x64, dy64, H, BK, BN, R1024, 0.5)
+    assert rel_err(outs[1].float().cpu().numpy(), ref) <= TOL[dtype]
+
+
 SMALL_LAYERS = [
     # (M, K, N, H, BK, BN): a hashed_weight beyond an LDS image, at most 4096 tiles
     (1024, 1024, 1024, 65536, 64, 64),     # the reference's CPU-runnable configuration
