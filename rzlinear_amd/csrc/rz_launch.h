@@ -385,16 +385,19 @@ static inline WeightGradPlan plan_weight_grad(int M, int K, int N, int H, int BK
       // measured), against reading the tiles back (their stores overlap the contraction, unless
       // it is shorter than they are), writing and reading the images, and two more launches
       const double elems = (double)pl.splits * (double)K * (double)N;
-      const double product_us = 2.0 * (double)M * K * N / (elem_bytes == 4 ? 110e6 : 900e6);
+      // (fp32, K = N = 10240: the contraction takes 427 us at M = 256, 805 us at M = 512)
+      const double product_us = 2.0 * (double)M * K * N / (elem_bytes == 4 ? 145e6 : 900e6);
       const double store_us = elems * tile_bytes / 4.0e6;
       // (K*N atomics take about 5.2 ps each; a long contraction hides up to 2.4 ps of that — K = 2048,
       //  N = 8192, bf16: M = 128 87 us in all against 57 us folded, M = 1024 108 against 79 us)
       const double hidden = 0.45 * product_us < elems * 2.4e-6 ? 0.45 * product_us : elems * 2.4e-6;
       const double atomics_us = elems * 5.2e-6 - hidden;
-      // (a workgroup of the fold kernel reads some 15 GB/s: few workgroups cannot use the memory system)
+      // (a workgroup of the fold kernel reads some 20 GB/s: few workgroups cannot use the memory system; all of
+      //  them together 6 TB/s of fp32 tiles — K = N = 10240: 85 us — and 4.7 TB/s of 16-bit ones — 58 us —
+      //  where the instructions per load set the pace)
       const double read_bytes = elems * tile_bytes * (1.0 + (double)BK * BN / f.window);
-      const double all_us = (read_bytes + 2.0 * (double)f.partial_bytes) / 4.5e6;
-      const double one_us = read_bytes / ((double)f.windows * f.shares) / 15e3;
+      const double all_us = (read_bytes + 2.0 * (double)f.partial_bytes) / (tile_bytes == 4 ? 6.0e6 : 4.7e6);
+      const double one_us = read_bytes / ((double)f.windows * f.shares) / (tile_bytes == 4 ? 24e3 : 19e3);
       // (few tiles: every element is read once, by a kernel of a few microseconds; it is taken even where
       //  the atomics would be a little faster — K = N = 1024: 5 us against 3 us on top of the contraction —
       //  because it adds in a fixed order: the same bits on every call)
@@ -406,7 +409,10 @@ static inline WeightGradPlan plan_weight_grad(int M, int K, int N, int H, int BK
         //  kernel also pays its fill, drain and store — about 5 us for a round of 256 tiles, 10 us
         //  in fp32, in proportion to the tile's area — which matters when M is small)
         const double round_us = (elem_bytes == 4 ? 10.0 : 5.0) * (double)pl.tile * pl.tile / 65536.0;
-        pl.fold_us = product_us + fold_us + round_us * (double)((pl.workgroups + kComputeUnits - 1) / kComputeUnits);
+        // (a contraction shorter than the stores of its tiles takes the time of the stores — fp32, K = N = 10240,
+        //  H = 2^20, M = 32: 220 us in all)
+        const double contraction_us = product_us + round_us * (double)((pl.workgroups + kComputeUnits - 1) / kComputeUnits);
+        pl.fold_us = (contraction_us > store_us ? contraction_us : store_us) + fold_us - (store_us > product_us ? store_us - product_us : 0.0);
       }
     }
   }
@@ -489,12 +495,13 @@ static inline WindowPlan plan_window(int M, int K, int N, int H, int BK, int BN,
   // fixed order, one after the other: with many tiles per element that chain is what takes the
   // time, about 1.7 us a link (K = 2048, N = 8192, H = 200000: 84 links, 158 us at M = 32 — folded
   // 57 us; K = N = 10240, H = 200000: 524 links, 1048 us).
-  const double chain_us = 1.7 * (double)K * (double)N / (double)H + 10.0;
+  // (fp32, K = N = 10240, H = 2^20, M = 32: 100 links, 260 us — folded 220 us)
+  const double chain_us = (elem_bytes == 4 ? 2.4 : 1.7) * (double)K * (double)N / (double)H + 10.0;
   if (t_window < chain_us) t_window = chain_us;
   // ... against what the contraction kernel's plan would take: the fold, or the atomic scatter
   const double t_scatter = 0.9 * (double)K * N / 184e3 + 2.0 * M * (double)K * N / 800e6;
   const double t_other = other.fold.use ? other.fold_us : t_scatter;
-  pl.use = t.window == 1 || t_window * 1.1 < t_other;
+  pl.use = t.window == 1 || t_window < t_other;
   return pl;
 }
 
