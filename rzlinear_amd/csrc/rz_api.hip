@@ -627,7 +627,7 @@ extern "C" {
 
 #define RZ_API __attribute__((visibility("default")))
 
-RZ_API int rz_version(void) { return 400; }
+RZ_API int rz_version(void) { return 500; }
 
 RZ_API const char* rz_status_string(int status) {
   switch (status) {
