@@ -91,7 +91,11 @@ typedef struct rz_tuning {
                      -1 = always fp32 tiles */
   int finish;     /* forward / input-grad with a cut contraction: 0 = automatic (the slice that arrives last at a
                      tile of the output adds the slices' partial results up and stores it: no second kernel),
-                     -1 = always a second kernel; the results are the same bits either way */
+                     -1 = always a second kernel; the results are the same bits either way.  The arrivals are
+                     counted in a device array that the library owns and divides among streams: each of the
+                     first sixteen streams per device that launch such a contraction keeps a part of its own,
+                     so calls on different streams never share a counter; a further stream, a stream under
+                     capture and an output of more than 4096 tiles get the second kernel */
   int poll_limit; /* weight-grad by windows: 0 = default; > 0 = how often a wavefront looks at the flags of the
                      earlier strips it waits for before it gives up and the window is stored as NaN (a bounded
                      wait; tests set a tiny value to see every wavefront leave the kernel all the same) */

@@ -247,20 +247,32 @@ static hipError_t reduce_slices_dtype(int dtype, const float* part, void* C, con
 }
 
 // ---- counters of the cut contractions that finish in one kernel ---------------------------------
-// One 32-bit counter per tile of the output and launch (GemmParams::finish), in a file-scope device
-// array: zero when the library is loaded, and set back to zero by the workgroup that finishes a tile.
-// Launches take consecutive ranges of the array in turn, so two launches share counters only if
-// kFinishCounters tiles' worth of launches are in flight at once.  In host code the array's name is a
-// handle for hipGetSymbolAddress, looked up once per device with that device current.
-static constexpr unsigned kFinishCounters = 1u << 16;
+// One 32-bit counter per tile of the output (GemmParams::finish), in a file-scope device array: zero
+// when the library is loaded, and set back to zero by the workgroup that finishes a tile.  The array
+// is divided among streams: the first sixteen streams per device that launch such a contraction each
+// get a part of their own, for good; launches on one stream run one after the other and leave their
+// counters at zero, so every launch of a stream starts at the first counter of the stream's part, and
+// launches on different streams, which may run at the same time, never share a counter.  A stream
+// beyond the sixteenth, a stream under capture (its kernels will run again later, on whatever stream the
+// graph is launched on) and an output of more tiles than a part has counters get the second kernel
+// instead.  In host code the array's name is a handle for hipGetSymbolAddress, looked up once per
+// device with that device current.
+static constexpr unsigned kFinishStreams = 16, kFinishPerStream = 4096;
+static constexpr unsigned kFinishCounters = kFinishStreams * kFinishPerStream;
 static constexpr int kFinishMaxDevices = 64;
 static __device__ __align__(256) unsigned finish_counters[kFinishCounters];
 static std::atomic<unsigned*> finish_counters_ptr[kFinishMaxDevices];
-static std::atomic<unsigned> finish_turn{0};
+static std::atomic<uintptr_t> finish_owner[kFinishMaxDevices][kFinishStreams];   // stream handle + 1 (0: nobody's yet)
 
-// Counters for a launch with `tiles` output tiles, or null (the caller then launches the second kernel).
-static unsigned* finish_counters_for(long long tiles) {
-  if (tiles < 1 || tiles > (long long)(kFinishCounters / 4)) return nullptr;
+// Counters for a launch with `tiles` output tiles on stream s, or null (the caller then launches the second kernel).
+static unsigned* finish_counters_for(long long tiles, hipStream_t s) {
+  if (tiles < 1 || tiles > (long long)kFinishPerStream) return nullptr;
+  hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(s, &capture) != hipSuccess) {
+    (void)hipGetLastError();
+    return nullptr;
+  }
+  if (capture != hipStreamCaptureStatusNone) return nullptr;
   int dev = -1;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kFinishMaxDevices) return nullptr;
   unsigned* base = finish_counters_ptr[dev].load(std::memory_order_acquire);
@@ -273,14 +285,13 @@ static unsigned* finish_counters_for(long long tiles) {
     base = static_cast<unsigned*>(q);
     finish_counters_ptr[dev].store(base, std::memory_order_release);   // (a racing thread stores the same value)
   }
-  // the next `tiles` counters, from the start of the array if they would run off its end
-  unsigned seen = finish_turn.load(std::memory_order_relaxed);
-  for (;;) {
-    const unsigned at = seen % kFinishCounters;
-    const unsigned start = at + (unsigned)tiles <= kFinishCounters ? at : 0u;
-    const unsigned next = seen - at + start + (unsigned)tiles + (start == 0u && at != 0u ? kFinishCounters : 0u);
-    if (finish_turn.compare_exchange_weak(seen, next, std::memory_order_relaxed)) return base + start;
+  const uintptr_t key = reinterpret_cast<uintptr_t>(s) + 1;   // (the null stream has a part like any other)
+  for (unsigned i = 0; i < kFinishStreams; i++) {
+    uintptr_t owner = finish_owner[dev][i].load(std::memory_order_acquire);
+    if (owner == 0 && finish_owner[dev][i].compare_exchange_strong(owner, key, std::memory_order_acq_rel)) owner = key;
+    if (owner == key) return base + i * kFinishPerStream;
   }
+  return nullptr;
 }
 
 // Forward (op kForward) or input-grad through one code path: p holds the operands; with a
@@ -298,7 +309,7 @@ static int run_plain_op(int op, int dtype, GemmParams p, const void* bias, void*
       p.partial = (float*)workspace;
       // the slice that arrives last at a tile finishes it (adds the slices in slice order, then the
       // bias: the bits of the second kernel's sum) — unless told otherwise, or out of counters
-      p.finish = (tuning.finish != -1 && sp.splits <= finish_slices(sp.tile, p.I, p.J)) ? finish_counters_for(tile_count(p.I, p.J, sp.tile)) : nullptr;
+      p.finish = (tuning.finish != -1 && sp.splits <= finish_slices(sp.tile, p.I, p.J)) ? finish_counters_for(tile_count(p.I, p.J, sp.tile), s) : nullptr;
       p.bias = p.finish != nullptr ? bias : nullptr;
       if (launch_gemm(dtype, op, p, nullptr, &sp, tuning, s) != hipSuccess) return RZ_ERR_LAUNCH;
       if (p.finish != nullptr) return RZ_OK;
@@ -1005,7 +1016,7 @@ RZ_API int rz_plan_query(int op, int M, int K, int N, int H, int BK, int BN, int
   const KernelForm f = kernel_form(op, I, J, R, chunk, sp.tile, tile_count(I, J, sp.tile) * sp.splits, eb, t);
   out[0] = sp.tile; out[1] = sp.splits; out[2] = chunk; out[3] = f.step; out[4] = cut ? 1 : 0;
   out[5] = (int32_t)(tile_count(I, J, sp.tile) * sp.splits);
-  out[6] = (cut && t.finish != -1 && sp.splits <= finish_slices(sp.tile, I, J)) ? 1 : 0;
+  out[6] = (cut && t.finish != -1 && sp.splits <= finish_slices(sp.tile, I, J) && tile_count(I, J, sp.tile) <= (long long)kFinishPerStream) ? 1 : 0;
   return RZ_OK;
 }
 

@@ -189,6 +189,41 @@ FINISH_CASES = [
 ]
 
 
+def test_cut_contractions_on_many_streams_at_once(oracle):
+    """The counters of the slices that finish their own tiles live in the library, divided among streams:
+    launches on different streams may run at the same time and must not share a counter.  Twenty streams
+    (more than the library keeps parts for: the rest take the second kernel) each run cut forward
+    contractions of two shapes, again and again, with nothing between them; every output must have the bits
+    of the two-kernel form computed alone on the default stream."""
+    from rzlinear_amd import _lib
+    from rzlinear_amd.impl.RzLinearForward import rz_linear_forward_bias_tl
+    dtype = torch.bfloat16
+    code = _lib.dtype_code(torch.empty(0, dtype=dtype))
+    cases = [(128, 10240, 10240, 6553600, 32, 64), (64, 4096, 4096, 50000, 64, 64)]   # three and four slices
+    _say("cut contractions on many streams")
+    work = []
+    for c, (M, K, N, H, BK, BN) in enumerate(cases):
+        q = _lib.plan_query(0, M, K, N, H, BK, BN, code)
+        assert q["mode"] == "split" and q["shares"] == 1, q     # cut, and finished by the kernel itself
+        (x, hw, _), _ = make_inputs(M, K, N, H, dtype, seed=50 + c)
+        bias = torch.randn((N,), generator=torch.Generator().manual_seed(c)).to(dtype).cuda()
+        kw = dict(BLOCK_SIZE_K=BK, BLOCK_SIZE_N=BN)
+        with _lib.tuning(finish=-1):
+            want = rz_linear_forward_bias_tl(x, hw, bias, 0.5, M, K, N, H, *rargs(R1024), **kw)
+        work.append((x, hw, bias, (M, K, N, H), kw, want))
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream() for _ in range(20)]
+    outs = []
+    for rep in range(6):
+        for i, st in enumerate(streams):
+            x, hw, bias, dims, kw, want = work[(i + rep) % 2]
+            with torch.cuda.stream(st):
+                outs.append((rz_linear_forward_bias_tl(x, hw, bias, 0.5, *dims, *rargs(R1024), **kw), want, i, rep))
+    torch.cuda.synchronize()
+    for y, want, i, rep in outs:
+        assert torch.equal(y, want), (i, rep)
+
+
 @pytest.mark.parametrize("dtype", DTYPES, ids=lambda d: str(d).split(".")[-1])
 @pytest.mark.parametrize("case", FINISH_CASES, ids=lambda s: "x".join(map(str, s)))
 def test_the_last_slice_to_arrive_finishes_the_tile(oracle, case, dtype):
