@@ -528,12 +528,14 @@ static int weight_grad_impl(const void* X, const void* dY, void* dHW, void* dbia
     fp.plan_header = nullptr;
     fp.plan_start = nullptr;
     fp.plan_list = nullptr;
+    fp.plan_capacity = 0;
     if (planned) {
       fp.offsets = layer_plan + lay.offsets_at;
       fp.plan_header = layer_plan;
       if (!f.small && lay.fold_windows == f.windows && lay.fold_window == f.window) {
         fp.plan_start = layer_plan + lay.fold_start_at;
         fp.plan_list = layer_plan + lay.fold_list_at;
+        fp.plan_capacity = (int)lay.fold_capacity;
       }
     } else if (f.small) {
       fp.offsets = nullptr;   // (the kernel hashes the few offsets it needs)

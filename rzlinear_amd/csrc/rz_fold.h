@@ -45,6 +45,7 @@ struct FoldParams {
   const int32_t* plan_header;   // `offsets` belongs to a layer plan (else null): its header, checked against this call's
   const int32_t* plan_start;    // the plan's list of every window's tiles (else null: the kernel looks for them): [windows + 1] ...
   const int32_t* plan_list;     // ... and the tile indices, in the order in which the kernel's own search numbers them
+  int plan_capacity;            // ... of which the plan has room for this many
   float* partial;       // [shares][pitch]: every workgroup writes its window of its share's image ...
   void* out;            // ... or, with a single share (partial == null), its window of dHW itself:
   int out_dtype;        //     an rz_dtype code,
@@ -306,12 +307,15 @@ __global__ __launch_bounds__(kFoldThreads) void fold_tiles_kernel(const FoldPara
 
   if (p.plan_list != nullptr) {
     // The layer plan lists the window's tiles, numbered as below: nothing to look for.
-    const int begin = p.plan_start[win], all = plan_ok ? p.plan_start[win + 1] - begin : 0;
+    // (what a plan says is kept inside the plan and inside the table of offsets whatever it holds: a
+    //  spoilt plan gives a wrong dHW, never an access out of bounds)
+    const int begin = min(max(p.plan_start[win], 0), p.plan_capacity);
+    const int all = plan_ok ? min(max(p.plan_start[win + 1], begin), p.plan_capacity) - begin : 0;
     const int want_lo = (int)((long long)share * all / p.shares), want_hi = (int)((long long)(share + 1) * all / p.shares);
     for (int chunk_lo = want_lo; chunk_lo < want_hi; chunk_lo += cap) {   // (uniform)
       const int chunk_hi = (chunk_lo + cap) < want_hi ? (chunk_lo + cap) : want_hi;
       if (chunk_lo != want_lo) __syncthreads();   // (the wavefronts are done reading the previous chunk's list)
-      for (int q = chunk_lo + tid; q < chunk_hi; q += kFoldThreads) put(q - chunk_lo, p.plan_list[begin + q]);
+      for (int q = chunk_lo + tid; q < chunk_hi; q += kFoldThreads) put(q - chunk_lo, min(max(p.plan_list[begin + q], 0), ntiles - 1));
       __syncthreads();
       walk((chunk_hi - chunk_lo) * per_tile);
     }

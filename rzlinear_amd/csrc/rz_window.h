@@ -223,8 +223,11 @@ struct WindowKernel {
         return;
       }
     }
-    const int plan_lo = planned ? p.plan_start[blockIdx.x] : 0;
-    const int plan_n = planned ? p.plan_start[blockIdx.x + 1] - plan_lo : 0;
+    // (what a plan says is kept inside the plan, the tiles and hashed_weight whatever it holds: a spoilt plan
+    //  gives a wrong dHW, never an access out of bounds)
+    const int plan_entries = planned ? p.plan_header[11] : 0;
+    const int plan_lo = planned ? min(max(p.plan_start[blockIdx.x], 0), plan_entries) : 0;
+    const int plan_n = planned ? min(max(p.plan_start[blockIdx.x + 1], plan_lo), plan_entries) - plan_lo : 0;
     const int list_total = planned ? plan_n : total;   // what the rounds below work through: entries, or tile ids
     int lo = 0;
     while (lo < list_total) {
@@ -234,8 +237,8 @@ struct WindowKernel {
         found = plan_n - lo < kList ? plan_n - lo : kList;
         __syncthreads();   // (the previous round's list is no longer read)
         for (int i = tid; i < found; i += kThreads) {
-          sm.list[i] = p.plan_list[plan_lo + lo + i];
-          sm.offs[i] = p.plan_offs[plan_lo + lo + i];
+          sm.list[i] = min(max(p.plan_list[plan_lo + lo + i], 0), (total << ushift) - 1);
+          sm.offs[i] = min(max(p.plan_offs[plan_lo + lo + i], 0), p.H - 1);
           sm.done[i] = 0;
         }
         hi = lo + found;
