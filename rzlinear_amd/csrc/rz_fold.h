@@ -295,13 +295,19 @@ __global__ __launch_bounds__(kFoldThreads) void fold_tiles_kernel(const FoldPara
     issue(r0);
     while (true) {   // (uniform per wavefront; no barrier inside)
       refill();
+      if (todo == 0ull) {   // (nothing left to load: no round of empty slots, whose loads would still be waited for)
+        add(r0);
+        break;
+      }
       issue(r1);
       add(r0);
-      if (r1.lim[0] == -1) break;   // (entries fill a round from its first slot)
       refill();
+      if (todo == 0ull) {
+        add(r1);
+        break;
+      }
       issue(r0);
       add(r1);
-      if (r0.lim[0] == -1) break;
     }
   };
 
