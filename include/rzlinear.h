@@ -196,8 +196,11 @@ size_t rz_weight_grad_workspace_bytes(int M, int K, int N, int H, int BK, int BN
  * the reference rounds the running sum at every atomic add).  The LDS-image, fold and
  * window paths add in a fixed order (plain read-add-write in LDS, ordered by barriers, by list
  * order or by flags; partial images are added in index order): the same inputs give the same
- * bits on every call.  Only the global-atomic path (few W tiles and a hashed_weight too large
- * for LDS) leaves the summation order across tiles open, as the reference does.
+ * bits on every call.  Two cases leave the summation order across tiles open, as the reference
+ * does everywhere: the global-atomic path (hashed tiles of more than 16384 elements over a
+ * hashed_weight too large for LDS, or where rz_tuning asks for it), and hashed tiles of 16 rows or
+ * 16 columns on the LDS-image path (an MFMA block then spans several hashed tiles whose slices may
+ * overlap, and they are added into the image with LDS atomics).
  */
 int rz_weight_grad(const void* X, const void* dY, void* dHW, void* workspace,
                    size_t workspace_bytes, int M, int K, int N, int H, int BK, int BN,
