@@ -96,16 +96,16 @@ TRAFFIC = {
     },
     ("ffn", "bf16"): {
         "profile": "profiles/rz_gemm_fold_bf16_ffn.txt",
-        "bytes": {"forward": int((70697.6 * 2.0 + 262144.0) * 1024),      # algorithmic: 320.1 MiB
-                  "input_grad": int((132314.1 * 2.0 + 65536.0) * 1024),
+        "bytes": {"forward": int((70690.9 * 2.0 + 262144.0) * 1024),      # algorithmic: 320.1 MiB
+                  "input_grad": int((132331.1 * 2.0 + 65536.0) * 1024),
                   # contraction (X, dY re-read by the XCDs' tile groups; X^T.dY written tile by tile in bf16: 128 MiB)
                   "weight_grad": int((786599.9 * 2.0 + 131072.0) * 1024)},
     },
     ("grid_1024_10240", "bf16"): {
         "profile": "profiles/rz_gemm_fold_bf16_grid_1024_10240.txt",
-        "bytes": {"forward": int((396155.6 * 2.0 + 143380.0) * 1024),     # (three slices: fp32 partial planes written, read back by the slice that finishes)
-                  "input_grad": int((382373.9 * 2.0 + 143380.0) * 1024),
-                  "weight_grad": int((172199.1 * 2.0 + 204800.0) * 1024)},      # (X^T.dY tile by tile in bf16: 200 MiB)
+        "bytes": {"forward": int((396677.9 * 2.0 + 143380.0) * 1024),     # (three slices: fp32 partial planes written, read back by the slice that finishes)
+                  "input_grad": int((382509.1 * 2.0 + 143380.1) * 1024),
+                  "weight_grad": int((172198.8 * 2.0 + 204800.0) * 1024)},      # (X^T.dY tile by tile in bf16: 200 MiB)
     },
 }
 
